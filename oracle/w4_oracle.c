@@ -1,0 +1,671 @@
+/*
+ * CPU oracle for the fused-dequant hot path -- TEST INFRASTRUCTURE ONLY.
+ * Nothing that ships links or loads this file; it is the checker for the HIP
+ * kernels and for the C++ host headers.
+ *
+ * Each function restates, in plain C with software binary16 conversion, the
+ * arithmetic of the reference host header it cites.  How each one is pinned
+ * (tests/test_oracle_*.py):
+ *   f16<->f32, E4M3 encode ... exhaustive / dense sweeps against numpy's
+ *                              float16 and a brute-force nearest-value search
+ *   generators ............... mt19937_64's standard 10000th-value check and a
+ *                              stream comparison with libstdc++ built by g++
+ *   quantize / dequant_all ... reference hand pins (all-zero groups, throw
+ *                              list), per-element bounds, and the recorded
+ *                              rel-L2 tables of ERROR_ANALYSIS.md and
+ *                              data/w4a16_*_bench.json
+ *   quantize_mx .............. all-3.0 -> byte 126 / code 7, sign, zero,
+ *                              no-saturation invariant, recorded rel L2
+ *   gemm_oracle .............. [1,2]x[[3,4],[5,6]] = [11,17]; numpy FP64 GEMM
+ *   attention ................ zero keys -> mean of V; |score|~3e4 stability;
+ *                              numpy FP64 softmax
+ *   FP8 cache ................ all-1.0 -> 0x7E pin, recorded rel L2
+ *   paged scatter ............ block-table-resolved rows equal contiguous rows
+ */
+#include "w4_oracle.h"
+
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+static __thread char g_err[256];
+static int g_threads = 1;
+
+const char* orc_last_error(void) { return g_err; }
+
+void orc_set_threads(int n) { g_threads = n < 1 ? 1 : n; }
+
+static int fail(const char* msg) {
+  snprintf(g_err, sizeof g_err, "%s", msg);
+  return ORC_EINVAL;
+}
+
+/* ------------------------------------------------------------------------ */
+/* binary16 <-> binary32, software                                           */
+
+float orc_f16_to_f32(uint16_t h) {
+  const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  const uint32_t ex = (h >> 10) & 0x1Fu;
+  const uint32_t man = h & 0x3FFu;
+  uint32_t bits;
+  if (ex == 0) {
+    if (man == 0) {
+      bits = sign;
+    } else { /* subnormal: man * 2^-24, exact in float */
+      float v = (float)man * 5.9604644775390625e-08f;
+      memcpy(&bits, &v, 4);
+      bits |= sign;
+    }
+  } else if (ex == 31) {
+    bits = sign | 0x7F800000u | (man << 13);
+  } else {
+    bits = sign | ((ex + 112u) << 23) | (man << 13);
+  }
+  float out;
+  memcpy(&out, &bits, 4);
+  return out;
+}
+
+uint16_t orc_f32_to_f16(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  const uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+  const uint32_t ax = x & 0x7FFFFFFFu;
+  if (ax >= 0x7F800000u) { /* inf or NaN */
+    if (ax == 0x7F800000u) return (uint16_t)(sign | 0x7C00u);
+    return (uint16_t)(sign | 0x7E00u | ((ax >> 13) & 0x3FFu));
+  }
+  if (ax >= 0x477FF000u) /* >= 65520: rounds to infinity */
+    return (uint16_t)(sign | 0x7C00u);
+  if (ax < 0x33000000u) /* < 2^-25: rounds to zero (2^-25 itself ties to 0) */
+    return sign;
+  const int e = (int)(ax >> 23) - 127;
+  uint32_t man = (ax & 0x7FFFFFu) | 0x800000u; /* 24-bit significand */
+  int shift;                                   /* bits dropped */
+  uint32_t base;
+  if (e >= -14) {
+    shift = 13;
+    base = (uint32_t)(e + 15) << 10;
+    man &= 0x7FFFFFu; /* hidden bit lives in the exponent field */
+  } else {
+    shift = 13 + (-14 - e); /* subnormal target */
+    base = 0;
+  }
+  uint32_t kept = man >> shift;
+  const uint32_t rem = man & ((1u << shift) - 1u);
+  const uint32_t half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (kept & 1u))) ++kept;
+  return (uint16_t)(sign | (base + kept)); /* a carry walks into the exponent */
+}
+
+/* pack.hpp:58-60: RNE_half(float(s) * (float)(q - z)). */
+uint16_t orc_dequant_one(uint16_t s, int q, int z) {
+  return orc_f32_to_f16(orc_f16_to_f32(s) * (float)(q - z));
+}
+
+/* mx.hpp:56-63: E2M1 magnitude (index>>1 is the exponent field, index&1 the
+ * mantissa bit) times 2^(se-127), one RNE rounding to half. */
+uint16_t orc_dequant_one_mx(uint8_t se, int q) {
+  const int i = q & 7;
+  const float mag = (i >> 1) == 0 ? ldexpf((float)(i & 1), -1)
+                                  : ldexpf((float)(2 + (i & 1)), (i >> 1) - 2);
+  const float s = ldexpf(1.0f, (int)se - 127);
+  const float v = (q & 8) ? -mag : mag;
+  return orc_f32_to_f16(s * v);
+}
+
+/* kvfp8.hpp:42-47: e==0 -> m*2^-9, else (8+m)*2^(e-10); NaN codes read 480. */
+float orc_decode_f8_e4m3(uint8_t b) {
+  const int e = (b >> 3) & 0xF, m = b & 7;
+  const float mag =
+      (e == 0) ? ldexpf((float)m, -9) : ldexpf((float)(8 + m), e - 10);
+  return (b & 0x80) ? -mag : mag;
+}
+
+uint16_t orc_dequant_one_f8(uint16_t s, uint8_t b) {
+  return orc_f32_to_f16(orc_f16_to_f32(s) * orc_decode_f8_e4m3(b));
+}
+
+/* The conversion kvfp8.hpp:117-119 asks of the CUDA/HIP fp8 header: float ->
+ * OCP E4M3, round to nearest even, finite saturation at +-448 (0x7E); NaN maps
+ * to 0x7F.  Written over the float bit pattern: E4M3 has bias 7, 3 mantissa
+ * bits, subnormal step 2^-9. */
+uint8_t orc_f32_to_e4m3_satfinite(float x) {
+  uint32_t u;
+  memcpy(&u, &x, 4);
+  const uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+  const uint32_t au = u & 0x7FFFFFFFu;
+  if (au > 0x7F800000u) return (uint8_t)(sign | 0x7Fu);
+  float ax;
+  memcpy(&ax, &au, 4);
+  if (ax >= 448.0f) return (uint8_t)(sign | 0x7Eu);
+  if (ax == 0.0f) return sign;
+  int e;
+  (void)frexpf(ax, &e); /* ax = f * 2^e, f in [0.5,1) -> exponent e-1 */
+  int ex = e - 1;
+  if (ex < -6) ex = -6; /* subnormal range shares the 2^-9 step */
+  /* units of 2^(ex-3) */
+  const float scaled = ldexpf(ax, 3 - ex); /* exact: power-of-two scaling */
+  float r = nearbyintf(scaled);            /* RNE in the default mode */
+  int mant = (int)r;                       /* 0..16 */
+  int efield;
+  if (ex == -6 && mant < 8) {
+    efield = 0; /* subnormal: value = mant * 2^-9 */
+  } else {
+    if (mant == 16) {
+      mant = 8;
+      ++ex;
+    }
+    efield = ex + 7;
+    mant -= 8;
+  }
+  if (efield > 15 || (efield == 15 && mant > 6)) return (uint8_t)(sign | 0x7Eu);
+  return (uint8_t)(sign | (efield << 3) | mant);
+}
+
+/* ------------------------------------------------------------------------ */
+/* Seeded generators: std::mt19937_64 and libstdc++'s normal_distribution
+ * (Marsaglia polar, second variate cached), as used by pack.hpp:186-200.     */
+
+typedef struct {
+  uint64_t mt[312];
+  int idx;
+} mt64;
+
+static void mt64_seed(mt64* g, uint64_t seed) {
+  g->mt[0] = seed;
+  for (int i = 1; i < 312; ++i)
+    g->mt[i] = 6364136223846793005ULL * (g->mt[i - 1] ^ (g->mt[i - 1] >> 62)) +
+               (uint64_t)i;
+  g->idx = 312;
+}
+
+static uint64_t mt64_next(mt64* g) {
+  if (g->idx >= 312) {
+    for (int i = 0; i < 312; ++i) {
+      const uint64_t y = (g->mt[i] & 0xFFFFFFFF80000000ULL) |
+                         (g->mt[(i + 1) % 312] & 0x7FFFFFFFULL);
+      g->mt[i] = g->mt[(i + 156) % 312] ^ (y >> 1) ^
+                 ((y & 1ULL) ? 0xB5026F5AA96619E9ULL : 0ULL);
+    }
+    g->idx = 0;
+  }
+  uint64_t y = g->mt[g->idx++];
+  y ^= (y >> 29) & 0x5555555555555555ULL;
+  y ^= (y << 17) & 0x71D67FFFEDA60000ULL;
+  y ^= (y << 37) & 0xFFF7EEE000000000ULL;
+  y ^= (y >> 43);
+  return y;
+}
+
+/* generate_canonical<double,53> over a 64-bit engine: one draw / 2^64. */
+static double mt64_canonical(mt64* g) {
+  double r = (double)mt64_next(g) / 18446744073709551616.0;
+  if (r >= 1.0) r = nextafter(1.0, 0.0);
+  return r;
+}
+
+typedef struct {
+  mt64 g;
+  int have;
+  double saved;
+} normal_gen;
+
+static double normal_next(normal_gen* n) {
+  if (n->have) {
+    n->have = 0;
+    return n->saved;
+  }
+  double x, y, r2;
+  do {
+    x = 2.0 * mt64_canonical(&n->g) - 1.0;
+    y = 2.0 * mt64_canonical(&n->g) - 1.0;
+    r2 = x * x + y * y;
+  } while (r2 > 1.0 || r2 == 0.0);
+  const double mult = sqrt(-2.0 * log(r2) / r2);
+  n->saved = x * mult;
+  n->have = 1;
+  return y * mult;
+}
+
+void orc_mt19937_64_stream(uint64_t seed, uint64_t* out, size_t n) {
+  mt64 g;
+  mt64_seed(&g, seed);
+  for (size_t i = 0; i < n; ++i) out[i] = mt64_next(&g);
+}
+
+void orc_normal_weights(double* out, size_t n, uint64_t seed) {
+  normal_gen ng;
+  mt64_seed(&ng.g, seed);
+  ng.have = 0;
+  for (size_t i = 0; i < n; ++i) out[i] = normal_next(&ng) * 1.0 + 0.0;
+}
+
+void orc_normal_activations(uint16_t* out, size_t n, uint64_t seed) {
+  normal_gen ng;
+  mt64_seed(&ng.g, seed);
+  ng.have = 0;
+  for (size_t i = 0; i < n; ++i)
+    out[i] = orc_f32_to_f16((float)(normal_next(&ng) * 1.0 + 0.0));
+}
+
+/* The other libstdc++ distributions the reference's error study draws from
+ * (benchmarks/error_analysis.cpp:44-61,134-137); used only to reproduce its
+ * recorded tables.  uniform_int over a 64-bit engine is the multiply-shift
+ * reduction (no rejection occurs for the power-of-two ranges used there). */
+static uint64_t mt64_uniform_int(mt64* g, uint64_t range) {
+  unsigned __int128 prod = (unsigned __int128)mt64_next(g) * range;
+  uint64_t low = (uint64_t)prod;
+  if (low < range) {
+    const uint64_t threshold = (0 - range) % range;
+    while (low < threshold) {
+      prod = (unsigned __int128)mt64_next(g) * range;
+      low = (uint64_t)prod;
+    }
+  }
+  return (uint64_t)(prod >> 64);
+}
+
+void orc_laplace_weights(double* out, size_t n, uint64_t seed) {
+  mt64 g;
+  mt64_seed(&g, seed);
+  for (size_t i = 0; i < n; ++i) {
+    const int pos = (int)mt64_uniform_int(&g, 2);
+    const double e = -log(1.0 - mt64_canonical(&g)) / 1.0;
+    out[i] = pos ? e : -e;
+  }
+}
+
+void orc_uniform_weights(double* out, size_t n, uint64_t seed) {
+  mt64 g;
+  mt64_seed(&g, seed);
+  for (size_t i = 0; i < n; ++i) out[i] = mt64_canonical(&g) * 2.0 + -1.0;
+}
+
+void orc_uniform_int_stream(uint64_t seed, uint64_t range, uint64_t* out,
+                            size_t n) {
+  mt64 g;
+  mt64_seed(&g, seed);
+  for (size_t i = 0; i < n; ++i) out[i] = mt64_uniform_int(&g, range);
+}
+
+/* ------------------------------------------------------------------------ */
+/* W4: pack.hpp                                                              */
+
+int orc_words(int n) { return (n + 7) / 8; }
+
+static int all_finite(const double* w, size_t n) {
+  for (size_t i = 0; i < n; ++i)
+    if (!isfinite(w[i])) return 0;
+  return 1;
+}
+
+/* pack.hpp:64-130.  q/scales/zeros are caller-allocated: N*words(K),
+ * N*G, N*words(G) (zeros untouched when symmetric). */
+int orc_quantize(const double* w, size_t w_len, int N, int K, int gs,
+                 int symmetric, uint32_t* q, uint16_t* scales,
+                 uint32_t* zeros) {
+  if (N < 1 || K < 1) return fail("quantize: bad dims");
+  if (gs < 8 || gs % 8 != 0)
+    return fail("quantize: gs must be a multiple of 8");
+  if (w_len != (size_t)N * (size_t)K) return fail("quantize: size");
+  if (!all_finite(w, w_len)) return fail("quantize: non-finite input");
+  const int G = (K + gs - 1) / gs;
+  const int wk = orc_words(K), wg = orc_words(G);
+  memset(q, 0, (size_t)N * wk * sizeof(uint32_t));
+  if (!symmetric) memset(zeros, 0, (size_t)N * wg * sizeof(uint32_t));
+  for (int n = 0; n < N; ++n) {
+    const double* row = w + (size_t)n * K;
+    for (int g = 0; g < G; ++g) {
+      const int k0 = g * gs, k1 = (k0 + gs < K) ? k0 + gs : K;
+      double lo = row[k0], hi = row[k0];
+      for (int k = k0 + 1; k < k1; ++k) {
+        if (row[k] < lo) lo = row[k];
+        if (row[k] > hi) hi = row[k];
+      }
+      double s;
+      int nonzero;
+      if (symmetric) {
+        const double amax = fabs(lo) > fabs(hi) ? fabs(lo) : fabs(hi);
+        s = amax > 0.0 ? amax / 7.0 : 1.0;
+        nonzero = (lo != 0.0 || hi != 0.0);
+      } else {
+        if (lo > 0.0) lo = 0.0; /* the range must bracket zero */
+        if (hi < 0.0) hi = 0.0;
+        s = hi > lo ? (hi - lo) / 15.0 : 1.0;
+        nonzero = (hi != lo);
+      }
+      const uint16_t sh = orc_f32_to_f16((float)s);
+      const float sf = orc_f16_to_f32(sh);
+      if (!isfinite(sf) || (sf == 0.0f && nonzero))
+        return fail("quantize: group scale outside FP16 range");
+      int z = 8;
+      if (!symmetric) {
+        z = (int)lround(-lo / (double)sf);
+        z = z < 0 ? 0 : (z > 15 ? 15 : z);
+      }
+      scales[(size_t)n * G + g] = sh;
+      for (int k = k0; k < k1; ++k) {
+        int c = (int)lround(row[k] / (double)sf) + z;
+        c = c < 0 ? 0 : (c > 15 ? 15 : c);
+        q[(size_t)n * wk + k / 8] |= (uint32_t)c << (4 * (k % 8));
+      }
+      if (!symmetric)
+        zeros[(size_t)n * wg + g / 8] |= (uint32_t)z << (4 * (g % 8));
+    }
+  }
+  return ORC_OK;
+}
+
+/* pack.hpp:134-161 (validate_packed + dequant_all).  Lengths stand in for the
+ * vector sizes the reference checks. */
+int orc_dequant_all(int N, int K, int gs, int G, int symmetric,
+                    const uint32_t* q, size_t q_len, const uint16_t* scales,
+                    size_t s_len, const uint32_t* zeros, size_t z_len,
+                    uint16_t* w) {
+  if (N < 1 || K < 1) return fail("packed: bad dims");
+  if (gs < 8 || gs % 8 != 0) return fail("packed: gs must be a multiple of 8");
+  if (G != (K + gs - 1) / gs) return fail("packed: G inconsistent with K, gs");
+  const int wk = orc_words(K), wg = orc_words(G);
+  if (q_len != (size_t)N * wk) return fail("packed: q size");
+  if (s_len != (size_t)N * G) return fail("packed: scales size");
+  if (!symmetric && z_len != (size_t)N * wg) return fail("packed: zeros size");
+  if (symmetric && z_len != 0)
+    return fail("packed: symmetric carries no zeros");
+  for (int n = 0; n < N; ++n)
+    for (int k = 0; k < K; ++k) {
+      const int g = k / gs;
+      const int c = (int)((q[(size_t)n * wk + k / 8] >> (4 * (k % 8))) & 0xF);
+      const int z =
+          symmetric
+              ? 8
+              : (int)((zeros[(size_t)n * wg + g / 8] >> (4 * (g % 8))) & 0xF);
+      w[(size_t)n * K + k] = orc_dequant_one(scales[(size_t)n * G + g], c, z);
+    }
+  return ORC_OK;
+}
+
+/* pack.hpp:166-184: C[m,n] = sum_k x[m,k]*w[n,k], double accumulation in k
+ * order over the FP16 inputs. */
+int orc_gemm_oracle(const uint16_t* x, size_t x_len, int M, int K,
+                    const uint16_t* w, size_t w_len, int N, double* c) {
+  if (M < 1 || N < 1 || K < 1) return fail("gemm_oracle: bad dims");
+  if (x_len != (size_t)M * (size_t)K || w_len != (size_t)N * (size_t)K)
+    return fail("gemm_oracle: size");
+  /* Widen x once; every (m,n) dot reuses it. */
+  double* xd = (double*)malloc((size_t)M * K * sizeof(double));
+  if (!xd) return fail("gemm_oracle: out of memory");
+  for (size_t i = 0; i < (size_t)M * K; ++i)
+    xd[i] = (double)orc_f16_to_f32(x[i]);
+#pragma omp parallel num_threads(g_threads)
+  {
+    double* wd = (double*)malloc((size_t)K * sizeof(double));
+#pragma omp for schedule(static)
+    for (int n = 0; n < N; ++n) {
+      for (int k = 0; k < K; ++k)
+        wd[k] = (double)orc_f16_to_f32(w[(size_t)n * K + k]);
+      for (int m = 0; m < M; ++m) {
+        const double* xr = xd + (size_t)m * K;
+        double acc = 0.0;
+        for (int k = 0; k < K; ++k) acc += xr[k] * wd[k];
+        c[(size_t)m * N + n] = acc;
+      }
+    }
+    free(wd);
+  }
+  free(xd);
+  return ORC_OK;
+}
+
+/* ------------------------------------------------------------------------ */
+/* MXFP4: mx.hpp                                                             */
+
+static const double kE2M1[8] = {0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0};
+
+int orc_blocks(int K) { return (K + 31) / 32; }
+
+/* mx.hpp:71-119. */
+int orc_quantize_mx(const double* w, size_t w_len, int N, int K, uint32_t* q,
+                    uint8_t* scales) {
+  if (N < 1 || K < 1) return fail("quantize_mx: bad dims");
+  if (w_len != (size_t)N * (size_t)K) return fail("quantize_mx: size");
+  if (!all_finite(w, w_len)) return fail("quantize_mx: non-finite input");
+  const int B = orc_blocks(K), wk = orc_words(K);
+  memset(q, 0, (size_t)N * wk * sizeof(uint32_t));
+  for (int n = 0; n < N; ++n) {
+    const double* row = w + (size_t)n * K;
+    for (int b = 0; b < B; ++b) {
+      const int k0 = b * 32, k1 = (k0 + 32 < K) ? k0 + 32 : K;
+      double amax = 0.0;
+      for (int k = k0; k < k1; ++k)
+        if (fabs(row[k]) > amax) amax = fabs(row[k]);
+      int e = 0;
+      if (amax > 0.0) {
+        e = (int)ceil(log2(amax / 6.0));
+        while (amax > 6.0 * ldexp(1.0, e)) ++e; /* no-saturation insurance */
+        if (e > 127) return fail("quantize_mx: block scale outside E8M0 range");
+        if (e < -127) e = -127;
+      }
+      const double s = ldexp(1.0, e);
+      scales[(size_t)n * B + b] = (uint8_t)(e + 127);
+      for (int k = k0; k < k1; ++k) {
+        const double v = row[k] / s;
+        const double av = fabs(v);
+        int idx = 0; /* nearest magnitude, ties keep the lower index */
+        for (int i = 1; i < 8; ++i)
+          if (fabs(kE2M1[i] - av) < fabs(kE2M1[idx] - av)) idx = i;
+        const uint32_t code = (uint32_t)((signbit(v) ? 8 : 0) | idx);
+        q[(size_t)n * wk + k / 8] |= code << (4 * (k % 8));
+      }
+    }
+  }
+  return ORC_OK;
+}
+
+/* mx.hpp:121-140. */
+int orc_dequant_all_mx(int N, int K, int B, const uint32_t* q, size_t q_len,
+                       const uint8_t* scales, size_t s_len, uint16_t* w) {
+  if (N < 1 || K < 1) return fail("packed mx: bad dims");
+  if (B != orc_blocks(K)) return fail("packed mx: B inconsistent with K");
+  const int wk = orc_words(K);
+  if (q_len != (size_t)N * wk) return fail("packed mx: q size");
+  if (s_len != (size_t)N * B) return fail("packed mx: scales size");
+  for (int n = 0; n < N; ++n)
+    for (int k = 0; k < K; ++k) {
+      const int c = (int)((q[(size_t)n * wk + k / 8] >> (4 * (k % 8))) & 0xF);
+      w[(size_t)n * K + k] =
+          orc_dequant_one_mx(scales[(size_t)n * B + k / 32], c);
+    }
+  return ORC_OK;
+}
+
+/* ------------------------------------------------------------------------ */
+/* W4 KV cache: kvcache.hpp                                                  */
+
+/* kvcache.hpp:60-108: H independent slabs, each quantized as a PackedW with
+ * N = S rows and K = D. */
+int orc_quantize_cache(const double* k, size_t k_len, const double* v,
+                       size_t v_len, int H, int S, int D, int gs,
+                       int symmetric, uint32_t* q_k, uint16_t* s_k,
+                       uint32_t* z_k, uint32_t* q_v, uint16_t* s_v,
+                       uint32_t* z_v) {
+  if (H < 1 || S < 1 || D < 1) return fail("quantize_cache: bad dims");
+  if (gs < 8 || gs % 8 != 0)
+    return fail("quantize_cache: gs must be a multiple of 8");
+  const size_t per = (size_t)S * D;
+  if (k_len != (size_t)H * per || v_len != (size_t)H * per)
+    return fail("quantize_cache: size");
+  const int G = (D + gs - 1) / gs;
+  const size_t nq = (size_t)S * orc_words(D), ns = (size_t)S * G,
+               nz = (size_t)S * orc_words(G);
+  for (int h = 0; h < H; ++h) {
+    int rc = orc_quantize(k + h * per, per, S, D, gs, symmetric, q_k + h * nq,
+                          s_k + h * ns, symmetric ? NULL : z_k + h * nz);
+    if (rc) return rc;
+    rc = orc_quantize(v + h * per, per, S, D, gs, symmetric, q_v + h * nq,
+                      s_v + h * ns, symmetric ? NULL : z_v + h * nz);
+    if (rc) return rc;
+  }
+  return ORC_OK;
+}
+
+/* kvcache.hpp:141-175 after dequant_head: FP64 scores from the FP16-exact
+ * inputs, max-subtracted softmax, FP64 weighted sum over V. */
+int orc_attention_f16(const uint16_t* q, const uint16_t* k16,
+                      const uint16_t* v16, int H, int heads_per_slab, int S,
+                      int D, double* out) {
+  if (H < 1 || S < 1 || D < 1 || heads_per_slab < 1)
+    return fail("attention_reference: bad dims");
+  const double inv_sqrt_d = 1.0 / sqrt((double)D);
+  const int HQ = H * heads_per_slab;
+#pragma omp parallel num_threads(g_threads)
+  {
+    double* scores = (double*)malloc((size_t)S * sizeof(double));
+    double* qd = (double*)malloc((size_t)D * sizeof(double));
+#pragma omp for schedule(dynamic, 1)
+    for (int hq = 0; hq < HQ; ++hq) {
+      const int slab = hq / heads_per_slab;
+      const uint16_t* kh = k16 + (size_t)slab * S * D;
+      const uint16_t* vh = v16 + (size_t)slab * S * D;
+      for (int d = 0; d < D; ++d)
+        qd[d] = (double)orc_f16_to_f32(q[(size_t)hq * D + d]);
+      double smax = -INFINITY;
+      for (int t = 0; t < S; ++t) {
+        double acc = 0.0;
+        for (int d = 0; d < D; ++d)
+          acc += qd[d] * (double)orc_f16_to_f32(kh[(size_t)t * D + d]);
+        scores[t] = acc * inv_sqrt_d;
+        if (scores[t] > smax) smax = scores[t];
+      }
+      double denom = 0.0;
+      for (int t = 0; t < S; ++t) {
+        scores[t] = exp(scores[t] - smax);
+        denom += scores[t];
+      }
+      for (int t = 0; t < S; ++t) scores[t] /= denom;
+      double* o = out + (size_t)hq * D;
+      for (int d = 0; d < D; ++d) o[d] = 0.0;
+      /* position-major walk: each o[d] still adds its terms in t order */
+      for (int t = 0; t < S; ++t) {
+        const double p = scores[t];
+        const uint16_t* vr = vh + (size_t)t * D;
+        for (int d = 0; d < D; ++d) o[d] += p * (double)orc_f16_to_f32(vr[d]);
+      }
+    }
+    free(scores);
+    free(qd);
+  }
+  return ORC_OK;
+}
+
+/* ------------------------------------------------------------------------ */
+/* FP8 KV cache: kvfp8.hpp                                                   */
+
+/* kvfp8.hpp:70-128: scale = amax/448 per (position, group), stored FP16;
+ * elements are float(x / float(scale)) converted RNE to E4M3. */
+int orc_quantize_cache_f8(const double* k, size_t k_len, const double* v,
+                          size_t v_len, int H, int S, int D, int gs,
+                          uint8_t* q_k, uint16_t* s_k, uint8_t* q_v,
+                          uint16_t* s_v) {
+  if (H < 1 || S < 1 || D < 1) return fail("quantize_cache_f8: bad dims");
+  if (gs < 8 || gs % 8 != 0)
+    return fail("quantize_cache_f8: gs must be a multiple of 8");
+  const size_t total = (size_t)H * S * D;
+  if (k_len != total || v_len != total) return fail("quantize_cache_f8: size");
+  if (!all_finite(k, total) || !all_finite(v, total))
+    return fail("quantize_cache_f8: non-finite input");
+  const int G = (D + gs - 1) / gs;
+  for (int side = 0; side < 2; ++side) {
+    const double* src = side ? v : k;
+    uint8_t* qc = side ? q_v : q_k;
+    uint16_t* sc = side ? s_v : s_k;
+    for (size_t row = 0; row < (size_t)H * S; ++row) {
+      const double* r = src + row * D;
+      for (int g = 0; g < G; ++g) {
+        const int d0 = g * gs, d1 = (d0 + gs < D) ? d0 + gs : D;
+        double amax = 0.0;
+        for (int d = d0; d < d1; ++d)
+          if (fabs(r[d]) > amax) amax = fabs(r[d]);
+        const double s = amax > 0.0 ? amax / 448.0 : 1.0;
+        const uint16_t sh = orc_f32_to_f16((float)s);
+        const float sf = orc_f16_to_f32(sh);
+        if (!isfinite(sf) || (sf == 0.0f && amax > 0.0))
+          return fail("quantize_cache_f8: group scale outside FP16 range");
+        sc[row * G + g] = sh;
+        for (int d = d0; d < d1; ++d)
+          qc[row * D + d] =
+              orc_f32_to_e4m3_satfinite((float)(r[d] / (double)sf));
+      }
+    }
+  }
+  return ORC_OK;
+}
+
+/* kvfp8.hpp:131-146 over `rows` positions (one head's slab, or all of them). */
+int orc_dequant_f8(const uint8_t* q, const uint16_t* s, int rows, int D,
+                   int gs, uint16_t* w) {
+  if (rows < 1 || D < 1) return fail("cache f8: bad dims");
+  if (gs < 8 || gs % 8 != 0)
+    return fail("cache f8: gs must be a multiple of 8");
+  const int G = (D + gs - 1) / gs;
+  for (size_t t = 0; t < (size_t)rows; ++t)
+    for (int d = 0; d < D; ++d)
+      w[t * D + d] = orc_dequant_one_f8(s[t * G + d / gs], q[t * D + d]);
+  return ORC_OK;
+}
+
+/* ------------------------------------------------------------------------ */
+/* Paged pool: kvpaged.hpp:72-134.  Logical page i of every head lands at
+ * physical page bt[i]; rows past S in the last page stay zero. */
+int orc_paged_scatter(const void* src, void* dst, int H, int S, int page,
+                      const int* bt, int bt_len, size_t row_elems,
+                      size_t elem_size) {
+  if (H < 1 || S < 1) return fail("paged_from: bad dims");
+  if (page < 1) return fail("paged_from: bad page size");
+  const int lpages = (S + page - 1) / page;
+  if (bt_len != lpages) return fail("paged_from: block table size");
+  char* seen = (char*)calloc((size_t)bt_len, 1);
+  for (int i = 0; i < bt_len; ++i) {
+    if (bt[i] < 0 || bt[i] >= bt_len || seen[bt[i]]++) {
+      free(seen);
+      return fail("paged_from: bad block table");
+    }
+  }
+  free(seen);
+  const size_t rb = row_elems * elem_size;
+  const size_t pool_rows = (size_t)bt_len * page;
+  memset(dst, 0, (size_t)H * pool_rows * rb);
+  for (int h = 0; h < H; ++h)
+    for (int t = 0; t < S; ++t) {
+      const size_t row = (size_t)bt[t / page] * page + (size_t)(t % page);
+      memcpy((char*)dst + ((size_t)h * pool_rows + row) * rb,
+             (const char*)src + ((size_t)h * S + t) * rb, rb);
+    }
+  return ORC_OK;
+}
+
+/* ------------------------------------------------------------------------ */
+
+double orc_rel_l2_f16_vs_f64(const double* a, const uint16_t* b, size_t n) {
+  double num = 0.0, den = 0.0;
+  for (size_t i = 0; i < n; ++i) {
+    const double d = (double)orc_f16_to_f32(b[i]) - a[i];
+    num += d * d;
+    den += a[i] * a[i];
+  }
+  return sqrt(num / (den > 0.0 ? den : 1.0));
+}
+
+double orc_max_abs_f16_vs_f64(const double* a, const uint16_t* b, size_t n) {
+  double m = 0.0;
+  for (size_t i = 0; i < n; ++i) {
+    const double d = fabs((double)orc_f16_to_f32(b[i]) - a[i]);
+    if (d > m) m = d;
+  }
+  return m;
+}

@@ -1,0 +1,152 @@
+/*
+ * C ABI of libw4amd.so: the gfx950 launcher behind the w4::gpu C++ API.
+ *
+ * Every entry point validates its arguments before it touches the device (a
+ * bad call never dereferences a pointer, allocates or launches), then enqueues
+ * its kernels on `stream` and returns without synchronising.  All data
+ * pointers are device pointers owned by the caller.  Halves cross the boundary
+ * as IEEE binary16 bit patterns (w4_half has the storage of __half).
+ *
+ * Return value: W4_OK, W4_EINVAL (the reference throws std::invalid_argument
+ * here) or W4_ERUNTIME (the reference throws std::runtime_error from
+ * cuda_check).  w4_last_error() returns the thread's last message.
+ *
+ * The citations name the reference function each entry point replaces
+ * (paths relative to the reference repository).
+ */
+#ifndef W4_ABI_H
+#define W4_ABI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint16_t w4_half;
+typedef void* w4_stream; /* hipStream_t; NULL is the default stream */
+
+enum { W4_OK = 0, W4_EINVAL = 1, W4_ERUNTIME = 2 };
+
+/* Packed W4 weights, device view.  include/w4/dequant.cuh:31-37 */
+typedef struct w4_packed_view {
+  int N, K, gs, G;
+  int symmetric;
+  const uint32_t* q;     /* N * words(K), 8 nibbles per word, low first   */
+  const w4_half* scales; /* N * G                                          */
+  const uint32_t* zeros; /* N * words(G) nibbles; NULL when symmetric      */
+} w4_packed_view;
+
+/* Packed MXFP4 weights, device view.  include/w4/mxfused.cuh:26-30 */
+typedef struct w4_packed_mx_view {
+  int N, K, B;           /* B = ceil(K / 32)                               */
+  const uint32_t* q;     /* N * words(K) E2M1 codes                        */
+  const uint8_t* scales; /* N * B E8M0 bytes                               */
+} w4_packed_mx_view;
+
+/* W4 KV cache, device view: H slabs of S rows.  include/w4/kvattention.cuh:39-48 */
+typedef struct w4_kv_view {
+  int H, S, D, gs, G;
+  int symmetric;
+  const uint32_t* q_k;
+  const w4_half* s_k;
+  const uint32_t* z_k;
+  const uint32_t* q_v;
+  const w4_half* s_v;
+  const uint32_t* z_v;
+} w4_kv_view;
+
+/* FP8-E4M3 KV cache, device view.  include/w4/kvflash.cuh:390-396 */
+typedef struct w4_kv_f8_view {
+  int H, S, D, gs, G;
+  const uint8_t* q_k;
+  const w4_half* s_k;
+  const uint8_t* q_v;
+  const w4_half* s_v;
+} w4_kv_f8_view;
+
+const char* w4_last_error(void);
+
+/* M at or above this goes to the matrix-core kernel in w4_gemm / w4_gemm_mx.
+ * include/w4/dispatch.cuh:25 (re-measured for gfx950). */
+int w4_dispatch_mma_min_m(void);
+
+/* ---- packed-weight GEMM: c[M,N] = x[M,K] * W[N,K]^T, FP16 in/out ---------- */
+/* w: N*K halves, bit-identical to the host dequant_all.  dequant.cuh:62-82 */
+int w4_dequant(const w4_packed_view* p, w4_half* w, w4_stream stream);
+/* fused.cuh:172-214; w_out (optional) receives every dequantized weight */
+int w4_gemm_fused(const w4_packed_view* p, const w4_half* x, w4_half* c, int M,
+                  w4_stream stream, w4_half* w_out);
+/* mma.cuh:234-260 */
+int w4_gemm_mma(const w4_packed_view* p, const w4_half* x, w4_half* c, int M,
+                w4_stream stream, w4_half* w_out);
+/* dispatch.cuh:27-34 */
+int w4_gemm(const w4_packed_view* p, const w4_half* x, w4_half* c, int M,
+            w4_stream stream, w4_half* w_out);
+
+/* mxfused.cuh:57-69, 166-198, 291-307; dispatch.cuh:36-43 */
+int w4_dequant_mx(const w4_packed_mx_view* p, w4_half* w, w4_stream stream);
+int w4_gemm_fused_mx(const w4_packed_mx_view* p, const w4_half* x, w4_half* c,
+                     int M, w4_stream stream, w4_half* w_out);
+int w4_gemm_mma_mx(const w4_packed_mx_view* p, const w4_half* x, w4_half* c,
+                   int M, w4_stream stream, w4_half* w_out);
+int w4_gemm_mx(const w4_packed_mx_view* p, const w4_half* x, w4_half* c, int M,
+               w4_stream stream, w4_half* w_out);
+
+/* Plain FP16 GEMM (FP32 accumulate) over already-dequantized W: the two-pass
+ * baseline.  dequant.cuh:87-100 (cublasGemmEx there, hipBLASLt here). */
+int w4_gemm_fp16(const w4_half* w, const w4_half* x, w4_half* c, int M, int N,
+                 int K, w4_stream stream);
+
+/* ---- split-S flash-decode attention: one query token per head ------------- */
+/* kvflash.cuh:350-363.  q, out: H*D halves; k_out/v_out (optional): H*S*D */
+int w4_attention_w4_flash(const w4_kv_view* p, const w4_half* q, w4_half* out,
+                          w4_stream stream, w4_half* k_out, w4_half* v_out);
+/* kvflash.cuh:365-384 */
+int w4_attention_fp16_flash(const w4_half* q, const w4_half* k16,
+                            const w4_half* v16, w4_half* out, int H, int S,
+                            int D, w4_stream stream);
+/* kvflash.cuh:572-590 */
+int w4_attention_f8_flash(const w4_kv_f8_view* p, const w4_half* q,
+                          w4_half* out, w4_stream stream, w4_half* k_out,
+                          w4_half* v_out);
+/* kvflash.cuh:725-764.  p->S is the logical length; each head's pool slab has
+ * npages*page rows; logical row t lives at bt[t/page]*page + t%page. */
+int w4_attention_w4_flash_paged(const w4_kv_view* p, const int* bt, int page,
+                                int npages, const w4_half* q, w4_half* out,
+                                w4_stream stream, w4_half* k_out,
+                                w4_half* v_out);
+/* kvflash.cuh:435-457: rows of E4M3 bytes -> halves, scale per (row, group) */
+int w4_dequant_f8(const uint8_t* q, const w4_half* s, w4_half* w, int S, int D,
+                  int gs, w4_stream stream);
+
+/* ---- batched / grouped-query forms (no counterpart in the reference, which
+ * has one query head per cache slab and one block table per call).  The cache
+ * views hold B*Hkv slabs; `group` = Hq/Hkv query heads share each slab, so q
+ * and out are (H*group)*D halves ordered slab-major.  group = 1 reduces to the
+ * entry points above. ------------------------------------------------------- */
+int w4_attention_w4_flash_gqa(const w4_kv_view* p, int group, const w4_half* q,
+                              w4_half* out, w4_stream stream, w4_half* k_out,
+                              w4_half* v_out);
+int w4_attention_fp16_flash_gqa(const w4_half* q, const w4_half* k16,
+                                const w4_half* v16, w4_half* out, int H,
+                                int group, int S, int D, w4_stream stream);
+/* scale_mode 0: s_k/s_v hold one FP16 scale per (row, group) as in the
+ * reference; 1: one FP16 scale per slab (s_k/s_v have p->H entries). */
+int w4_attention_f8_flash_gqa(const w4_kv_f8_view* p, int group, int scale_mode,
+                              const w4_half* q, w4_half* out, w4_stream stream,
+                              w4_half* k_out, w4_half* v_out);
+/* One pool shared by all sequences: the view's H = Hkv slabs of npages*page
+ * rows; bt holds nseq tables of bt_stride entries; sequence s reads slab
+ * (s, h) -> pool slab h through table s.  q/out: nseq*Hkv*group*D halves. */
+int w4_attention_w4_flash_paged_batched(const w4_kv_view* p, const int* bt,
+                                        int nseq, int bt_stride, int page,
+                                        int npages, int group,
+                                        const w4_half* q, w4_half* out,
+                                        w4_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

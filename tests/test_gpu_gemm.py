@@ -1,0 +1,146 @@
+"""GPU parity gates for the packed-weight GEMM path, through the C ABI.
+
+Mirrors the reference device suite (tests/test_gpu.cu:54-498): for every config
+and sign mode the materialising dequant and the w_out hooks of both fused
+kernels must equal the oracle's dequant_all bit for bit, the GEMM outputs must
+be within rel L2 1e-3 of the FP64 oracle, the two kernels within 2e-3 of each
+other, and the dispatcher must reproduce its callee's bytes.
+"""
+import numpy as np
+import pytest
+import torch
+
+import orc
+import w4amd
+from devutil import DevPacked, DevPackedMx, bits, f64, halves, ptr, to_dev
+
+pytestmark = pytest.mark.gpu
+
+CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
+        (2, 32, 128, 64), (3, 40, 256, 128), (5, 72, 40, 8), (17, 64, 128, 16),
+        (33, 48, 104, 24), (20, 32, 100, 8), (65, 96, 100, 16),
+        # shapes that take the aligned dwordx4 paths
+        (1, 512, 4096, 128), (7, 96, 2048, 32), (9, 80, 1024, 64), (64, 64, 512, 128)]
+TOL, CROSS = 1e-3, 2e-3  # rel L2 vs the FP64 oracle; between two gated paths
+
+
+def _run(fn, view, x_d, M, N, K, hook=True):
+    c_d = halves(M * N, 0x7E00)
+    w_d = halves(N * K, 0x7E00) if hook else None
+    fn(view, ptr(x_d), ptr(c_d), M, 0, ptr(w_d))
+    return bits(c_d), (bits(w_d) if hook else None)
+
+
+@pytest.mark.parametrize("sym", [True, False], ids=["sym", "asym"])
+@pytest.mark.parametrize("i", range(len(CFGS)))
+def test_w4_gemm_gates(i, sym):
+    c = w4amd.capi()
+    M, N, K, gs = CFGS[i]
+    seed = 0x44A1 ^ (i * 977 + (0 if sym else 1))
+    p = orc.quantize(orc.normal_weights(N * K, seed), N, K, gs, sym)
+    w_ref = orc.dequant_all(p)
+    x = orc.normal_activations(M * K, seed + 1)
+    ref = orc.gemm_oracle(x, M, K, w_ref, N)
+    dp, x_d = DevPacked(p), to_dev(x)
+
+    w_d = halves(N * K, 0x7E00)
+    c.dequant(dp.view, ptr(w_d))
+    assert np.array_equal(bits(w_d), w_ref), "dequant bitwise"
+
+    cf, wf = _run(c.gemm_fused, dp.view, x_d, M, N, K)
+    assert np.array_equal(wf, w_ref), "fused w_out bitwise"
+    assert orc.rel_l2(cf.view(np.float16), ref) <= TOL
+    cm, wm = _run(c.gemm_mma, dp.view, x_d, M, N, K)
+    assert np.array_equal(wm, w_ref), "mma w_out bitwise"
+    assert orc.rel_l2(cm.view(np.float16), ref) <= TOL
+    den = np.sqrt(np.sum(ref ** 2))
+    cross = np.sqrt(np.sum((cf.view(np.float16).astype(np.float64) -
+                            cm.view(np.float16).astype(np.float64)) ** 2)) / den
+    assert cross <= CROSS
+    # without the hook the outputs are the same bytes
+    cf2, _ = _run(c.gemm_fused, dp.view, x_d, M, N, K, hook=False)
+    cm2, _ = _run(c.gemm_mma, dp.view, x_d, M, N, K, hook=False)
+    assert np.array_equal(cf, cf2) and np.array_equal(cm, cm2)
+    # dispatcher: same bytes as the callee it selects, hook intact
+    cd, wd = _run(c.gemm, dp.view, x_d, M, N, K)
+    want = cf if M < c.load().w4_dispatch_mma_min_m() else cm
+    assert np.array_equal(cd, want) and np.array_equal(wd, w_ref)
+    # two-pass baseline: dequant + plain FP16 GEMM
+    c2 = halves(M * N, 0x7E00)
+    c.gemm_fp16(ptr(w_d), ptr(x_d), ptr(c2), M, N, K)
+    assert orc.rel_l2(f64(c2), ref) <= TOL
+
+
+@pytest.mark.parametrize("i", range(len(CFGS)))
+def test_mx_gemm_gates(i):
+    c = w4amd.capi()
+    M, N, K, _ = CFGS[i]
+    seed = 0x1E4A ^ (i * 977)
+    p = orc.quantize_mx(orc.normal_weights(N * K, seed), N, K)
+    w_ref = orc.dequant_all_mx(p)
+    x = orc.normal_activations(M * K, seed + 1)
+    ref = orc.gemm_oracle(x, M, K, w_ref, N)
+    dp, x_d = DevPackedMx(p), to_dev(x)
+
+    w_d = halves(N * K, 0x7E00)
+    c.dequant_mx(dp.view, ptr(w_d))
+    assert np.array_equal(bits(w_d), w_ref), "mx dequant bitwise"
+    cf, wf = _run(c.gemm_fused_mx, dp.view, x_d, M, N, K)
+    assert np.array_equal(wf, w_ref), "mx fused w_out bitwise"
+    assert orc.rel_l2(cf.view(np.float16), ref) <= TOL
+    cm, wm = _run(c.gemm_mma_mx, dp.view, x_d, M, N, K)
+    assert np.array_equal(wm, w_ref), "mx mma w_out bitwise"
+    assert orc.rel_l2(cm.view(np.float16), ref) <= TOL
+    cd, wd = _run(c.gemm_mx, dp.view, x_d, M, N, K)
+    want = cf if M < c.load().w4_dispatch_mma_min_m() else cm
+    assert np.array_equal(cd, want) and np.array_equal(wd, w_ref)
+
+
+def test_w4_dequant_exhaustive_scales():
+    """Every FP16 scale x every code x every zero-point: the device dequant step
+    equals RNE_half(float(s) * (q - z)) bit for bit (NaN scales excluded)."""
+    c = w4amd.capi()
+    allh = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    fin = allh[~np.isnan(allh.view(np.float16))]
+    N = fin.size
+    # row n: scale fin[n]; 16 groups of 16 codes; group g has zero-point g, codes 0..15
+    K, gs = 16 * 16, 16
+    q = np.zeros((N, K // 8), np.uint32)
+    for k in range(K):
+        q[:, k // 8] |= np.uint32(k % 16) << np.uint32(4 * (k % 8))
+    zeros = np.zeros((N, 2), np.uint32)
+    for g in range(16):
+        zeros[:, g // 8] |= np.uint32(g) << np.uint32(4 * (g % 8))
+    scales = np.repeat(fin[:, None], 16, axis=1)
+    p = orc.PackedW(N, K, gs, False, q.ravel(), np.ascontiguousarray(scales).ravel(), zeros.ravel())
+    want = orc.dequant_all(p)
+    dp = DevPacked(p)
+    w_d = halves(N * K, 0x7E00)
+    c.dequant(dp.view, ptr(w_d))
+    assert np.array_equal(bits(w_d), want)
+    x_d = halves(K, 0x3C00)
+    c_d, w2 = halves(N), halves(N * K, 0x7E00)
+    c.gemm_fused(dp.view, ptr(x_d), ptr(c_d), 1, 0, ptr(w2))
+    assert np.array_equal(bits(w2), want)
+    c.gemm_mma(dp.view, ptr(x_d), ptr(c_d), 1, 0, ptr(w2.fill_(0x7E00)))
+    assert np.array_equal(bits(w2), want)
+
+
+def test_mx_dequant_exhaustive():
+    """All 255 valid scale bytes x 16 codes."""
+    c = w4amd.capi()
+    N, K = 255, 32
+    q = np.zeros((N, 4), np.uint32)
+    for k in range(K):
+        q[:, k // 8] |= np.uint32(k % 16) << np.uint32(4 * (k % 8))
+    p = orc.PackedWm(N, K, q.ravel(), np.arange(255, dtype=np.uint8))
+    want = orc.dequant_all_mx(p)
+    dp = DevPackedMx(p)
+    w_d = halves(N * K, 0x7E00)
+    c.dequant_mx(dp.view, ptr(w_d))
+    assert np.array_equal(bits(w_d), want)
+    x_d, c_d, w2 = halves(K, 0), halves(N), halves(N * K, 0x7E00)
+    c.gemm_fused_mx(dp.view, ptr(x_d), ptr(c_d), 1, 0, ptr(w2))
+    assert np.array_equal(bits(w2), want)
+    c.gemm_mma_mx(dp.view, ptr(x_d), ptr(c_d), 1, 0, ptr(w2.fill_(0x7E00)))
+    assert np.array_equal(bits(w2), want)

@@ -1,0 +1,55 @@
+"""Builds libw4amd.so (the gfx950 kernels + C ABI) in-tree with hipcc.
+
+    python w4a16-dequant-gemm_amd/build.py            # build if sources changed
+    python w4a16-dequant-gemm_amd/build.py --force
+"""
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(PKG, "csrc")
+LIB = os.path.join(PKG, "lib", "libw4amd.so")
+SOURCES = ["abi.hip", "dequant.hip", "gemm_simt.hip", "gemm_mfma.hip", "flash.hip", "baseline.hip"]
+HEADERS = ["dq.cuh", "kernels.h", os.path.join("..", "..", "include", "w4_abi.h")]
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    # packed-FP32 VALU forms stay off for every kernel in this library
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def _stale():
+    if not os.path.exists(LIB):
+        return True
+    t = os.path.getmtime(LIB)
+    deps = [os.path.join(CSRC, f) for f in SOURCES + HEADERS] + [os.path.abspath(__file__)]
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def build(force=False, verbose=True):
+    if not force and not _stale():
+        return LIB
+    os.makedirs(os.path.dirname(LIB), exist_ok=True)
+    objs, procs = [], []
+    os.makedirs(os.path.join(PKG, "lib", "obj"), exist_ok=True)
+    for src in SOURCES:
+        obj = os.path.join(PKG, "lib", "obj", src.replace(".hip", ".o"))
+        objs.append(obj)
+        cmd = ["hipcc", *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        procs.append((src, subprocess.Popen(cmd, stderr=subprocess.PIPE, text=True)))
+    for src, p in procs:
+        _, err = p.communicate()
+        err = "\n".join(l for l in err.splitlines() if "packed-fp32-ops" not in l)
+        if p.returncode != 0:
+            raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+        if verbose and err.strip():
+            print(err, file=sys.stderr)
+    subprocess.check_call(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs,
+                           "-lhipblaslt"])
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(force="--force" in sys.argv))

@@ -1,0 +1,356 @@
+// The C ABI of libw4amd.so: argument contracts first, then launches.
+//
+// Each entry point rejects a malformed call before any device work: the checks
+// read only the view structs and compare pointers with null, so a bad call
+// never dereferences, allocates or launches.  The contract lists follow the
+// reference launch wrappers (dequant.cuh:63-77, fused.cuh:175-194,
+// mma.cuh:237-254, mxfused.cuh:32-37,59-64,169-178,294-301,
+// kvflash.cuh:37-54,368-376,437-452,579-582,733-754).
+#include <hip/hip_runtime.h>
+#include <limits.h>
+#include <stdio.h>
+
+#include <mutex>
+
+#include "kernels.h"
+
+namespace {
+
+thread_local char g_msg[256] = "";
+
+int invalid(const char* msg) {
+  snprintf(g_msg, sizeof g_msg, "%s", msg);
+  return W4_EINVAL;
+}
+
+int runtime(const char* what, hipError_t e) {
+  snprintf(g_msg, sizeof g_msg, "%s: %s", what, hipGetErrorString(e));
+  return W4_ERUNTIME;
+}
+
+#define REQUIRE(cond, msg) \
+  do {                     \
+    if (!(cond)) return invalid(msg); \
+  } while (0)
+
+int done(const char* what, hipError_t e) {
+  return e == hipSuccess ? W4_OK : runtime(what, e);
+}
+
+// Measured on MI355X: the matrix-core kernel overtakes the vector kernel from
+// this activation-row count on.
+constexpr int DISPATCH_MMA_MIN_M = 2;
+
+// Largest M the reference's launch grids accept; kept so callers see the same
+// rejections (fused.cuh:187-194, mma.cuh:253-254).
+constexpr long long FUSED_MAX_M = 65535LL * 4;
+constexpr long long MMA_MAX_M = 65535LL * 64;
+
+int check_packed(const w4_packed_view* p, const char* who) {
+  static thread_local char buf[96];
+#define PK(cond, text)                                   \
+  do {                                                   \
+    if (!(cond)) {                                       \
+      snprintf(buf, sizeof buf, "%s: %s", who, text);    \
+      return invalid(buf);                               \
+    }                                                    \
+  } while (0)
+  PK(p != nullptr, "null view");
+  PK(p->N >= 1 && p->K >= 1, "bad dims");
+  PK(p->gs >= 8 && p->gs % 8 == 0, "gs must be a multiple of 8");
+  PK(p->G == (p->K + p->gs - 1) / p->gs, "G inconsistent with K, gs");
+  PK(p->q && p->scales, "null pointer");
+  PK(p->symmetric || p->zeros, "asymmetric without zeros");
+  PK(!p->symmetric || !p->zeros, "symmetric carries no zeros");
+#undef PK
+  return W4_OK;
+}
+
+int check_mx(const w4_packed_mx_view* p) {
+  REQUIRE(p != nullptr, "mx: null view");
+  REQUIRE(p->N >= 1 && p->K >= 1, "mx: bad dims");
+  REQUIRE(p->B == (p->K + 31) / 32, "mx: B inconsistent with K");
+  REQUIRE(p->q && p->scales, "mx: null pointer");
+  return W4_OK;
+}
+
+// Grow-only device scratch for the split-S partials, shared by all calls (calls
+// on different streams must not overlap, as with the reference's
+// kv_part_scratch, kvflash.cuh:56-69).
+std::mutex g_scratch_mu;
+float* g_scratch = nullptr;
+size_t g_scratch_cap = 0;
+
+hipError_t scratch_floats(size_t n, float** out) {
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (n > g_scratch_cap) {
+    float* nb = nullptr;
+    hipError_t e = hipMalloc((void**)&nb, n * sizeof(float));
+    if (e != hipSuccess) return e;
+    if (g_scratch) (void)hipFree(g_scratch);
+    g_scratch = nb;
+    g_scratch_cap = n;
+  }
+  *out = g_scratch;
+  return hipSuccess;
+}
+
+int check_kv_common(int H, int S, int D, int gs, int G, const char* who) {
+  static thread_local char buf[96];
+#define KV(cond, text)                                   \
+  do {                                                   \
+    if (!(cond)) {                                       \
+      snprintf(buf, sizeof buf, "%s: %s", who, text);    \
+      return invalid(buf);                               \
+    }                                                    \
+  } while (0)
+  KV(H >= 1 && S >= 1 && D >= 1, "bad dims");
+  KV(D <= 512, "D exceeds the 512-element bound");
+  KV(gs >= 8 && gs % 8 == 0, "gs must be a multiple of 8");
+  KV(G == (D + gs - 1) / gs, "G inconsistent with D, gs");
+#undef KV
+  return W4_OK;
+}
+
+int run_flash(w4k::FlashArgs& a, w4_stream stream, const char* what) {
+  float* scratch = nullptr;
+  hipError_t e = scratch_floats(w4k::flash_scratch_floats(a), &scratch);
+  if (e != hipSuccess) return runtime("flash scratch", e);
+  return done(what, w4k::launch_flash(a, scratch, (hipStream_t)stream));
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* w4_last_error(void) { return g_msg; }
+
+int w4_dispatch_mma_min_m(void) { return DISPATCH_MMA_MIN_M; }
+
+// ---- W4 ----------------------------------------------------------------------
+
+int w4_dequant(const w4_packed_view* p, w4_half* w, w4_stream stream) {
+  if (int rc = check_packed(p, "dequant")) return rc;
+  REQUIRE(w != nullptr, "dequant: null pointer");
+  REQUIRE((long long)p->N * ((p->K + 7) / 8) < (1LL << 31), "dequant: N*words(K) exceeds 2^31");
+  return done("dequant", w4k::launch_dequant(w4k::view_of(*p), w, (hipStream_t)stream));
+}
+
+int w4_gemm_fused(const w4_packed_view* p, const w4_half* x, w4_half* c, int M,
+                  w4_stream stream, w4_half* w_out) {
+  if (int rc = check_packed(p, "fused")) return rc;
+  REQUIRE(x && c, "fused: null pointer");
+  REQUIRE(M >= 1, "fused: bad M");
+  REQUIRE(M <= FUSED_MAX_M && p->N <= INT_MAX - 32, "fused: launch grid out of range");
+  return done("fused_kernel",
+              w4k::launch_gemm_simt(w4k::view_of(*p), x, c, M, (hipStream_t)stream, w_out));
+}
+
+int w4_gemm_mma(const w4_packed_view* p, const w4_half* x, w4_half* c, int M,
+                w4_stream stream, w4_half* w_out) {
+  if (int rc = check_packed(p, "mma")) return rc;
+  REQUIRE(x && c, "mma: null pointer");
+  REQUIRE(M >= 1, "mma: bad M");
+  REQUIRE(M <= MMA_MAX_M && p->N <= INT_MAX - 64, "mma: launch grid out of range");
+  return done("mma_kernel",
+              w4k::launch_gemm_mfma(w4k::view_of(*p), x, c, M, (hipStream_t)stream, w_out));
+}
+
+int w4_gemm(const w4_packed_view* p, const w4_half* x, w4_half* c, int M, w4_stream stream,
+            w4_half* w_out) {
+  return M < DISPATCH_MMA_MIN_M ? w4_gemm_fused(p, x, c, M, stream, w_out)
+                                : w4_gemm_mma(p, x, c, M, stream, w_out);
+}
+
+// ---- MXFP4 ---------------------------------------------------------------------
+
+int w4_dequant_mx(const w4_packed_mx_view* p, w4_half* w, w4_stream stream) {
+  if (int rc = check_mx(p)) return rc;
+  REQUIRE(w != nullptr, "mx dequant: null output");
+  REQUIRE((long long)p->N * ((p->K + 7) / 8) < (1LL << 31),
+          "mx dequant: N*words(K) exceeds 2^31");
+  return done("dequant_mx", w4k::launch_dequant(w4k::view_of(*p), w, (hipStream_t)stream));
+}
+
+int w4_gemm_fused_mx(const w4_packed_mx_view* p, const w4_half* x, w4_half* c, int M,
+                     w4_stream stream, w4_half* w_out) {
+  if (int rc = check_mx(p)) return rc;
+  REQUIRE(x && c, "mx fused: null pointer");
+  REQUIRE(M >= 1, "mx fused: bad M");
+  REQUIRE(M <= FUSED_MAX_M && p->N <= INT_MAX - 32, "mx fused: launch grid out of range");
+  return done("fused_kernel_mx",
+              w4k::launch_gemm_simt(w4k::view_of(*p), x, c, M, (hipStream_t)stream, w_out));
+}
+
+int w4_gemm_mma_mx(const w4_packed_mx_view* p, const w4_half* x, w4_half* c, int M,
+                   w4_stream stream, w4_half* w_out) {
+  if (int rc = check_mx(p)) return rc;
+  REQUIRE(x && c, "mx mma: null pointer");
+  REQUIRE(M >= 1, "mx mma: bad M");
+  REQUIRE(M <= MMA_MAX_M && p->N <= INT_MAX - 64, "mx mma: launch grid out of range");
+  return done("mma_kernel_mx",
+              w4k::launch_gemm_mfma(w4k::view_of(*p), x, c, M, (hipStream_t)stream, w_out));
+}
+
+int w4_gemm_mx(const w4_packed_mx_view* p, const w4_half* x, w4_half* c, int M,
+               w4_stream stream, w4_half* w_out) {
+  return M < DISPATCH_MMA_MIN_M ? w4_gemm_fused_mx(p, x, c, M, stream, w_out)
+                                : w4_gemm_mma_mx(p, x, c, M, stream, w_out);
+}
+
+// ---- attention -------------------------------------------------------------------
+
+static int check_kv_w4(const w4_kv_view* p, const char* who) {
+  REQUIRE(p != nullptr, "kv flash: null view");
+  if (int rc = check_kv_common(p->H, p->S, p->D, p->gs, p->G, who)) return rc;
+  REQUIRE(p->q_k && p->s_k && p->q_v && p->s_v, "kv flash: null pointer");
+  REQUIRE(p->symmetric || (p->z_k && p->z_v), "kv flash: asymmetric without zeros");
+  REQUIRE(!p->symmetric || (!p->z_k && !p->z_v), "kv flash: symmetric carries no zeros");
+  REQUIRE(p->S <= 65535 * 256, "kv flash: S exceeds the tile-grid bound");
+  return W4_OK;
+}
+
+static void fill_w4(w4k::FlashArgs& a, const w4_kv_view* p, int group) {
+  a = w4k::FlashArgs{};
+  a.kind = 1;
+  a.H = p->H; a.S = p->S; a.D = p->D; a.gs = p->gs; a.G = p->G;
+  a.symmetric = p->symmetric;
+  a.group = group;
+  a.k = p->q_k; a.v = p->q_v; a.s_k = p->s_k; a.s_v = p->s_v;
+  a.z_k = p->z_k; a.z_v = p->z_v;
+  a.Hkv = p->H;
+}
+
+int w4_attention_w4_flash_gqa(const w4_kv_view* p, int group, const w4_half* q, w4_half* out,
+                              w4_stream stream, w4_half* k_out, w4_half* v_out) {
+  if (int rc = check_kv_w4(p, "kv flash")) return rc;
+  REQUIRE(q && out, "kv flash w4: null pointer");
+  REQUIRE(group >= 1 && group <= 64, "kv flash w4: bad query group");
+  w4k::FlashArgs a;
+  fill_w4(a, p, group);
+  a.q = q; a.out = out; a.k_out = k_out; a.v_out = v_out;
+  return run_flash(a, stream, "flash_w4");
+}
+
+int w4_attention_w4_flash(const w4_kv_view* p, const w4_half* q, w4_half* out,
+                          w4_stream stream, w4_half* k_out, w4_half* v_out) {
+  return w4_attention_w4_flash_gqa(p, 1, q, out, stream, k_out, v_out);
+}
+
+int w4_attention_fp16_flash_gqa(const w4_half* q, const w4_half* k16, const w4_half* v16,
+                                w4_half* out, int H, int group, int S, int D,
+                                w4_stream stream) {
+  REQUIRE(H >= 1 && S >= 1 && D >= 1, "kv flash fp16: bad dims");
+  REQUIRE(D <= 512, "kv flash fp16: D exceeds the 512-element bound");
+  REQUIRE(S <= 65535 * 256, "kv flash fp16: S exceeds the tile-grid bound");
+  REQUIRE(q && k16 && v16 && out, "kv flash fp16: null pointer");
+  REQUIRE(group >= 1 && group <= 64, "kv flash fp16: bad query group");
+  w4k::FlashArgs a{};
+  a.kind = 0;
+  a.H = H; a.S = S; a.D = D; a.gs = 8; a.G = 1; a.symmetric = 1; a.group = group;
+  a.k = k16; a.v = v16; a.Hkv = H;
+  a.q = q; a.out = out;
+  return run_flash(a, stream, "flash_fp16");
+}
+
+int w4_attention_fp16_flash(const w4_half* q, const w4_half* k16, const w4_half* v16,
+                            w4_half* out, int H, int S, int D, w4_stream stream) {
+  return w4_attention_fp16_flash_gqa(q, k16, v16, out, H, 1, S, D, stream);
+}
+
+int w4_attention_f8_flash_gqa(const w4_kv_f8_view* p, int group, int scale_mode,
+                              const w4_half* q, w4_half* out, w4_stream stream,
+                              w4_half* k_out, w4_half* v_out) {
+  REQUIRE(p != nullptr, "kv f8 flash: null view");
+  if (int rc = check_kv_common(p->H, p->S, p->D, p->gs, p->G, "kv f8 flash")) return rc;
+  REQUIRE(p->q_k && p->s_k && p->q_v && p->s_v, "kv f8 flash: null pointer");
+  REQUIRE(p->S <= 65535 * 256, "kv f8 flash: S exceeds the tile-grid bound");
+  REQUIRE(q && out, "kv f8 flash: null io pointer");
+  REQUIRE(p->D % 4 == 0, "kv f8 flash: D must be a multiple of 4");
+  REQUIRE((uintptr_t)p->q_k % 4 == 0 && (uintptr_t)p->q_v % 4 == 0,
+          "kv f8 flash: cache bases 4-byte aligned");
+  REQUIRE(group >= 1 && group <= 64, "kv f8 flash: bad query group");
+  REQUIRE(scale_mode == 0 || scale_mode == 1, "kv f8 flash: bad scale mode");
+  w4k::FlashArgs a{};
+  a.kind = 2;
+  a.H = p->H; a.S = p->S; a.D = p->D; a.gs = p->gs; a.G = p->G; a.symmetric = 1;
+  a.group = group; a.scale_mode = scale_mode;
+  a.k = p->q_k; a.v = p->q_v; a.s_k = p->s_k; a.s_v = p->s_v; a.Hkv = p->H;
+  a.q = q; a.out = out; a.k_out = k_out; a.v_out = v_out;
+  return run_flash(a, stream, "flash_f8");
+}
+
+int w4_attention_f8_flash(const w4_kv_f8_view* p, const w4_half* q, w4_half* out,
+                          w4_stream stream, w4_half* k_out, w4_half* v_out) {
+  return w4_attention_f8_flash_gqa(p, 1, 0, q, out, stream, k_out, v_out);
+}
+
+static int check_paged(const w4_kv_view* p, const int* bt, int page, int npages) {
+  REQUIRE(p != nullptr, "kv paged flash: null view");
+  if (int rc = check_kv_common(p->H, p->S, p->D, p->gs, p->G, "kv paged flash")) return rc;
+  REQUIRE(p->q_k && p->s_k && p->q_v && p->s_v && bt, "kv paged flash: null pointer");
+  REQUIRE(p->symmetric || (p->z_k && p->z_v), "kv paged flash: asymmetric without zeros");
+  REQUIRE(!p->symmetric || (!p->z_k && !p->z_v), "kv paged flash: symmetric carries zeros");
+  REQUIRE(page >= 1 && npages >= 1 && (long long)npages * page >= (long long)p->S,
+          "kv paged flash: bad page geometry");
+  REQUIRE((long long)npages * page < (1LL << 31), "kv paged flash: pool rows exceed 2^31");
+  REQUIRE(p->S <= 65535 * 256, "kv paged flash: S exceeds tile-grid bound");
+  return W4_OK;
+}
+
+int w4_attention_w4_flash_paged(const w4_kv_view* p, const int* bt, int page, int npages,
+                                const w4_half* q, w4_half* out, w4_stream stream,
+                                w4_half* k_out, w4_half* v_out) {
+  if (int rc = check_paged(p, bt, page, npages)) return rc;
+  REQUIRE(q && out, "kv paged flash: null io");
+  w4k::FlashArgs a;
+  fill_w4(a, p, 1);
+  a.bt = bt; a.bt_stride = 0; a.page = page; a.pool_rows = npages * page;
+  a.Hkv = p->H;  // one table for every head: sequence index is always 0
+  a.q = q; a.out = out; a.k_out = k_out; a.v_out = v_out;
+  return run_flash(a, stream, "flash_w4_paged");
+}
+
+int w4_attention_w4_flash_paged_batched(const w4_kv_view* p, const int* bt, int nseq,
+                                        int bt_stride, int page, int npages, int group,
+                                        const w4_half* q, w4_half* out, w4_stream stream) {
+  if (int rc = check_paged(p, bt, page, npages)) return rc;
+  REQUIRE(q && out, "kv paged flash: null io");
+  REQUIRE(nseq >= 1 && group >= 1 && group <= 64, "kv paged flash: bad batch");
+  REQUIRE(bt_stride >= (p->S + page - 1) / page, "kv paged flash: table stride too short");
+  REQUIRE((long long)nseq * p->H < (1LL << 31), "kv paged flash: too many slabs");
+  w4k::FlashArgs a;
+  fill_w4(a, p, group);
+  a.H = nseq * p->H;
+  a.Hkv = p->H;
+  a.bt = bt; a.bt_stride = bt_stride; a.page = page; a.pool_rows = npages * page;
+  a.q = q; a.out = out;
+  return run_flash(a, stream, "flash_w4_paged");
+}
+
+int w4_dequant_f8(const uint8_t* q, const w4_half* s, w4_half* w, int S, int D, int gs,
+                  w4_stream stream) {
+  REQUIRE(S >= 1 && D >= 1, "f8 dequant: bad dims");
+  REQUIRE(gs >= 8 && gs % 8 == 0, "f8 dequant: gs must be a multiple of 8");
+  REQUIRE(q && s && w, "f8 dequant: null pointer");
+  REQUIRE((long long)S * ((D + 3) / 4) < (1LL << 31), "f8 dequant: S*words4(D) exceeds 2^31");
+  REQUIRE(D % 4 == 0, "f8 dequant: D must be a multiple of 4");
+  REQUIRE((uintptr_t)q % 4 == 0, "f8 dequant: q must be 4-byte aligned");
+  return done("dequant_f8", w4k::launch_dequant_f8(q, s, w, S, D, gs, (hipStream_t)stream));
+}
+
+}  // extern "C"
+
+// ---- two-pass baseline -------------------------------------------------------------
+extern "C" int w4_gemm_fp16_impl(const w4_half*, const w4_half*, w4_half*, int, int, int,
+                                 w4_stream);
+extern "C" const char* w4_blas_last_error(void);
+
+extern "C" int w4_gemm_fp16(const w4_half* w, const w4_half* x, w4_half* c, int M, int N,
+                            int K, w4_stream stream) {
+  REQUIRE(M >= 1 && N >= 1 && K >= 1, "gemm_fp16: bad dims");
+  REQUIRE(w && x && c, "gemm_fp16: null pointer");
+  const int rc = w4_gemm_fp16_impl(w, x, c, M, N, K, stream);
+  if (rc != W4_OK) snprintf(g_msg, sizeof g_msg, "%s", w4_blas_last_error());
+  return rc;
+}

@@ -1,0 +1,189 @@
+// Fused dequant + GEMM on the matrix cores (v_mfma_f32_16x16x32_f16).
+//
+// One packed word -- 8 consecutive k of one weight row -- is exactly one lane's
+// A operand of a 16x16x32 MFMA (lane l: row l%16, k-block l/16).  A lane loads
+// a dwordx4 (4 words of its row), expands each word in VGPRs and feeds four
+// MFMAs; packed W never passes through LDS and FP16 W never exists in memory.
+// The contraction order inside a 128-k chunk is permuted (MFMA j takes word j
+// of every lane, i.e. k-block 4*(l/16)+j); the B operand reads the activations
+// with the same permutation, so the sum is unchanged.
+//
+// D = A*B gives lane l the outputs (n = 4*(l/16)+i, m = l%16): four consecutive
+// n of one activation row, stored as one 8-byte write.
+//
+// Skinny kernel (this file's first kernel): a workgroup owns 16 weight rows and
+// up to 64 activation rows; its 4 waves split K chunk-wise and combine through
+// LDS in a fixed order, so results are deterministic and every CU streams W
+// even when N/16 is only a few hundred.
+#include "dq.cuh"
+#include "kernels.h"
+
+namespace w4k {
+
+constexpr int MMA_WAVES = 4;
+constexpr int MMA_CHUNK = 128;  // k per lane-load step (16 words per row)
+
+__device__ __forceinline__ h8 pack_h8(const h2 n[4]) {
+  return h8{n[0][0], n[0][1], n[1][0], n[1][1], n[2][0], n[2][1], n[3][0], n[3][1]};
+}
+
+// 8 activations x[m][k .. k+8), zero past M / K.
+template <bool XVEC>
+__device__ __forceinline__ h8 load_x8(const w4_half* __restrict__ x, int M, int K, int m,
+                                      int k) {
+  u4 v = {0u, 0u, 0u, 0u};
+  if (m < M && k < K) {
+    const uint16_t* src = x + (size_t)m * K + k;
+    if (XVEC) {
+      v = *(const u4*)src;
+    } else {
+      uint16_t t[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) t[j] = (k + j < K) ? src[j] : (uint16_t)0;
+      v = u4{t[0] | ((uint32_t)t[1] << 16), t[2] | ((uint32_t)t[3] << 16),
+             t[4] | ((uint32_t)t[5] << 16), t[6] | ((uint32_t)t[7] << 16)};
+    }
+  }
+  return __builtin_bit_cast(h8, v);
+}
+
+template <int MX, int MTILES, bool HOOK, bool FAST>
+__global__ __launch_bounds__(MMA_WAVES * 64) void mfma_skinny_kernel(
+    const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
+    w4_half* __restrict__ w_out) {
+  __shared__ f4 red[MMA_WAVES - 1][MTILES][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, b = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int m0 = blockIdx.y * (16 * MTILES);
+  const int wpr = words(p.K);
+  const int n = min(n0 + r, p.N - 1);
+  const bool row_ok = n0 + r < p.N;
+  const bool hook = HOOK && blockIdx.y == 0 && row_ok;
+  const int wg = MX ? 0 : words(p.G);
+  const int nchunks = (p.K + MMA_CHUNK - 1) / MMA_CHUNK;
+
+  f4 acc[MTILES];
+#pragma unroll
+  for (int t = 0; t < MTILES; ++t) acc[t] = f4{0.f, 0.f, 0.f, 0.f};
+
+  for (int ch = wave; ch < nchunks; ch += MMA_WAVES) {
+    const int w0 = ch * 16 + 4 * b;  // first of this lane's 4 words
+    u4 qw = {0u, 0u, 0u, 0u};
+    if (FAST) {
+      qw = __builtin_nontemporal_load((const u4*)(p.q + (size_t)n * wpr + w0));
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (w0 + j < wpr) qw[j] = p.q[(size_t)n * wpr + w0 + j];
+    }
+    MxBlock mb;
+    bool any_wide = false;
+    if (MX) {
+      const int blk = min(w0 >> 2, p.B - 1);
+      mb = mx_block(((const uint8_t*)p.scales)[(size_t)n * p.B + blk]);
+      any_wide = __builtin_amdgcn_ballot_w64(mb.wide) != 0;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k0 = (w0 + j) * 8;
+      h2 d[4], nat[4];
+      if (MX) {
+        dq_mx(qw[j], mb, any_wide, d);
+      } else {
+        const int g = min(k0 / p.gs, p.G - 1);
+        const int z = p.symmetric ? 8
+                                  : (int)((p.zeros[(size_t)n * wg + (g >> 3)] >>
+                                           (4 * (g & 7))) & 0xF);
+        dq_w4(qw[j], w4_group(((const uint16_t*)p.scales)[(size_t)n * p.G + g], z), d);
+      }
+      to_natural(d, nat);
+      if (hook && k0 < p.K) {
+        uint16_t* out = w_out + (size_t)n * p.K + k0;
+        if (FAST) {
+          *(u4*)out = u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (k0 + e < p.K) {
+              const uint32_t pair = as_u32(nat[e >> 1]);
+              out[e] = (uint16_t)((e & 1) ? pair >> 16 : pair & 0xFFFFu);
+            }
+        }
+      }
+      const h8 a = pack_h8(nat);
+#pragma unroll
+      for (int t = 0; t < MTILES; ++t) {
+        const h8 bx = load_x8<FAST>(x, M, p.K, m0 + 16 * t + r, k0);
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bx, acc[t], 0, 0, 0);
+      }
+    }
+  }
+
+  // Fixed-order combine of the four K slices: wave 0 adds waves 1, 2, 3.
+  if (wave > 0) {
+#pragma unroll
+    for (int t = 0; t < MTILES; ++t) red[wave - 1][t][lane] = acc[t];
+  }
+  __syncthreads();
+  if (wave == 0) {
+#pragma unroll
+    for (int t = 0; t < MTILES; ++t) {
+      f4 s = acc[t];
+#pragma unroll
+      for (int w = 0; w < MMA_WAVES - 1; ++w) s += red[w][t][lane];
+      const int m = m0 + 16 * t + r;  // activation row of this lane
+      const int nn = n0 + 4 * b;      // first of its 4 weight rows
+      if (m < M) {
+        uint16_t hv[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const _Float16 h = (_Float16)s[i];
+          hv[i] = __builtin_bit_cast(uint16_t, h);
+        }
+        uint16_t* dst = c + (size_t)m * p.N + nn;
+        if (nn + 3 < p.N && (p.N & 3) == 0 && (((uintptr_t)c & 7) == 0)) {
+          *(u2*)dst = u2{hv[0] | ((uint32_t)hv[1] << 16), hv[2] | ((uint32_t)hv[3] << 16)};
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (nn + i < p.N) dst[i] = hv[i];
+        }
+      }
+    }
+  }
+}
+
+template <int MX, int MTILES>
+static hipError_t launch_tiles(const WView& v, const w4_half* x, w4_half* c, int M,
+                               hipStream_t s, w4_half* w_out) {
+  const bool fast = (v.K % 32 == 0) && (((uintptr_t)v.q & 15) == 0) &&
+                    (((uintptr_t)x & 15) == 0) &&
+                    (w_out == nullptr || ((uintptr_t)w_out & 15) == 0);
+  const dim3 grid((unsigned)((v.N + 15) / 16),
+                  (unsigned)((M + 16 * MTILES - 1) / (16 * MTILES)));
+#define W4_GO(HOOK, FAST) \
+  mfma_skinny_kernel<MX, MTILES, HOOK, FAST><<<grid, MMA_WAVES * 64, 0, s>>>(v, x, c, M, w_out)
+  if (w_out) {
+    if (fast) W4_GO(true, true); else W4_GO(true, false);
+  } else {
+    if (fast) W4_GO(false, true); else W4_GO(false, false);
+  }
+#undef W4_GO
+  return hipGetLastError();
+}
+
+template <int MX>
+static hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M,
+                             hipStream_t s, w4_half* w_out) {
+  if (M <= 16) return launch_tiles<MX, 1>(v, x, c, M, s, w_out);
+  if (M <= 32) return launch_tiles<MX, 2>(v, x, c, M, s, w_out);
+  return launch_tiles<MX, 4>(v, x, c, M, s, w_out);
+}
+
+hipError_t launch_gemm_mfma(const WView& v, const w4_half* x, w4_half* c, int M,
+                            hipStream_t s, w4_half* w_out) {
+  return v.mx ? launch_fmt<1>(v, x, c, M, s, w_out) : launch_fmt<0>(v, x, c, M, s, w_out);
+}
+
+}  // namespace w4k

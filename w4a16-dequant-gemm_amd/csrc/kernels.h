@@ -1,0 +1,69 @@
+// Launch functions of the gfx950 kernels (one per kernel family).  They take
+// already-validated arguments and only enqueue work on `stream`.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/w4_abi.h"
+
+namespace w4k {
+
+// Which packed format a weight view carries.
+struct WView {
+  int mx;  // 0: W4 affine (scales FP16, optional zero-points), 1: MXFP4
+  int N, K;
+  int gs, G, symmetric;  // W4 only
+  int B;                 // MX only
+  const uint32_t* q;
+  const void* scales;  // w4_half* (W4) or uint8_t* (MX)
+  const uint32_t* zeros;
+};
+
+inline WView view_of(const w4_packed_view& p) {
+  return WView{0, p.N, p.K, p.gs, p.G, p.symmetric, 0, p.q, p.scales, p.zeros};
+}
+inline WView view_of(const w4_packed_mx_view& p) {
+  return WView{1, p.N, p.K, 32, p.B, 1, p.B, p.q, p.scales, nullptr};
+}
+
+// dequant.hip
+hipError_t launch_dequant(const WView& v, w4_half* w, hipStream_t s);
+hipError_t launch_dequant_f8(const uint8_t* q, const w4_half* sc, w4_half* w,
+                             int S, int D, int gs, hipStream_t s);
+
+// gemm_simt.hip
+hipError_t launch_gemm_simt(const WView& v, const w4_half* x, w4_half* c, int M,
+                            hipStream_t s, w4_half* w_out);
+// gemm_mfma.hip
+hipError_t launch_gemm_mfma(const WView& v, const w4_half* x, w4_half* c, int M,
+                            hipStream_t s, w4_half* w_out);
+
+// flash.hip -- one description for the four cache kinds
+struct FlashArgs {
+  int kind;  // 0 FP16, 1 W4, 2 FP8
+  int H;     // cache slabs addressed by a (sequence, kv-head) pair: nseq * Hkv
+  int S, D, gs, G, symmetric;
+  int group;       // query heads per slab
+  int scale_mode;  // FP8: 0 per (row, group), 1 per slab
+  const void* k;   // FP16: halves; W4: packed words; FP8: bytes
+  const void* v;
+  const w4_half* s_k;
+  const w4_half* s_v;
+  const uint32_t* z_k;
+  const uint32_t* z_v;
+  // paging (W4 only): bt == nullptr means contiguous slabs of S rows
+  const int* bt;
+  int bt_stride;   // entries per sequence table
+  int page, pool_rows;
+  int Hkv;         // paged: pool slabs; sequence = slab / Hkv
+  const w4_half* q;
+  w4_half* out;
+  w4_half* k_out;
+  w4_half* v_out;
+};
+// Floats of scratch the split-S partials need for these arguments.
+size_t flash_scratch_floats(const FlashArgs& a);
+hipError_t launch_flash(const FlashArgs& a, float* scratch, hipStream_t s);
+
+}  // namespace w4k

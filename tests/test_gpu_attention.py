@@ -1,0 +1,242 @@
+"""GPU parity gates for split-S flash-decode attention, through the C ABI.
+
+Follows the reference device suite (tests/test_gpu.cu:506-1467): k_out/v_out
+hooks equal the oracle's per-head dequant bit for bit, outputs are within rel
+L2 1e-3 of the FP64 softmax(QK^T/sqrt(D))V over the dequantized cache, the FP16
+flash path over the dequantized cache is within 2e-3 of the W4 path, and the
+paged kernel reproduces the contiguous kernel's bytes.
+"""
+import numpy as np
+import pytest
+import torch
+
+import orc
+import w4amd
+from devutil import DevKV, DevKVF8, bits, f64, halves, ptr, to_dev
+
+pytestmark = pytest.mark.gpu
+TOL, CROSS = 1e-3, 2e-3
+
+ATT = [(1, 1, 64, 32), (2, 7, 64, 8), (4, 128, 128, 128), (2, 300, 96, 32), (3, 65, 40, 8),
+       (1, 4096, 64, 64)]
+BIG = [(2, 5000, 64, 32), (1, 9000, 128, 64)]
+
+
+def _w4_case(H, S, D, gs, sym, seed, group=1):
+    k = orc.normal_weights(H * S * D, seed)
+    v = orc.normal_weights(H * S * D, seed + 1)
+    q = orc.normal_activations(H * group * D, seed + 2)
+    c4 = orc.quantize_cache(k, v, H, S, D, gs, sym)
+    return c4, q
+
+
+def _check_w4(c4, q, group=1):
+    c = w4amd.capi()
+    H, S, D = c4.H, c4.S, c4.D
+    kd, vd = orc.dequant_cache(c4, False), orc.dequant_cache(c4, True)
+    ref = orc.attention_f16(q, kd, vd, H, group, S, D)
+    dk, q_d = DevKV(c4), to_dev(q)
+    out = halves(H * group * D, 0x7E00)
+    ko, vo = halves(H * S * D, 0x7E00), halves(H * S * D, 0x7E00)
+    c.attention_w4_flash(dk.view, ptr(q_d), ptr(out), 0, ptr(ko), ptr(vo), group=group)
+    assert np.array_equal(bits(ko), kd.ravel()), "k_out bitwise"
+    assert np.array_equal(bits(vo), vd.ravel()), "v_out bitwise"
+    o_w4 = bits(out).copy()
+    assert orc.rel_l2(o_w4.view(np.float16), ref) <= TOL
+    # no hooks: same bytes
+    out2 = halves(H * group * D, 0x7E00)
+    c.attention_w4_flash(dk.view, ptr(q_d), ptr(out2), group=group)
+    assert np.array_equal(bits(out2), o_w4)
+    # FP16 flash over the dequantized cache: oracle gate + cross gate
+    k16, v16, o16 = to_dev(kd), to_dev(vd), halves(H * group * D, 0x7E00)
+    c.attention_fp16_flash(ptr(q_d), ptr(k16), ptr(v16), ptr(o16), H, S, D, group=group)
+    assert orc.rel_l2(f64(o16), ref) <= TOL
+    den = np.sqrt(np.sum(ref ** 2))
+    cross = np.sqrt(np.sum((f64(o16) - o_w4.view(np.float16).astype(np.float64)) ** 2)) / den
+    assert cross <= CROSS
+    return o_w4, dk, q_d, kd, vd, ref
+
+
+@pytest.mark.parametrize("sym", [True, False], ids=["sym", "asym"])
+@pytest.mark.parametrize("i", range(len(ATT)))
+def test_w4_flash(i, sym):
+    H, S, D, gs = ATT[i]
+    c4, q = _w4_case(H, S, D, gs, sym, 0x77B5 ^ (i * 977 + (0 if sym else 1)))
+    _check_w4(c4, q)
+
+
+@pytest.mark.parametrize("sym", [True, False], ids=["sym", "asym"])
+@pytest.mark.parametrize("i", range(len(BIG)))
+def test_w4_flash_long(i, sym):
+    H, S, D, gs = BIG[i]
+    c4, q = _w4_case(H, S, D, gs, sym, 0x51D0 ^ (i * 977 + (0 if sym else 1)))
+    _check_w4(c4, q)
+
+
+@pytest.mark.parametrize("group", [2, 3, 4, 7])
+def test_w4_flash_grouped_query(group):
+    c4, q = _w4_case(3, 700, 128, 32, True, 0x6A11 + group, group)
+    _check_w4(c4, q, group)
+
+
+F8 = [(1, 1, 64, 32), (2, 7, 64, 8), (4, 128, 128, 128), (2, 300, 96, 32), (3, 65, 40, 8),
+      (1, 9000, 128, 64)]
+
+
+@pytest.mark.parametrize("i", range(len(F8)))
+def test_f8_flash(i):
+    c = w4amd.capi()
+    H, S, D, gs = F8[i]
+    seed = 0xF80A ^ (i * 977)
+    k = orc.normal_weights(H * S * D, seed)
+    v = orc.normal_weights(H * S * D, seed + 1)
+    q = orc.normal_activations(H * D, seed + 2)
+    c8 = orc.quantize_cache_f8(k, v, H, S, D, gs)
+    kd, vd = orc.dequant_cache_f8(c8, False), orc.dequant_cache_f8(c8, True)
+    ref = orc.attention_f16(q, kd, vd, H, 1, S, D)
+    d8, q_d = DevKVF8(c8), to_dev(q)
+    out, ko, vo = halves(H * D, 0x7E00), halves(H * S * D, 0x7E00), halves(H * S * D, 0x7E00)
+    c.attention_f8_flash(d8.view, ptr(q_d), ptr(out), 0, ptr(ko), ptr(vo))
+    assert np.array_equal(bits(ko), kd.ravel()) and np.array_equal(bits(vo), vd.ravel())
+    assert orc.rel_l2(f64(out), ref) <= TOL
+    # device two-pass: dequant_f8 per side, then FP16 flash
+    k16, v16, o16 = halves(H * S * D), halves(H * S * D), halves(H * D)
+    c.dequant_f8(ptr(d8.t[0]), ptr(d8.t[1]), ptr(k16), H * S, D, gs)
+    c.dequant_f8(ptr(d8.t[2]), ptr(d8.t[3]), ptr(v16), H * S, D, gs)
+    assert np.array_equal(bits(k16), kd.ravel()) and np.array_equal(bits(v16), vd.ravel())
+    c.attention_fp16_flash(ptr(q_d), ptr(k16), ptr(v16), ptr(o16), H, S, D)
+    den = np.sqrt(np.sum(ref ** 2))
+    assert np.sqrt(np.sum((f64(o16) - f64(out)) ** 2)) / den <= CROSS
+
+
+def test_f8_every_code_and_slab_scale():
+    """All 256 byte codes under several scales (hooks bit-exact), then the
+    per-slab scale mode against the reference arithmetic on a broadcast scale."""
+    c = w4amd.capi()
+    H, S, D, gs = 2, 64, 32, 32
+    c8 = orc.KVCacheF8()
+    c8.H, c8.S, c8.D, c8.gs, c8.G = H, S, D, gs, 1
+    codes = (np.arange(H * S * D) % 256).astype(np.uint8)
+    c8.q_k, c8.q_v = codes, codes[::-1].copy()
+    sc = np.array([0x3C00, 0x0001, 0x03FF, 0x5BFF, 0x7BFF, 0x2E66, 0x8400, 0x1400], np.uint16)
+    c8.s_k = np.resize(sc, H * S)
+    c8.s_v = np.resize(sc[::-1], H * S)
+    kd, vd = orc.dequant_cache_f8(c8, False), orc.dequant_cache_f8(c8, True)
+    d8 = DevKVF8(c8)
+    q_d = to_dev(np.zeros(H * D, np.uint16))
+    out, ko, vo = halves(H * D), halves(H * S * D, 0x7E00), halves(H * S * D, 0x7E00)
+    c.attention_f8_flash(d8.view, ptr(q_d), ptr(out), 0, ptr(ko), ptr(vo))
+    assert np.array_equal(bits(ko), kd.ravel()) and np.array_equal(bits(vo), vd.ravel())
+    # per-slab scale: one FP16 scale per slab == the same value in every slot
+    rng = np.random.default_rng(2)
+    kk = rng.standard_normal(H * S * D)
+    c8 = orc.quantize_cache_f8(kk, kk[::-1].copy(), H, S, D, gs)
+    slab_k = np.array([0x2000, 0x2400], np.uint16)
+    slab_v = np.array([0x2200, 0x1C00], np.uint16)
+    c8b = orc.KVCacheF8()
+    c8b.__dict__.update(c8.__dict__)
+    c8b.s_k, c8b.s_v = np.repeat(slab_k, S), np.repeat(slab_v, S)
+    q = orc.normal_activations(H * 2 * D, 77)
+    ref = orc.attention_reference_f8(q, c8b, heads_per_slab=2)
+    d8 = DevKVF8(c8, slab_k, slab_v)
+    out = halves(H * 2 * D, 0x7E00)
+    ko, vo = halves(H * S * D, 0x7E00), halves(H * S * D, 0x7E00)
+    c.attention_f8_flash(d8.view, ptr(to_dev(q)), ptr(out), 0, ptr(ko), ptr(vo), group=2, scale_mode=1)
+    assert np.array_equal(bits(ko), orc.dequant_cache_f8(c8b, False).ravel())
+    assert orc.rel_l2(f64(out), ref) <= TOL
+
+
+PAGED = [(2, 300, 96, 32, 16), (2, 520, 64, 32, 16), (1, 1000, 128, 64, 64), (3, 65, 40, 8, 32),
+         (1, 5000, 64, 32, 256)]
+
+
+def _paged_pool(c4, page, bt):
+    """Device copy of the cache scattered into a pool by `bt` (kvpaged.hpp:72-134)."""
+    c = w4amd.capi()
+    H, S, D, G = c4.H, c4.S, c4.D, c4.G
+    wd, wg = orc.words(D), orc.words(G)
+    t = [to_dev(orc.paged_scatter(c4.q_k, H, S, page, bt, wd)),
+         to_dev(orc.paged_scatter(c4.s_k, H, S, page, bt, G)),
+         None if c4.symmetric else to_dev(orc.paged_scatter(c4.z_k, H, S, page, bt, wg)),
+         to_dev(orc.paged_scatter(c4.q_v, H, S, page, bt, wd)),
+         to_dev(orc.paged_scatter(c4.s_v, H, S, page, bt, G)),
+         None if c4.symmetric else to_dev(orc.paged_scatter(c4.z_v, H, S, page, bt, wg))]
+    view = c.kv_view(H, S, D, c4.gs, G, c4.symmetric, *[ptr(x) for x in t])
+    return t, view
+
+
+@pytest.mark.parametrize("sym", [True, False], ids=["sym", "asym"])
+@pytest.mark.parametrize("i", range(len(PAGED)))
+def test_paged_equals_contiguous(i, sym):
+    c = w4amd.capi()
+    H, S, D, gs, page = PAGED[i]
+    seed = 0x9A6E ^ (i * 977 + (0 if sym else 1))
+    c4, q = _w4_case(H, S, D, gs, sym, seed)
+    o_w4, dk, q_d, kd, vd, ref = _check_w4(c4, q)
+    npages = (S + page - 1) // page
+    bt = np.random.default_rng(seed ^ 0x5ED).permutation(npages).astype(np.int32)
+    keep, view = _paged_pool(c4, page, bt)
+    bt_d = to_dev(bt)
+    out, ko, vo = halves(H * D, 0x7E00), halves(H * S * D, 0x7E00), halves(H * S * D, 0x7E00)
+    c.attention_w4_flash_paged(view, ptr(bt_d), page, npages, ptr(q_d), ptr(out), 0, ptr(ko), ptr(vo))
+    assert np.array_equal(bits(out), o_w4), "paged output == contiguous output, bytewise"
+    assert np.array_equal(bits(ko), kd.ravel()) and np.array_equal(bits(vo), vd.ravel())
+
+
+def test_paged_batched_prefix_sharing():
+    """Four sequences over one pool; the first three share their leading pages.
+    Each sequence's output equals the contiguous kernel run on its logical cache."""
+    c = w4amd.capi()
+    Hkv, D, gs, page, group = 2, 64, 32, 16, 2
+    S, prefix = 520, 208                     # 13 shared pages
+    nseq = 4
+    lp = (S + page - 1) // page
+    pp = prefix // page
+    rng = np.random.default_rng(0xCAFE)
+    # logical caches: sequences 0..2 share the prefix rows, sequence 3 is independent
+    base_k = orc.normal_weights(Hkv * S * D, 0xBEEF).reshape(Hkv, S, D)
+    base_v = orc.normal_weights(Hkv * S * D, 0xBEE0).reshape(Hkv, S, D)
+    caches = []
+    for s in range(nseq):
+        k = orc.normal_weights(Hkv * S * D, 0x1000 + s).reshape(Hkv, S, D)
+        v = orc.normal_weights(Hkv * S * D, 0x2000 + s).reshape(Hkv, S, D)
+        if s < 3:
+            k[:, :prefix], v[:, :prefix] = base_k[:, :prefix], base_v[:, :prefix]
+        caches.append(orc.quantize_cache(k, v, Hkv, S, D, gs, True))
+    # pool: shared prefix pages once, then each sequence's own pages, shuffled placement
+    npages = pp + 3 * (lp - pp) + lp
+    phys = rng.permutation(npages).astype(np.int32)
+    tables = np.zeros((nseq, lp), np.int32)
+    nxt = pp
+    for s in range(nseq):
+        for i in range(lp):
+            if s < 3 and i < pp:
+                tables[s, i] = phys[i]
+            else:
+                tables[s, i] = phys[nxt]
+                nxt += 1
+    assert nxt == npages
+    wd, G = orc.words(D), caches[0].G
+    pool = {n: np.zeros((Hkv, npages * page, w), dt) for n, w, dt in
+            (("q_k", wd, np.uint32), ("q_v", wd, np.uint32), ("s_k", G, np.uint16), ("s_v", G, np.uint16))}
+    for s, c4 in enumerate(caches):
+        for n in pool:
+            src = getattr(c4, n).reshape(Hkv, S, -1)
+            for t in range(S):
+                pool[n][:, tables[s, t // page] * page + t % page] = src[:, t]
+    dev = {n: to_dev(a.ravel()) for n, a in pool.items()}
+    view = c.kv_view(Hkv, S, D, gs, G, True, ptr(dev["q_k"]), ptr(dev["s_k"]), 0, ptr(dev["q_v"]),
+                     ptr(dev["s_v"]), 0)
+    q = orc.normal_activations(nseq * Hkv * group * D, 0xFEED)
+    q_d, bt_d = to_dev(q), to_dev(tables.ravel())
+    out = halves(nseq * Hkv * group * D, 0x7E00)
+    c.attention_w4_flash_paged_batched(view, ptr(bt_d), nseq, lp, page, npages, group, ptr(q_d), ptr(out))
+    got = bits(out).reshape(nseq, Hkv * group * D)
+    qs = q.reshape(nseq, Hkv * group * D)
+    for s, c4 in enumerate(caches):
+        ref = orc.attention_reference(qs[s], c4, heads_per_slab=group)
+        assert orc.rel_l2(got[s].view(np.float16), ref) <= TOL
+        dk = DevKV(c4)
+        o = halves(Hkv * group * D, 0x7E00)
+        c.attention_w4_flash(dk.view, ptr(to_dev(qs[s])), ptr(o), group=group)
+        assert np.array_equal(bits(o), got[s]), "paged batch == contiguous, bytewise"

@@ -10,8 +10,9 @@ import sys
 PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG, "csrc")
 LIB = os.path.join(PKG, "lib", "libw4amd.so")
+BENCH_LIB = os.path.join(PKG, "lib", "libw4bench.so")
 SOURCES = ["abi.hip", "dequant.hip", "gemm_simt.hip", "gemm_mfma.hip", "flash.hip", "baseline.hip"]
-HEADERS = ["dq.cuh", "kernels.h", os.path.join("..", "..", "include", "w4_abi.h")]
+HEADERS = ["dq.cuh", "kernels.h", "bench_kernels.hip", os.path.join("..", "..", "include", "w4_abi.h")]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed-FP32 VALU forms stay off for every kernel in this library
@@ -48,6 +49,10 @@ def build(force=False, verbose=True):
             print(err, file=sys.stderr)
     subprocess.check_call(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs,
                            "-lhipblaslt"])
+    # bandwidth yardsticks used only by bench.py
+    subprocess.check_call(["hipcc", *[f for f in FLAGS if not f.startswith("-W")], "-shared",
+                           os.path.join(CSRC, "bench_kernels.hip"), "-o", BENCH_LIB],
+                          stderr=subprocess.DEVNULL)
     return LIB
 
 

@@ -21,9 +21,7 @@ __global__ __launch_bounds__(256) void dequant_words(WView p, w4_half* __restric
   const uint32_t qw = p.q[idx];
   h2 d[4], nat[4];
   if (MX) {
-    const uint32_t se = ((const uint8_t*)p.scales)[(size_t)n * p.B + (k0 >> 5)];
-    const MxBlock mb = mx_block(se);
-    dq_mx(qw, mb, __builtin_amdgcn_ballot_w64(mb.wide) != 0, d);
+    dq_mx(qw, mx_scale(((const uint8_t*)p.scales)[(size_t)n * p.B + (k0 >> 5)]), nat);
   } else {
     const int g = k0 / p.gs;
     const uint16_t sb = ((const uint16_t*)p.scales)[(size_t)n * p.G + g];
@@ -31,8 +29,8 @@ __global__ __launch_bounds__(256) void dequant_words(WView p, w4_half* __restric
                       ? 8
                       : (int)((p.zeros[(size_t)n * words(p.G) + (g >> 3)] >> (4 * (g & 7))) & 0xF);
     dq_w4(qw, w4_group(sb, z), d);
+    to_natural(d, nat);
   }
-  to_natural(d, nat);
   uint16_t* out = w + (size_t)n * p.K + k0;
   if (VEC) {
     *(u4*)out = u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};

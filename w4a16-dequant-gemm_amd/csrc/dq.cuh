@@ -8,9 +8,10 @@
 //   * the scale has an 11-bit significand and the value at most 4 significant
 //     bits, so the exact product fits FP32 and v_pk_mul_f16 performs the same
 //     single round-to-nearest-even (FP16 denormals are enabled on gfx950).
-// The pairs come out "strided": register i holds elements (i, i+4) of the
-// word, which is what two mask-and-or instructions per pair give for free.
-// to_natural() re-pairs them as (0,1),(2,3),(4,5),(6,7) with v_perm_b32.
+// W4 and FP8 pairs come out "strided": register i holds elements (i, i+4) of
+// the word (FP8: (i, i+2) of 4 bytes), which is what one mask-and-or per pair
+// gives for free.  to_natural() re-pairs them as (0,1),(2,3),(4,5),(6,7) with
+// v_perm_b32.  MXFP4 uses the gfx950 FP4 convert and comes out in natural order.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -48,14 +49,24 @@ __device__ __forceinline__ W4Group w4_group(uint16_t scale_bits, int z) {
   return g;
 }
 
+// (a & mask) | orv in one VOP3 instruction (the compiler otherwise emits an
+// AND and an OR with literal operands).
+__device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t orv) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(orv));
+  return r;
+}
+
 // d[i] = (w[i], w[i+4]) dequantized, i = 0..3.
 __device__ __forceinline__ void dq_w4(uint32_t w, const W4Group& g, h2 d[4]) {
   const uint32_t w8 = w >> 8;
+  uint32_t magic = 0x64006400u;
+  asm("" : "+v"(magic));  // keep the constant in a VGPR for the VOP3 form
   // 0x6400 | n reads as 1024 + n; 0x6400 | (n << 4) as 1024 + 16 n.
-  const h2 a0 = as_h2((w & 0x000F000Fu) | 0x64006400u);
-  const h2 a1 = as_h2((w & 0x00F000F0u) | 0x64006400u);
-  const h2 a2 = as_h2((w8 & 0x000F000Fu) | 0x64006400u);
-  const h2 a3 = as_h2((w8 & 0x00F000F0u) | 0x64006400u);
+  const h2 a0 = as_h2(and_or(w, 0x000F000Fu, magic));
+  const h2 a1 = as_h2(and_or(w, 0x00F000F0u, magic));
+  const h2 a2 = as_h2(and_or(w8, 0x000F000Fu, magic));
+  const h2 a3 = as_h2(and_or(w8, 0x00F000F0u, magic));
   const h2 sixteenth = splat((_Float16)0.0625f);
   d[0] = (a0 - g.zlo) * g.s;                 // (1024 + n) - (1024 + z): exact
   d[1] = (a1 * sixteenth - g.zhi) * g.s;     // (64 + n) - (64 + z): exact
@@ -64,49 +75,22 @@ __device__ __forceinline__ void dq_w4(uint32_t w, const W4Group& g, h2 d[4]) {
 }
 
 // ---- MXFP4: E2M1 codes with an E8M0 block scale ----------------------------
-// A code's magnitude bits i (3 bits) placed at half bits 9..11 read as
-// e2m1(i) * 2^-14 (the subnormal encoding covers i = 0, 1), so the element is
-// bits * 2^(se - 113).  The power of two is applied as up to three FP16
-// multiplies; only the last one that is not 1.0 can round.
-struct MxBlock {
-  h2 a, b, c;
-  bool wide;  // b or c differ from 1.0 (block scale above 2^-98 * 2^113...)
-};
-
-__device__ __forceinline__ uint32_t pow2_half_bits(int t) {
-  // 2^t for t in [-24, 15] as FP16 bits (subnormal below -14)
-  return t >= -14 ? (uint32_t)(t + 15) << 10 : 1u << (t + 24);
+// gfx950 converts two E2M1 codes of one byte, times 2^(exponent of the scale
+// operand), to packed FP16 in one instruction.  With the E8M0 byte placed in
+// the exponent field of the float operand the result is bit-identical to
+// RNE_half(2^(se-127) * e2m1(code)) for every scale byte 0..254 and every code
+// (checked exhaustively by the GPU test suite), including results that land in
+// the FP16 subnormal range or overflow to infinity.
+// n[j] = (w[2j], w[2j+1]): the pairs come out in natural order.
+__device__ __forceinline__ float mx_scale(uint32_t se) {
+  return __builtin_bit_cast(float, se << 23);
 }
 
-__device__ __forceinline__ MxBlock mx_block(uint32_t se) {
-  const int t = (int)se - 113;
-  MxBlock m;
-  const int ta = t < -24 ? -24 : (t > 15 ? 15 : t);
-  m.a = splat_bits(pow2_half_bits(ta));
-  const int tb = t - 15 < 0 ? 0 : (t - 15 > 15 ? 15 : t - 15);
-  const int tc = t - 30 < 0 ? 0 : (t - 30 > 15 ? 15 : t - 30);
-  m.b = splat_bits(pow2_half_bits(tb));
-  m.c = splat_bits(pow2_half_bits(tc));
-  m.wide = t > 15;
-  return m;
-}
-
-// d[i] = (w[i], w[i+4]) dequantized.  `any_wide` is wave-uniform.
-__device__ __forceinline__ void dq_mx(uint32_t w, const MxBlock& m, bool any_wide,
-                                      h2 d[4]) {
-  const uint32_t mag = 0x0E000E00u, sgn = 0x80008000u;
-  h2 v0 = as_h2(((w << 9) & mag) | ((w << 12) & sgn));
-  h2 v1 = as_h2(((w << 5) & mag) | ((w << 8) & sgn));
-  h2 v2 = as_h2(((w << 1) & mag) | ((w << 4) & sgn));
-  h2 v3 = as_h2(((w >> 3) & mag) | (w & sgn));
-  d[0] = v0 * m.a;
-  d[1] = v1 * m.a;
-  d[2] = v2 * m.a;
-  d[3] = v3 * m.a;
-  if (any_wide) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) d[i] = (d[i] * m.b) * m.c;
-  }
+__device__ __forceinline__ void dq_mx(uint32_t w, float scale, h2 n[4]) {
+  n[0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 0);
+  n[1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 1);
+  n[2] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 2);
+  n[3] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, scale, 3);
 }
 
 // ---- FP8 E4M3 bytes ----------------------------------------------------------
@@ -152,10 +136,21 @@ __device__ __forceinline__ float dot2(h2 a, h2 b, float acc) {
   return __builtin_amdgcn_fdot2(a, b, acc, false);
 }
 
-// Wave64 sum of `v`: every lane ends with the total.
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+// Wave64 sum of `v` with DPP adds only (no LDS traffic): quad swaps, row
+// mirrors, then the two row broadcasts.  Lane 63 ends with the total.
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ float dpp_add(float v) {
+  const int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROWMASK, 0xF, true);
+  return v + __builtin_bit_cast(float, t);
+}
+
+__device__ __forceinline__ float wave_sum_to_lane63(float v) {
+  v = dpp_add<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+  v = dpp_add<0x141, 0xF>(v);  // row_half_mirror
+  v = dpp_add<0x140, 0xF>(v);  // row_mirror: every lane of a row holds the row sum
+  v = dpp_add<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
+  v = dpp_add<0x143, 0xC>(v);  // row_bcast31 into rows 2 and 3
   return v;
 }
 

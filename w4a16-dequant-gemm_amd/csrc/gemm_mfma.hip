@@ -77,27 +77,22 @@ __global__ __launch_bounds__(MMA_WAVES * 64) void mfma_skinny_kernel(
       for (int j = 0; j < 4; ++j)
         if (w0 + j < wpr) qw[j] = p.q[(size_t)n * wpr + w0 + j];
     }
-    MxBlock mb;
-    bool any_wide = false;
-    if (MX) {
-      const int blk = min(w0 >> 2, p.B - 1);
-      mb = mx_block(((const uint8_t*)p.scales)[(size_t)n * p.B + blk]);
-      any_wide = __builtin_amdgcn_ballot_w64(mb.wide) != 0;
-    }
+    float mxs = 0.0f;
+    if (MX) mxs = mx_scale(((const uint8_t*)p.scales)[(size_t)n * p.B + min(w0 >> 2, p.B - 1)]);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int k0 = (w0 + j) * 8;
       h2 d[4], nat[4];
       if (MX) {
-        dq_mx(qw[j], mb, any_wide, d);
+        dq_mx(qw[j], mxs, nat);
       } else {
         const int g = min(k0 / p.gs, p.G - 1);
         const int z = p.symmetric ? 8
                                   : (int)((p.zeros[(size_t)n * wg + (g >> 3)] >>
                                            (4 * (g & 7))) & 0xF);
         dq_w4(qw[j], w4_group(((const uint16_t*)p.scales)[(size_t)n * p.G + g], z), d);
+        to_natural(d, nat);
       }
-      to_natural(d, nat);
       if (hook && k0 < p.K) {
         uint16_t* out = w_out + (size_t)n * p.K + k0;
         if (FAST) {

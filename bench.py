@@ -63,6 +63,31 @@ class Bench:
         self.yard = C.CDLL(os.path.join(ROOT, "w4a16-dequant-gemm_amd", "lib", "libw4bench.so"))
         self.yard.w4bench_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_void_p]
         self.yard.w4bench_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p]
+        self.yard.w4bench_gemm_loop.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p,
+                                                C.c_int, C.c_int, C.c_void_p]
+
+    def loop_ms(self, entry, views, x_ptr, c_ptr, M, steps, warmup, reps=5):
+        """Mean ms per call over `steps` launches issued by a C loop (no
+        interpreter between launches), HIP events on the launch stream; median of reps."""
+        torch = self.torch
+        fn = C.cast(getattr(self.capi.load(), entry), C.c_void_p)
+        arr = (C.c_void_p * len(views))(*[C.addressof(v) for v in views])
+
+        def run(n):
+            rc = self.yard.w4bench_gemm_loop(fn, arr, len(views), x_ptr, c_ptr, M, n, self.stream)
+            if rc:
+                raise RuntimeError("gemm loop failed: %d" % rc)
+        run(warmup)
+        torch.cuda.synchronize()
+        out = []
+        for _ in range(reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            run(steps)
+            b.record()
+            torch.cuda.synchronize()
+            out.append(a.elapsed_time(b) / steps)
+        return sorted(out)[len(out) // 2]
 
     # -- yardsticks ---------------------------------------------------------
     def bandwidth(self):
@@ -108,9 +133,7 @@ class Bench:
         torch = self.torch
         x = torch.randn(M * K, device="cuda").to(torch.float16)
         c = torch.empty(M * N, dtype=torch.float16, device="cuda")
-        n = len(views)
-        ms = _median_events_ms(torch, lambda i: fn(views[i % n][0], x.data_ptr(), c.data_ptr(), M,
-                                                   self.stream, 0), self.steps, self.warmup)
+        ms = self.loop_ms(fn, [v[0] for v in views], x.data_ptr(), c.data_ptr(), M, self.steps, self.warmup)
         return ms * 1e3
 
 
@@ -167,14 +190,14 @@ def headline(b, args):
     for _ in range(copies - 1):
         d2 = DevPacked(p)
         views.append((d2.view, d2))
-    x16 = x_d
-    fn = lambda i: capi.gemm(views[i % copies][0], ptr(x16), ptr(c_d), M, b.stream, 0)
-    cold_ms = _events_ms(torch, fn, args.steps, args.warmup)
-    fn1 = lambda i: capi.gemm(views[0][0], ptr(x16), ptr(c_d), M, b.stream, 0)
-    warm_ms = _median_events_ms(torch, fn1, args.steps, args.warmup)
+    vlist = [v[0] for v in views]
+    # the K timed steps: one C launch loop bracketed by HIP events
+    cold_ms = b.loop_ms("w4_gemm", vlist, ptr(x_d), ptr(c_d), M, args.steps, args.warmup, reps=1)
+    cold_med_ms = b.loop_ms("w4_gemm", vlist, ptr(x_d), ptr(c_d), M, args.steps, 2)
+    warm_ms = b.loop_ms("w4_gemm", vlist[:1], ptr(x_d), ptr(c_d), M, args.steps, args.warmup)
     return {
         "N": N, "K": K, "gs": gs, "M": M, "bytes": nbytes, "copies": copies,
-        "cold_ms": cold_ms, "warm_ms": warm_ms, "hook_bitwise": hook_ok, "rel_l2_vs_oracle": rel,
+        "cold_ms": cold_ms, "cold_median5_ms": cold_med_ms, "warm_ms": warm_ms, "hook_bitwise": hook_ok, "rel_l2_vs_oracle": rel,
         "cpu": {"quantize_s": t_quant, "dequant_all_s": t_deq, "gemm_oracle_s": t_gemm,
                 "fused_equiv_s": cpu_s},
     }
@@ -192,8 +215,8 @@ def extras_gemm(b, full):
         views = b.rand_w4(N, K, gs, False, copies)
         for M in (1, 2, 4, 8, 9, 16, 64):
             nb = w4_bytes(N, K, gs, False, M)
-            us_s = b.gemm_us(capi.gemm_fused, views, M, N, K)
-            us_m = b.gemm_us(capi.gemm_mma, views, M, N, K)
+            us_s = b.gemm_us("w4_gemm_fused", views, M, N, K)
+            us_m = b.gemm_us("w4_gemm_mma", views, M, N, K)
             rows.append({"N": N, "K": K, "gs": gs, "M": M, "bytes": nb, "simt_us": us_s, "mfma_us": us_m,
                          "simt_GBs": nb / us_s * 1e-3, "mfma_GBs": nb / us_m * 1e-3,
                          "winner": "simt" if us_s <= us_m else "mfma"})
@@ -206,8 +229,8 @@ def extras_gemm(b, full):
     views = b.rand_mx(N, K, max(2, int(400e6 // mx_bytes(N, K, 1)) + 1))
     for M in (1, 16, 128):
         nb = mx_bytes(N, K, M)
-        us_s = b.gemm_us(capi.gemm_fused_mx, views, M, N, K) if M <= 16 else None
-        us_m = b.gemm_us(capi.gemm_mma_mx, views, M, N, K)
+        us_s = b.gemm_us("w4_gemm_fused_mx", views, M, N, K) if M <= 16 else None
+        us_m = b.gemm_us("w4_gemm_mma_mx", views, M, N, K)
         rows.append({"N": N, "K": K, "M": M, "bytes": nb, "simt_us": us_s, "mfma_us": us_m,
                      "best_GBs": nb / min(u for u in (us_s, us_m) if u) * 1e-3,
                      "mfma_TFLOPs": 2.0 * M * N * K / us_m * 1e-6})

@@ -1,0 +1,255 @@
+#pragma once
+
+// w4::gpu -- the device entry points of the fused-dequant path, as thin C++
+// wrappers over the C ABI of libw4amd.so (include/w4_abi.h).  Signatures follow
+// the reference's launch wrappers (dequant.cuh, fused.cuh, mma.cuh,
+// mxfused.cuh, dispatch.cuh, kvattention.cuh, kvflash.cuh; cited per function)
+// with hipStream_t in place of cudaStream_t.  Contract violations throw
+// std::invalid_argument before anything touches the device; HIP failures throw
+// std::runtime_error.  All pointers are device pointers owned by the caller;
+// launches are asynchronous on `stream`.
+//
+// Link with -lw4amd.
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+#include "../w4_abi.h"
+#include "kvcache.hpp"
+#include "kvfp8.hpp"
+#include "kvpaged.hpp"
+#include "mx.hpp"
+#include "pack.hpp"
+
+namespace w4::gpu {
+
+// dequant.cuh:19-23
+inline void hip_check(hipError_t e, const char* what) {
+  if (e != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+// dequant.cuh:31-37 (field order and types are the ABI's)
+struct DevicePackedW {
+  int N, K, gs, G;
+  int symmetric;
+  const uint32_t* q;
+  const __half* scales;
+  const uint32_t* zeros;
+};
+
+// mxfused.cuh:26-30
+struct DevicePackedWm {
+  int N, K, B;
+  const uint32_t* q;
+  const uint8_t* scales;
+};
+
+// kvattention.cuh:39-48
+struct DeviceKVW4 {
+  int H, S, D, gs, G;
+  int symmetric;
+  const uint32_t* q_k;
+  const __half* s_k;
+  const uint32_t* z_k;
+  const uint32_t* q_v;
+  const __half* s_v;
+  const uint32_t* z_v;
+};
+
+// kvflash.cuh:390-396
+struct DeviceKVF8 {
+  int H, S, D, gs, G;
+  const uint8_t* q_k;
+  const __half* s_k;
+  const uint8_t* q_v;
+  const __half* s_v;
+};
+
+constexpr int KV_MAX_D = 512;    // kvattention.cuh:37
+constexpr int FLASH_TILE = 256;  // kvflash.cuh:35
+
+namespace detail {
+
+inline void raise(int rc) {
+  if (rc == W4_OK) return;
+  const std::string msg = w4_last_error();
+  if (rc == W4_EINVAL) throw std::invalid_argument(msg);
+  throw std::runtime_error(msg);
+}
+
+inline const w4_half* h(const __half* p) { return reinterpret_cast<const w4_half*>(p); }
+inline w4_half* h(__half* p) { return reinterpret_cast<w4_half*>(p); }
+
+inline w4_packed_view abi(const DevicePackedW& p) {
+  return w4_packed_view{p.N, p.K, p.gs, p.G, p.symmetric, p.q, h(p.scales), p.zeros};
+}
+inline w4_packed_mx_view abi(const DevicePackedWm& p) {
+  return w4_packed_mx_view{p.N, p.K, p.B, p.q, p.scales};
+}
+inline w4_kv_view abi(const DeviceKVW4& p) {
+  return w4_kv_view{p.H, p.S, p.D, p.gs, p.G, p.symmetric, p.q_k, h(p.s_k), p.z_k,
+                    p.q_v, h(p.s_v), p.z_v};
+}
+inline w4_kv_f8_view abi(const DeviceKVF8& p) {
+  return w4_kv_f8_view{p.H, p.S, p.D, p.gs, p.G, p.q_k, h(p.s_k), p.q_v, h(p.s_v)};
+}
+
+}  // namespace detail
+
+// dispatch.cuh:25 -- the activation-row count from which gemm()/gemm_mx() use
+// the matrix-core kernel, as measured on MI355X.
+inline int dispatch_mma_min_m() { return w4_dispatch_mma_min_m(); }
+
+// dequant.cuh:62-82
+inline void dequant(const DevicePackedW& p, __half* w, hipStream_t stream = 0) {
+  const auto v = detail::abi(p);
+  detail::raise(w4_dequant(&v, detail::h(w), stream));
+}
+
+// fused.cuh:172-214
+inline void gemm_fused(const DevicePackedW& p, const __half* x, __half* c, int M,
+                       hipStream_t stream = 0, __half* w_out = nullptr) {
+  const auto v = detail::abi(p);
+  detail::raise(w4_gemm_fused(&v, detail::h(x), detail::h(c), M, stream, detail::h(w_out)));
+}
+
+// mma.cuh:234-260
+inline void gemm_mma(const DevicePackedW& p, const __half* x, __half* c, int M,
+                     hipStream_t stream = 0, __half* w_out = nullptr) {
+  const auto v = detail::abi(p);
+  detail::raise(w4_gemm_mma(&v, detail::h(x), detail::h(c), M, stream, detail::h(w_out)));
+}
+
+// dispatch.cuh:27-34
+inline void gemm(const DevicePackedW& p, const __half* x, __half* c, int M,
+                 hipStream_t stream = 0, __half* w_out = nullptr) {
+  const auto v = detail::abi(p);
+  detail::raise(w4_gemm(&v, detail::h(x), detail::h(c), M, stream, detail::h(w_out)));
+}
+
+// mxfused.cuh:32-37
+inline void validate_mx(const DevicePackedWm& p) {
+  w4::detail::require(p.N >= 1 && p.K >= 1, "mx: bad dims");
+  w4::detail::require(p.B == mx::blocks(p.K), "mx: B inconsistent with K");
+  w4::detail::require(p.q && p.scales, "mx: null pointer");
+}
+
+// mxfused.cuh:57-69
+inline void dequant_mx(const DevicePackedWm& p, __half* w, hipStream_t stream = 0) {
+  const auto v = detail::abi(p);
+  detail::raise(w4_dequant_mx(&v, detail::h(w), stream));
+}
+
+// mxfused.cuh:166-198
+inline void gemm_fused_mx(const DevicePackedWm& p, const __half* x, __half* c, int M,
+                          hipStream_t stream = 0, __half* w_out = nullptr) {
+  const auto v = detail::abi(p);
+  detail::raise(w4_gemm_fused_mx(&v, detail::h(x), detail::h(c), M, stream, detail::h(w_out)));
+}
+
+// mxfused.cuh:291-307
+inline void gemm_mma_mx(const DevicePackedWm& p, const __half* x, __half* c, int M,
+                        hipStream_t stream = 0, __half* w_out = nullptr) {
+  const auto v = detail::abi(p);
+  detail::raise(w4_gemm_mma_mx(&v, detail::h(x), detail::h(c), M, stream, detail::h(w_out)));
+}
+
+// dispatch.cuh:36-43
+inline void gemm_mx(const DevicePackedWm& p, const __half* x, __half* c, int M,
+                    hipStream_t stream = 0, __half* w_out = nullptr) {
+  const auto v = detail::abi(p);
+  detail::raise(w4_gemm_mx(&v, detail::h(x), detail::h(c), M, stream, detail::h(w_out)));
+}
+
+// dequant.cuh:87-106.  The reference passes a cuBLAS handle; the hipBLASLt
+// handle lives inside the library, so the handle type here is an empty tag.
+struct BlasHandle {};
+inline BlasHandle make_blas() { return BlasHandle{}; }
+inline void gemm_fp16(BlasHandle, const __half* w, const __half* x, __half* c, int M, int N,
+                      int K, hipStream_t stream = 0) {
+  detail::raise(w4_gemm_fp16(detail::h(w), detail::h(x), detail::h(c), M, N, K, stream));
+}
+
+// kvflash.cuh:350-363
+inline void attention_w4_flash(const DeviceKVW4& p, const __half* q, __half* out,
+                               hipStream_t stream = 0, __half* k_out = nullptr,
+                               __half* v_out = nullptr) {
+  const auto v = detail::abi(p);
+  detail::raise(w4_attention_w4_flash(&v, detail::h(q), detail::h(out), stream,
+                                      detail::h(k_out), detail::h(v_out)));
+}
+
+// kvflash.cuh:365-384
+inline void attention_fp16_flash(const __half* q, const __half* k16, const __half* v16,
+                                 __half* out, int H, int S, int D, hipStream_t stream = 0) {
+  detail::raise(w4_attention_fp16_flash(detail::h(q), detail::h(k16), detail::h(v16),
+                                        detail::h(out), H, S, D, stream));
+}
+
+// kvflash.cuh:572-590
+inline void attention_f8_flash(const DeviceKVF8& p, const __half* q, __half* out,
+                               hipStream_t stream = 0, __half* k_out = nullptr,
+                               __half* v_out = nullptr) {
+  const auto v = detail::abi(p);
+  detail::raise(w4_attention_f8_flash(&v, detail::h(q), detail::h(out), stream,
+                                      detail::h(k_out), detail::h(v_out)));
+}
+
+// kvflash.cuh:725-764
+inline void attention_w4_flash_paged(const DeviceKVW4& p, const int* bt, int page, int npages,
+                                     const __half* q, __half* out, hipStream_t stream = 0,
+                                     __half* k_out = nullptr, __half* v_out = nullptr) {
+  const auto v = detail::abi(p);
+  detail::raise(w4_attention_w4_flash_paged(&v, bt, page, npages, detail::h(q), detail::h(out),
+                                            stream, detail::h(k_out), detail::h(v_out)));
+}
+
+// kvflash.cuh:435-457
+inline void dequant_f8(const uint8_t* q, const __half* s, __half* w, int S, int D, int gs,
+                       hipStream_t stream = 0) {
+  detail::raise(w4_dequant_f8(q, detail::h(s), detail::h(w), S, D, gs, stream));
+}
+
+// ---- batched / grouped-query forms (additive; no reference counterpart) ------
+// The views hold nseq * Hkv slabs; `group` query heads share each slab; q and
+// out hold (slabs * group) * D halves, slab-major.
+inline void attention_w4_flash_gqa(const DeviceKVW4& p, int group, const __half* q, __half* out,
+                                   hipStream_t stream = 0, __half* k_out = nullptr,
+                                   __half* v_out = nullptr) {
+  const auto v = detail::abi(p);
+  detail::raise(w4_attention_w4_flash_gqa(&v, group, detail::h(q), detail::h(out), stream,
+                                          detail::h(k_out), detail::h(v_out)));
+}
+
+inline void attention_fp16_flash_gqa(const __half* q, const __half* k16, const __half* v16,
+                                     __half* out, int H, int group, int S, int D,
+                                     hipStream_t stream = 0) {
+  detail::raise(w4_attention_fp16_flash_gqa(detail::h(q), detail::h(k16), detail::h(v16),
+                                            detail::h(out), H, group, S, D, stream));
+}
+
+// scale_mode 0: scales per (row, group) as in the reference; 1: one per slab.
+inline void attention_f8_flash_gqa(const DeviceKVF8& p, int group, int scale_mode,
+                                   const __half* q, __half* out, hipStream_t stream = 0,
+                                   __half* k_out = nullptr, __half* v_out = nullptr) {
+  const auto v = detail::abi(p);
+  detail::raise(w4_attention_f8_flash_gqa(&v, group, scale_mode, detail::h(q), detail::h(out),
+                                          stream, detail::h(k_out), detail::h(v_out)));
+}
+
+// One pool (p.H = Hkv slabs of npages*page rows) shared by nseq sequences, each
+// with its own table of bt_stride entries.
+inline void attention_w4_flash_paged_batched(const DeviceKVW4& p, const int* bt, int nseq,
+                                             int bt_stride, int page, int npages, int group,
+                                             const __half* q, __half* out,
+                                             hipStream_t stream = 0) {
+  const auto v = detail::abi(p);
+  detail::raise(w4_attention_w4_flash_paged_batched(&v, bt, nseq, bt_stride, page, npages, group,
+                                                    detail::h(q), detail::h(out), stream));
+}
+
+}  // namespace w4::gpu

@@ -40,3 +40,17 @@ extern "C" int w4bench_copy(const void* src, void* dst, size_t bytes, int blocks
   stream_copy<<<blocks, 256, 0, (hipStream_t)stream>>>((const u4*)src, (u4*)dst, bytes / 16);
   return (int)hipGetLastError();
 }
+
+// Host-side launch loop: `steps` back-to-back calls of one GEMM entry point,
+// rotating through `nviews` weight views, without returning to the caller's
+// interpreter between launches.
+typedef int (*w4bench_gemm_fn)(const void* view, const void* x, void* c, int M, void* stream,
+                               void* w_out);
+extern "C" int w4bench_gemm_loop(w4bench_gemm_fn fn, const void* const* views, int nviews,
+                                 const void* x, void* c, int M, int steps, void* stream) {
+  for (int i = 0; i < steps; ++i) {
+    const int rc = fn(views[i % nviews], x, c, M, stream, nullptr);
+    if (rc) return rc;
+  }
+  return 0;
+}

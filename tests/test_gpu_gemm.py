@@ -20,7 +20,9 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         (2, 32, 128, 64), (3, 40, 256, 128), (5, 72, 40, 8), (17, 64, 128, 16),
         (33, 48, 104, 24), (20, 32, 100, 8), (65, 96, 100, 16),
         # shapes that take the aligned dwordx4 paths
-        (1, 512, 4096, 128), (7, 96, 2048, 32), (9, 80, 1024, 64), (64, 64, 512, 128)]
+        (1, 512, 4096, 128), (7, 96, 2048, 32), (9, 80, 1024, 64), (64, 64, 512, 128),
+        # shapes of the unrolled decode kernel (K = 2048, 4096, 8192; whole workgroups of rows)
+        (2, 64, 2048, 64), (1, 128, 8192, 128), (4, 72, 4096, 32), (3, 40, 6144, 128), (8, 16, 2048, 128)]
 TOL, CROSS = 1e-3, 2e-3  # rel L2 vs the FP64 oracle; between two gated paths
 
 

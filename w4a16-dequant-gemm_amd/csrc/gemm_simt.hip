@@ -7,9 +7,11 @@
 // the MT activation rows from LDS.  Products are v_dot2_f32_f16 into FP32
 // accumulators; the K reduction is finished with DPP adds.
 //
-// The loads of block b+1 (codes, scales, zero-points) are issued before block
-// b is expanded, and block 0 is requested before the activations are staged,
-// so HBM latency overlaps both the staging barrier and the ALU work.
+// Memory returns loads in issue order, so the order of requests is part of the
+// design: the activations first (the staging barrier then waits for nothing
+// else), block 0 of the weights right behind them (in flight across the
+// barrier), and block b+1 (codes, scales, zero-points) before block b is
+// expanded, so HBM latency overlaps the barrier and the ALU work.
 //
 // Activations are staged in LDS once per workgroup, paired to match what the
 // dequant step produces ((k, k+4) for W4, natural for MXFP4), and laid out so
@@ -122,7 +124,6 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_fast_kernel(
     for (int m = 0; m < MT; ++m) acc[r][m] = 0.0f;
 
   LaneBlock<MX, R, GS32> cur, nxt;
-  if (wave_on) load_block(cur, p, n0, wpr, wg, lane * 4);  // in flight during staging
 
   const int nblk = (wpr + 255) / 256;
   for (int kc = 0, blk0 = 0; kc < p.K; kc += KC, blk0 += KC / 2048) {
@@ -130,7 +131,26 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_fast_kernel(
     const int groups = kc_len >> 3;  // K % 32 == 0 here
     const int slots = (groups + 255) & ~255;
     if (kc) __syncthreads();
-    stage_x<MX, MT, true>(xs, x, M, p.K, m0, kc, groups, slots, x_vec);
+    // Loads return in issue order: the activations are requested first so the
+    // staging barrier only waits for them, and the first weight block is
+    // requested right behind them so it is in flight across the barrier.
+    constexpr int XL = (KC / 8 * MT + SIMT_WAVES * 64 - 1) / (SIMT_WAVES * 64);
+    u4 xv[XL];
+#pragma unroll
+    for (int t = 0; t < XL; ++t) {
+      const int i = t * SIMT_WAVES * 64 + threadIdx.x;
+      const int m = i / slots, g8 = i - m * slots;
+      xv[t] = u4{0u, 0u, 0u, 0u};
+      if (i < slots * MT && g8 < groups) xv[t] = load_x8_guarded(x, M, p.K, m0 + m, kc + g8 * 8, x_vec);
+    }
+    if (kc == 0 && wave_on) load_block(cur, p, n0, wpr, wg, lane * 4);
+#pragma unroll
+    for (int t = 0; t < XL; ++t) {
+      const int i = t * SIMT_WAVES * 64 + threadIdx.x;
+      const int m = i / slots, g8 = i - m * slots;
+      const int slot = (g8 & ~255) + (g8 & 3) * 64 + ((g8 & 255) >> 2);
+      if (i < slots * MT) xs[m * slots + slot] = MX ? xv[t] : pair_strided(xv[t]);
+    }
     __syncthreads();
     if (!wave_on) continue;
 
@@ -184,14 +204,24 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_fast_kernel(
 #pragma unroll
     for (int m = 0; m < MT; ++m) acc[r][m] = wave_sum_to_lane63(acc[r][m]);
   if (lane == 63) {
+    const bool pair_ok = R == 2 && (p.N & 1) == 0 && (((uintptr_t)c & 3) == 0) && n0 + 1 < p.N;
 #pragma unroll
-    for (int r = 0; r < R; ++r)
+    for (int m = 0; m < MT; ++m) {
+      if (m0 + m >= M) continue;
+      uint16_t* dst = c + (size_t)(m0 + m) * p.N + n0;
+      if (pair_ok) {  // the wave's two rows leave as one 4-byte store
+        const _Float16 h0 = (_Float16)acc[0][m], h1 = (_Float16)acc[R - 1][m];
+        *(uint32_t*)dst = (uint32_t)__builtin_bit_cast(uint16_t, h0) |
+                          ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
+      } else {
 #pragma unroll
-      for (int m = 0; m < MT; ++m)
-        if (n0 + r < p.N && m0 + m < M) {
-          const _Float16 h = (_Float16)acc[r][m];
-          c[(size_t)(m0 + m) * p.N + n0 + r] = __builtin_bit_cast(uint16_t, h);
-        }
+        for (int r = 0; r < R; ++r)
+          if (n0 + r < p.N) {
+            const _Float16 h = (_Float16)acc[r][m];
+            dst[r] = __builtin_bit_cast(uint16_t, h);
+          }
+      }
+    }
   }
 }
 
@@ -281,10 +311,143 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_generic_kernel(
   }
 }
 
+// Fully unrolled form of the fast kernel for the shapes decode GEMMs have:
+// K = STEPS * 2048, one group per 32-k lane slice, whole workgroups of rows, no
+// hook.  Every load of a wave (activations first, then the STEPS * R weight
+// dwordx4 and their scales) is issued before anything is consumed, and the
+// waits are retired in that order.
+template <int MX, int MT, int R, int STEPS>
+__global__ __launch_bounds__(SIMT_WAVES * 64) void simt_unrolled_kernel(
+    const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M) {
+  __shared__ u4 xs[MT * STEPS * 256];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n0 = (blockIdx.x * SIMT_WAVES + wave) * R;
+  const int m0 = blockIdx.y * MT;
+  constexpr int K = STEPS * 2048, WPR = K / 8;
+  constexpr int XL = (MT * STEPS * 256) / (SIMT_WAVES * 64);
+  const int wg = MX ? 0 : words(p.G);
+
+  u4 xv[XL];
+#pragma unroll
+  for (int t = 0; t < XL; ++t) {
+    const int i = t * SIMT_WAVES * 64 + threadIdx.x;
+    const int m = i / (STEPS * 256), g8 = i % (STEPS * 256);
+    xv[t] = (m0 + m < M) ? *(const u4*)(x + (size_t)(m0 + m) * K + g8 * 8) : u4{0u, 0u, 0u, 0u};
+  }
+  uint32_t sc[STEPS][R], zp[STEPS][R];
+  u4 qw[STEPS][R];
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int n = n0 + r, k0 = s * 2048 + lane * 32;
+      if (MX) {
+        sc[s][r] = ((const uint8_t*)p.scales)[(size_t)n * p.B + (k0 >> 5)];
+        zp[s][r] = 0;
+      } else {
+        const int g = k0 / p.gs;
+        sc[s][r] = ((const uint16_t*)p.scales)[(size_t)n * p.G + g];
+        zp[s][r] = (uint32_t)zero_point(p, n, g, wg);
+      }
+    }
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      qw[s][r] = __builtin_nontemporal_load(
+          (const u4*)(p.q + (size_t)(n0 + r) * WPR + s * 256 + lane * 4));
+#pragma unroll
+  for (int t = 0; t < XL; ++t) {
+    const int i = t * SIMT_WAVES * 64 + threadIdx.x;
+    const int m = i / (STEPS * 256), g8 = i % (STEPS * 256);
+    const int slot = (g8 & ~255) + (g8 & 3) * 64 + ((g8 & 255) >> 2);
+    xs[m * STEPS * 256 + slot] = MX ? xv[t] : pair_strided(xv[t]);
+  }
+  __syncthreads();
+
+  float acc[R][MT];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[r][m] = 0.0f;
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    u4 xr[MT][4];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) xr[m][j] = xs[m * STEPS * 256 + s * 256 + j * 64 + lane];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const W4Group grp = w4_group((uint16_t)sc[s][r], (int)zp[s][r]);
+      const float mxs = mx_scale(sc[s][r]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        h2 d[4];
+        if (MX) dq_mx(qw[s][r][j], mxs, d);
+        else dq_w4(qw[s][r][j], grp, d);
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[r][m] = dot2(d[e], as_h2(xr[m][j][e]), acc[r][m]);
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[r][m] = wave_sum_to_lane63(acc[r][m]);
+  if (lane == 63) {
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      if (m0 + m >= M) continue;
+      uint16_t* dst = c + (size_t)(m0 + m) * p.N + n0;
+      if (R == 2) {  // N is a multiple of 8 here, so the pair is 4-byte aligned with c
+        const _Float16 h0 = (_Float16)acc[0][m], h1 = (_Float16)acc[R - 1][m];
+        *(uint32_t*)dst = (uint32_t)__builtin_bit_cast(uint16_t, h0) |
+                          ((uint32_t)__builtin_bit_cast(uint16_t, h1) << 16);
+      } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const _Float16 h = (_Float16)acc[r][m];
+          dst[r] = __builtin_bit_cast(uint16_t, h);
+        }
+      }
+    }
+  }
+}
+
+template <int MX, int MT, int STEPS>
+static hipError_t launch_unrolled(const WView& v, const w4_half* x, w4_half* c, int M,
+                                  hipStream_t s) {
+  const dim3 grid((unsigned)(v.N / (SIMT_WAVES * SIMT_R)), (unsigned)((M + MT - 1) / MT));
+  simt_unrolled_kernel<MX, MT, SIMT_R, STEPS><<<grid, SIMT_WAVES * 64, 0, s>>>(v, x, c, M);
+  return hipGetLastError();
+}
+
+// true (and launched) when the unrolled kernel applies
+template <int MX, int MT>
+static bool try_unrolled(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
+                         w4_half* w_out, hipError_t* err) {
+  if (w_out || v.K % 2048 || v.N % (SIMT_WAVES * SIMT_R)) return false;
+  if (!v.mx && v.gs % 32) return false;
+  if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)c & 3)) return false;
+  const int steps = v.K / 2048;
+  if (steps * MT > 8) return false;  // LDS: MT * K halves, at most 32 KiB
+  switch (steps) {
+    case 1: *err = launch_unrolled<MX, MT, 1>(v, x, c, M, s); return true;
+    case 2: *err = launch_unrolled<MX, MT, 2>(v, x, c, M, s); return true;
+    case 4: if (MT <= 2) { *err = launch_unrolled<MX, MT <= 2 ? MT : 1, 4>(v, x, c, M, s); return true; } return false;
+    default: return false;
+  }
+}
+
 template <int MX, int MT>
 static hipError_t launch_mt(const WView& v, const w4_half* x, w4_half* c, int M,
                             hipStream_t s, w4_half* w_out) {
   constexpr int R = SIMT_R;
+  hipError_t uerr = hipSuccess;
+  if (try_unrolled<MX, MT>(v, x, c, M, s, w_out, &uerr)) return uerr;
   const bool fast = (v.K % 32 == 0) && (((uintptr_t)v.q & 15) == 0) &&
                     (w_out == nullptr || ((uintptr_t)w_out & 15) == 0);
   const bool x_vec = (v.K % 8 == 0) && (((uintptr_t)x & 15) == 0);

@@ -149,6 +149,168 @@ __global__ __launch_bounds__(MMA_WAVES * 64) void mfma_skinny_kernel(
   }
 }
 
+// ---- large-M kernel -----------------------------------------------------------
+// Workgroup tile 256 (m) x 128 (n), k-step 64, 4 waves in a 2 x 2 grid, each
+// wave a 128 x 64 sub-tile (8 x 4 MFMA tiles, 128 accumulator VGPRs).  Both
+// operands go through LDS as FP16 with rows padded to 72 halves, which makes
+// every 16-lane ds_read_b128 group hit 16 distinct 16-byte bank groups.  The
+// packed weights of a k-step are one dwordx4 per thread; they are expanded in
+// VGPRs once per workgroup tile (so the dequant cost is amortised over 256
+// activation rows) and written to LDS in natural k order.  The global loads of
+// k-step t+1 are issued before the MFMAs of k-step t.
+//
+// Tiles are handed to workgroups so that the workgroups resident on one XCD
+// (ids congruent mod 8) walk the n-tiles of the same m-tile: the activation
+// slab stays in that XCD's L2 and every weight tile is fetched once per XCD.
+constexpr int TB_M = 256, TB_N = 128, TB_K = 64, TB_LD = TB_K + 8;
+
+template <int MX, bool HOOK, bool GS32>
+__global__ __launch_bounds__(256) void mfma_tile_kernel(const WView p,
+                                                        const w4_half* __restrict__ x,
+                                                        w4_half* __restrict__ c, const int M,
+                                                        w4_half* __restrict__ w_out,
+                                                        const int tiles_m, const int tiles_n) {
+  __shared__ __attribute__((aligned(16))) uint16_t xs[TB_M * TB_LD];
+  __shared__ __attribute__((aligned(16))) uint16_t ws[TB_N * TB_LD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
+  const int t = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+  if (t >= total) return;
+  const int m0 = (t / tiles_n) * TB_M, n0 = (t % tiles_n) * TB_N;
+  const int wm = (wave & 1) * 128, wn = (wave >> 1) * 64;
+  const int wpr = words(p.K);
+  const int wg = MX ? 0 : words(p.G);
+  const bool hook = HOOK && m0 == 0;
+  constexpr int NS = (MX || GS32) ? 1 : 4;
+
+  f4 acc[8][4];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
+
+  // what this thread fetches per k-step
+  const int wrow = tid >> 1, whalf = tid & 1;           // weight row, 32-k half of the step
+  const int wn_row = min(n0 + wrow, p.N - 1);
+  u4 xg[8];
+  u4 wq;
+  uint32_t wsb[NS], wzp[NS];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int id = i * 256 + tid, row = id >> 3, kc = id & 7;
+      const int m = m0 + row;
+      xg[i] = m < M ? *(const u4*)(x + (size_t)m * p.K + k0 + kc * 8) : u4{0u, 0u, 0u, 0u};
+    }
+    const int w0 = (k0 >> 3) + whalf * 4;
+    wq = __builtin_nontemporal_load((const u4*)(p.q + (size_t)wn_row * wpr + w0));
+#pragma unroll
+    for (int i = 0; i < NS; ++i) {
+      if (MX) {
+        wsb[i] = ((const uint8_t*)p.scales)[(size_t)wn_row * p.B + (w0 >> 2)];
+        wzp[i] = 0;
+      } else {
+        const int g = (8 * (w0 + i)) / p.gs;
+        wsb[i] = ((const uint16_t*)p.scales)[(size_t)wn_row * p.G + g];
+        wzp[i] = p.symmetric ? 8u
+                             : ((p.zeros[(size_t)wn_row * wg + (g >> 3)] >> (4 * (g & 7))) & 0xFu);
+      }
+    }
+  };
+
+  fetch(0);
+  for (int k0 = 0; k0 < p.K; k0 += TB_K) {
+    // registers -> LDS (weights expanded on the way)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int id = i * 256 + tid, row = id >> 3, kc = id & 7;
+      *(u4*)(xs + row * TB_LD + kc * 8) = xg[i];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      h2 d[4], nat[4];
+      if (MX) {
+        dq_mx(wq[j], mx_scale(wsb[0]), nat);
+      } else {
+        const int i = NS == 1 ? 0 : j;
+        dq_w4(wq[j], w4_group((uint16_t)wsb[i], (int)wzp[i]), d);
+        to_natural(d, nat);
+      }
+      const u4 v = u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
+      *(u4*)(ws + wrow * TB_LD + whalf * 32 + j * 8) = v;
+      if (hook && n0 + wrow < p.N)
+        *(u4*)(w_out + (size_t)(n0 + wrow) * p.K + k0 + whalf * 32 + j * 8) = v;
+    }
+    __syncthreads();
+    if (k0 + TB_K < p.K) fetch(k0 + TB_K);
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      h8 a[4], b[8];
+      const int koff = kk * 32 + (lane >> 4) * 8;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        a[j] = *(const h8*)(ws + (wn + j * 16 + (lane & 15)) * TB_LD + koff);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        b[i] = *(const h8*)(xs + (wm + i * 16 + (lane & 15)) * TB_LD + koff);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j], b[i], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  // lane holds c[m][n .. n+4) for m = tile row (lane & 15), n = 4 * (lane >> 4)
+  const bool vec_ok = (p.N & 3) == 0 && (((uintptr_t)c & 7) == 0);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int m = m0 + wm + i * 16 + (lane & 15);
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + wn + j * 16 + 4 * (lane >> 4);
+      uint16_t hv[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const _Float16 h = (_Float16)acc[i][j][e];
+        hv[e] = __builtin_bit_cast(uint16_t, h);
+      }
+      uint16_t* dst = c + (size_t)m * p.N + n;
+      if (vec_ok && n + 3 < p.N) {
+        *(u2*)dst = u2{hv[0] | ((uint32_t)hv[1] << 16), hv[2] | ((uint32_t)hv[3] << 16)};
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < p.N) dst[e] = hv[e];
+      }
+    }
+  }
+}
+
+template <int MX>
+static bool try_tile(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
+                     w4_half* w_out, hipError_t* err) {
+  if (M < 96 || v.K % TB_K) return false;
+  if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || (w_out && ((uintptr_t)w_out & 15))) return false;
+  const int tiles_m = (M + TB_M - 1) / TB_M, tiles_n = (v.N + TB_N - 1) / TB_N;
+  const long long total = (long long)tiles_m * tiles_n;
+  if (total > (1LL << 28)) return false;
+  const unsigned grid = (unsigned)(8 * ((total + 7) / 8));
+  const bool gs32 = v.mx || v.gs % 32 == 0;
+#define W4_GO(HOOK, GS) \
+  mfma_tile_kernel<MX, HOOK, GS><<<grid, 256, 0, s>>>(v, x, c, M, w_out, tiles_m, tiles_n)
+  if (w_out) {
+    if (gs32) W4_GO(true, true); else W4_GO(true, false);
+  } else {
+    if (gs32) W4_GO(false, true); else W4_GO(false, false);
+  }
+#undef W4_GO
+  *err = hipGetLastError();
+  return true;
+}
+
 template <int MX, int MTILES>
 static hipError_t launch_tiles(const WView& v, const w4_half* x, w4_half* c, int M,
                                hipStream_t s, w4_half* w_out) {
@@ -171,6 +333,8 @@ static hipError_t launch_tiles(const WView& v, const w4_half* x, w4_half* c, int
 template <int MX>
 static hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M,
                              hipStream_t s, w4_half* w_out) {
+  hipError_t terr = hipSuccess;
+  if (try_tile<MX>(v, x, c, M, s, w_out, &terr)) return terr;
   if (M <= 16) return launch_tiles<MX, 1>(v, x, c, M, s, w_out);
   if (M <= 32) return launch_tiles<MX, 2>(v, x, c, M, s, w_out);
   return launch_tiles<MX, 4>(v, x, c, M, s, w_out);

@@ -150,122 +150,152 @@ __global__ __launch_bounds__(MMA_WAVES * 64) void mfma_skinny_kernel(
 }
 
 // ---- large-M kernel -----------------------------------------------------------
-// Workgroup tile 256 (m) x 128 (n), k-step 64, 4 waves in a 2 x 2 grid, each
-// wave a 128 x 64 sub-tile (8 x 4 MFMA tiles, 128 accumulator VGPRs).  Both
+// Workgroup tile 256 (m) x 128 (n), k-step 64, 8 waves in a 4 x 2 grid, each
+// wave a 64 x 64 sub-tile (4 x 4 MFMA tiles, 64 accumulator VGPRs), two waves
+// per SIMD so one wave's LDS reads hide behind the other's MFMAs.  Both
 // operands go through LDS as FP16 with rows padded to 72 halves, which makes
 // every 16-lane ds_read_b128 group hit 16 distinct 16-byte bank groups.  The
-// packed weights of a k-step are one dwordx4 per thread; they are expanded in
+// packed weights of a k-step are one dwordx2 per thread; they are expanded in
 // VGPRs once per workgroup tile (so the dequant cost is amortised over 256
-// activation rows) and written to LDS in natural k order.  The global loads of
-// k-step t+1 are issued before the MFMAs of k-step t.
+// activation rows) and written to LDS in natural k order.
+//
+// A k-step of MFMAs is far shorter than an HBM round trip, so DEPTH k-steps are
+// kept in flight in registers; LDS is double buffered, one barrier per k-step.
+// The loop body is branch-free (rows past M and k-steps past K are clamped to
+// valid addresses and their results never stored), which lets the compiler
+// retire exactly the loads a k-step needs instead of draining the queue.
 //
 // Tiles are handed to workgroups so that the workgroups resident on one XCD
 // (ids congruent mod 8) walk the n-tiles of the same m-tile: the activation
 // slab stays in that XCD's L2 and every weight tile is fetched once per XCD.
-constexpr int TB_M = 256, TB_N = 128, TB_K = 64, TB_LD = TB_K + 8;
+constexpr int TB_M = 256, TB_N = 128, TB_K = 64, TB_LD = TB_K + 8, TB_THREADS = 512;
 
-template <int MX, bool HOOK, bool GS32>
-__global__ __launch_bounds__(256) void mfma_tile_kernel(const WView p,
-                                                        const w4_half* __restrict__ x,
-                                                        w4_half* __restrict__ c, const int M,
-                                                        w4_half* __restrict__ w_out,
-                                                        const int tiles_m, const int tiles_n) {
-  __shared__ __attribute__((aligned(16))) uint16_t xs[TB_M * TB_LD];
-  __shared__ __attribute__((aligned(16))) uint16_t ws[TB_N * TB_LD];
+// FMT: 0 W4 symmetric, 1 W4 asymmetric, 2 MXFP4
+template <int FMT, bool HOOK, bool GS16, int DEPTH>
+__global__ __launch_bounds__(TB_THREADS) void mfma_tile_kernel(
+    const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
+    w4_half* __restrict__ w_out, const int tiles_m, const int tiles_n) {
+  constexpr bool MX = FMT == 2;
+  __shared__ __attribute__((aligned(16))) uint16_t xs[2][TB_M * TB_LD];
+  __shared__ __attribute__((aligned(16))) uint16_t ws[2][TB_N * TB_LD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int total = tiles_m * tiles_n, per_xcd = (total + 7) / 8;
   const int t = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
   if (t >= total) return;
   const int m0 = (t / tiles_n) * TB_M, n0 = (t % tiles_n) * TB_N;
-  const int wm = (wave & 1) * 128, wn = (wave >> 1) * 64;
+  const int wm = (wave & 3) * 64, wn = (wave >> 2) * 64;
   const int wpr = words(p.K);
   const int wg = MX ? 0 : words(p.G);
   const bool hook = HOOK && m0 == 0;
-  constexpr int NS = (MX || GS32) ? 1 : 4;
+  constexpr int NS = (MX || GS16) ? 1 : 2;
+  const int nk = p.K / TB_K;
 
-  f4 acc[8][4];
+  f4 acc[4][4];
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
+  for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
 
-  // what this thread fetches per k-step
-  const int wrow = tid >> 1, whalf = tid & 1;           // weight row, 32-k half of the step
-  const int wn_row = min(n0 + wrow, p.N - 1);
-  u4 xg[8];
-  u4 wq;
-  uint32_t wsb[NS], wzp[NS];
-  auto fetch = [&](int k0) {
+  // What this thread fetches per k-step: 4 x 16 bytes of activations (row
+  // clamped to M-1) and 2 packed words of one weight row (clamped to N-1).
+  const int wrow = tid >> 2, wq4 = tid & 3;  // weight row of the tile, 16-k quarter of the step
+  const uint32_t* qrow = p.q + (size_t)min(n0 + wrow, p.N - 1) * wpr + wq4 * 2;
+  const size_t srow = (size_t)min(n0 + wrow, p.N - 1);
+  const uint16_t* xrow[4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int id = i * 256 + tid, row = id >> 3, kc = id & 7;
-      const int m = m0 + row;
-      xg[i] = m < M ? *(const u4*)(x + (size_t)m * p.K + k0 + kc * 8) : u4{0u, 0u, 0u, 0u};
-    }
-    const int w0 = (k0 >> 3) + whalf * 4;
-    wq = __builtin_nontemporal_load((const u4*)(p.q + (size_t)wn_row * wpr + w0));
+  for (int i = 0; i < 4; ++i) {
+    const int id = i * TB_THREADS + tid;
+    xrow[i] = x + (size_t)min(m0 + (id >> 3), M - 1) * p.K + (id & 7) * 8;
+  }
+  struct Slot {
+    u4 xg[4];
+    u2 wq;
+    uint32_t wsb[NS], wzw[NS];
+  };
+  Slot ring[DEPTH];
+  auto fetch = [&](Slot& sl, int kt) {
+    const int k0 = min(kt, nk - 1) * TB_K;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sl.xg[i] = *(const u4*)(xrow[i] + k0);
+    sl.wq = __builtin_nontemporal_load((const u2*)(qrow + (k0 >> 3)));
 #pragma unroll
     for (int i = 0; i < NS; ++i) {
+      const int w0 = (k0 >> 3) + wq4 * 2 + i;
       if (MX) {
-        wsb[i] = ((const uint8_t*)p.scales)[(size_t)wn_row * p.B + (w0 >> 2)];
-        wzp[i] = 0;
+        sl.wsb[i] = ((const uint8_t*)p.scales)[srow * p.B + (w0 >> 2)];
       } else {
-        const int g = (8 * (w0 + i)) / p.gs;
-        wsb[i] = ((const uint16_t*)p.scales)[(size_t)wn_row * p.G + g];
-        wzp[i] = p.symmetric ? 8u
-                             : ((p.zeros[(size_t)wn_row * wg + (g >> 3)] >> (4 * (g & 7))) & 0xFu);
+        const int g = (8 * w0) / p.gs;
+        sl.wsb[i] = ((const uint16_t*)p.scales)[srow * p.G + g];
+        if (FMT == 1) sl.wzw[i] = p.zeros[srow * wg + (g >> 3)];
       }
     }
   };
-
-  fetch(0);
-  for (int k0 = 0; k0 < p.K; k0 += TB_K) {
-    // registers -> LDS (weights expanded on the way)
+  auto stage = [&](const Slot& sl, int buf, int kt) {  // registers -> LDS, weights expanded
+    const int k0 = kt * TB_K;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int id = i * 256 + tid, row = id >> 3, kc = id & 7;
-      *(u4*)(xs + row * TB_LD + kc * 8) = xg[i];
+    for (int i = 0; i < 4; ++i) {
+      const int id = i * TB_THREADS + tid, row = id >> 3, kc = id & 7;
+      *(u4*)(xs[buf] + row * TB_LD + kc * 8) = sl.xg[i];
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < 2; ++j) {
       h2 d[4], nat[4];
       if (MX) {
-        dq_mx(wq[j], mx_scale(wsb[0]), nat);
+        dq_mx(sl.wq[j], mx_scale(sl.wsb[0]), nat);
       } else {
         const int i = NS == 1 ? 0 : j;
-        dq_w4(wq[j], w4_group((uint16_t)wsb[i], (int)wzp[i]), d);
+        int z = 8;
+        if (FMT == 1) {
+          const int g = (k0 + wq4 * 16 + 8 * j) / p.gs;
+          z = (int)((sl.wzw[i] >> (4 * (g & 7))) & 0xFu);
+        }
+        dq_w4(sl.wq[j], w4_group((uint16_t)sl.wsb[i], z), d);
         to_natural(d, nat);
       }
       const u4 v = u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
-      *(u4*)(ws + wrow * TB_LD + whalf * 32 + j * 8) = v;
+      *(u4*)(ws[buf] + wrow * TB_LD + wq4 * 16 + j * 8) = v;
       if (hook && n0 + wrow < p.N)
-        *(u4*)(w_out + (size_t)(n0 + wrow) * p.K + k0 + whalf * 32 + j * 8) = v;
+        *(u4*)(w_out + (size_t)(n0 + wrow) * p.K + k0 + wq4 * 16 + j * 8) = v;
     }
-    __syncthreads();
-    if (k0 + TB_K < p.K) fetch(k0 + TB_K);
+  };
+
 #pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      h8 a[4], b[8];
-      const int koff = kk * 32 + (lane >> 4) * 8;
+  for (int d = 0; d < DEPTH; ++d) fetch(ring[d], d);
+  stage(ring[0], 0, 0);
+  __syncthreads();
+  for (int kt0 = 0; kt0 < nk; kt0 += DEPTH) {  // nk is a multiple of DEPTH
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        a[j] = *(const h8*)(ws + (wn + j * 16 + (lane & 15)) * TB_LD + koff);
+    for (int d = 0; d < DEPTH; ++d) {
+      const int kt = kt0 + d;
+      const int buf = kt & 1;
+      fetch(ring[d], kt + DEPTH);  // slot d held k-step kt, which is already in LDS
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
-        b[i] = *(const h8*)(xs + (wm + i * 16 + (lane & 15)) * TB_LD + koff);
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
+      for (int kk = 0; kk < 2; ++kk) {
+        h8 a[4], b[4];
+        const int koff = kk * 32 + (lane >> 4) * 8;
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j], b[i], acc[i][j], 0, 0, 0);
+          a[j] = *(const h8*)(ws[buf] + (wn + j * 16 + (lane & 15)) * TB_LD + koff);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          b[i] = *(const h8*)(xs[buf] + (wm + i * 16 + (lane & 15)) * TB_LD + koff);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j], b[i], acc[i][j], 0, 0, 0);
+      }
+      // k-step kt+1 goes to the other buffer (a surplus copy of the last k-step
+      // on the final iteration: nobody reads it)
+      stage(ring[(d + 1) % DEPTH], buf ^ 1, min(kt + 1, nk - 1));
+      __syncthreads();
     }
-    __syncthreads();
   }
 
   // lane holds c[m][n .. n+4) for m = tile row (lane & 15), n = 4 * (lane >> 4)
   const bool vec_ok = (p.N & 3) == 0 && (((uintptr_t)c & 7) == 0);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < 4; ++i) {
     const int m = m0 + wm + i * 16 + (lane & 15);
     if (m >= M) continue;
 #pragma unroll
@@ -289,6 +319,28 @@ __global__ __launch_bounds__(256) void mfma_tile_kernel(const WView p,
   }
 }
 
+template <int FMT, bool HOOK, bool GS16, int DEPTH>
+static hipError_t launch_tile(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
+                              w4_half* w_out, int tiles_m, int tiles_n, unsigned grid) {
+  mfma_tile_kernel<FMT, HOOK, GS16, DEPTH>
+      <<<grid, TB_THREADS, 0, s>>>(v, x, c, M, w_out, tiles_m, tiles_n);
+  return hipGetLastError();
+}
+
+template <int FMT>
+static hipError_t launch_tile_fmt(const WView& v, const w4_half* x, w4_half* c, int M,
+                                  hipStream_t s, w4_half* w_out, int tm, int tn, unsigned grid) {
+  const bool gs16 = v.mx || v.gs % 16 == 0;
+  const int nk = v.K / TB_K;
+  if (w_out)
+    return gs16 ? launch_tile<FMT, true, true, 1>(v, x, c, M, s, w_out, tm, tn, grid)
+                : launch_tile<FMT, true, false, 1>(v, x, c, M, s, w_out, tm, tn, grid);
+  if (!gs16) return launch_tile<FMT, false, false, 1>(v, x, c, M, s, w_out, tm, tn, grid);
+  if (nk % 4 == 0) return launch_tile<FMT, false, true, 4>(v, x, c, M, s, w_out, tm, tn, grid);
+  if (nk % 2 == 0) return launch_tile<FMT, false, true, 2>(v, x, c, M, s, w_out, tm, tn, grid);
+  return launch_tile<FMT, false, true, 1>(v, x, c, M, s, w_out, tm, tn, grid);
+}
+
 template <int MX>
 static bool try_tile(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                      w4_half* w_out, hipError_t* err) {
@@ -298,16 +350,9 @@ static bool try_tile(const WView& v, const w4_half* x, w4_half* c, int M, hipStr
   const long long total = (long long)tiles_m * tiles_n;
   if (total > (1LL << 28)) return false;
   const unsigned grid = (unsigned)(8 * ((total + 7) / 8));
-  const bool gs32 = v.mx || v.gs % 32 == 0;
-#define W4_GO(HOOK, GS) \
-  mfma_tile_kernel<MX, HOOK, GS><<<grid, 256, 0, s>>>(v, x, c, M, w_out, tiles_m, tiles_n)
-  if (w_out) {
-    if (gs32) W4_GO(true, true); else W4_GO(true, false);
-  } else {
-    if (gs32) W4_GO(false, true); else W4_GO(false, false);
-  }
-#undef W4_GO
-  *err = hipGetLastError();
+  if (MX) *err = launch_tile_fmt<2>(v, x, c, M, s, w_out, tiles_m, tiles_n, grid);
+  else if (v.symmetric) *err = launch_tile_fmt<0>(v, x, c, M, s, w_out, tiles_m, tiles_n, grid);
+  else *err = launch_tile_fmt<1>(v, x, c, M, s, w_out, tiles_m, tiles_n, grid);
   return true;
 }
 

@@ -6,7 +6,8 @@ import ctypes as C
 import os
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG, "lib", "libw4amd.so")
+# W4AMD_LIB points at another build of the same library (kernel tuning builds)
+LIB_PATH = os.environ.get("W4AMD_LIB") or os.path.join(_PKG, "lib", "libw4amd.so")
 
 W4_OK, W4_EINVAL, W4_ERUNTIME = 0, 1, 2
 

@@ -150,9 +150,8 @@ __global__ __launch_bounds__(MMA_WAVES * 64) void mfma_skinny_kernel(
 }
 
 // ---- large-M kernel -----------------------------------------------------------
-// Workgroup tile 256 (m) x 128 (n), k-step 64, 8 waves in a 4 x 2 grid, each
-// wave a 64 x 64 sub-tile (4 x 4 MFMA tiles, 64 accumulator VGPRs), two waves
-// per SIMD so one wave's LDS reads hide behind the other's MFMAs.  Both
+// Workgroup tile 256 (m) x 128 (n), k-step 64, WM x WN waves each owning a
+// (256/WM) x (128/WN) sub-tile of 16x16 MFMA tiles.  Both
 // operands go through LDS as FP16 with rows padded to 72 halves, which makes
 // every 16-lane ds_read_b128 group hit 16 distinct 16-byte bank groups.  The
 // packed weights of a k-step are one dwordx2 per thread; they are expanded in
@@ -168,14 +167,20 @@ __global__ __launch_bounds__(MMA_WAVES * 64) void mfma_skinny_kernel(
 // Tiles are handed to workgroups so that the workgroups resident on one XCD
 // (ids congruent mod 8) walk the n-tiles of the same m-tile: the activation
 // slab stays in that XCD's L2 and every weight tile is fetched once per XCD.
-constexpr int TB_M = 256, TB_N = 128, TB_K = 64, TB_LD = TB_K + 8, TB_THREADS = 512;
+constexpr int TB_M = 256, TB_N = 128, TB_K = 64, TB_LD = TB_K + 8;
 
-// FMT: 0 W4 symmetric, 1 W4 asymmetric, 2 MXFP4
-template <int FMT, bool HOOK, bool GS16, int DEPTH>
-__global__ __launch_bounds__(TB_THREADS) void mfma_tile_kernel(
+// FMT: 0 W4 symmetric, 1 W4 asymmetric, 2 MXFP4.  WM x WN waves, each a
+// (256/WM) x (128/WN) sub-tile.
+template <int FMT, bool HOOK, bool GS16, int DEPTH, int WM, int WN>
+__global__ __launch_bounds__(WM * WN * 64) void mfma_tile_kernel(
     const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
     w4_half* __restrict__ w_out, const int tiles_m, const int tiles_n) {
   constexpr bool MX = FMT == 2;
+  constexpr int THREADS = WM * WN * 64;
+  constexpr int TI = TB_M / WM / 16, TJ = TB_N / WN / 16;  // MFMA tiles per wave
+  constexpr int XCH = TB_M * 8 / THREADS;                   // 16-byte activation chunks per thread
+  constexpr int WPT = TB_N * 8 / THREADS;                   // packed words per thread (2 or 4)
+  constexpr int TPR = 8 / WPT;                              // threads per weight row
   __shared__ __attribute__((aligned(16))) uint16_t xs[2][TB_M * TB_LD];
   __shared__ __attribute__((aligned(16))) uint16_t ws[2][TB_N * TB_LD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -183,44 +188,52 @@ __global__ __launch_bounds__(TB_THREADS) void mfma_tile_kernel(
   const int t = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
   if (t >= total) return;
   const int m0 = (t / tiles_n) * TB_M, n0 = (t % tiles_n) * TB_N;
-  const int wm = (wave & 3) * 64, wn = (wave >> 2) * 64;
+  const int wm = (wave % WM) * (TB_M / WM), wn = (wave / WM) * (TB_N / WN);
   const int wpr = words(p.K);
   const int wg = MX ? 0 : words(p.G);
   const bool hook = HOOK && m0 == 0;
-  constexpr int NS = (MX || GS16) ? 1 : 2;
+  constexpr int NS = (MX || GS16) ? 1 : WPT;  // GS16: one group per thread's words
   const int nk = p.K / TB_K;
 
-  f4 acc[4][4];
+  f4 acc[TI][TJ];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < TJ; ++j) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
 
-  // What this thread fetches per k-step: 4 x 16 bytes of activations (row
-  // clamped to M-1) and 2 packed words of one weight row (clamped to N-1).
-  const int wrow = tid >> 2, wq4 = tid & 3;  // weight row of the tile, 16-k quarter of the step
-  const uint32_t* qrow = p.q + (size_t)min(n0 + wrow, p.N - 1) * wpr + wq4 * 2;
+  // What this thread fetches per k-step: XCH x 16 bytes of activations (row
+  // clamped to M-1) and WPT packed words of one weight row (clamped to N-1).
+  const int wrow = tid / TPR, wpart = tid % TPR;
+  const uint32_t* qrow = p.q + (size_t)min(n0 + wrow, p.N - 1) * wpr + wpart * WPT;
   const size_t srow = (size_t)min(n0 + wrow, p.N - 1);
-  const uint16_t* xrow[4];
+  const uint16_t* xrow[XCH];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int id = i * TB_THREADS + tid;
+  for (int i = 0; i < XCH; ++i) {
+    const int id = i * THREADS + tid;
     xrow[i] = x + (size_t)min(m0 + (id >> 3), M - 1) * p.K + (id & 7) * 8;
   }
   struct Slot {
-    u4 xg[4];
-    u2 wq;
+    u4 xg[XCH];
+    uint32_t wq[WPT];
     uint32_t wsb[NS], wzw[NS];
   };
   Slot ring[DEPTH];
   auto fetch = [&](Slot& sl, int kt) {
     const int k0 = min(kt, nk - 1) * TB_K;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) sl.xg[i] = *(const u4*)(xrow[i] + k0);
-    sl.wq = __builtin_nontemporal_load((const u2*)(qrow + (k0 >> 3)));
+    for (int i = 0; i < XCH; ++i) sl.xg[i] = *(const u4*)(xrow[i] + k0);
+    if constexpr (WPT == 4) {
+      const u4 v = __builtin_nontemporal_load((const u4*)(qrow + (k0 >> 3)));
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sl.wq[j] = v[j];
+    } else {
+      const u2 v = __builtin_nontemporal_load((const u2*)(qrow + (k0 >> 3)));
+      sl.wq[0] = v[0];
+      sl.wq[1] = v[1];
+    }
 #pragma unroll
     for (int i = 0; i < NS; ++i) {
-      const int w0 = (k0 >> 3) + wq4 * 2 + i;
+      const int w0 = (k0 >> 3) + wpart * WPT + i;
       if (MX) {
         sl.wsb[i] = ((const uint8_t*)p.scales)[srow * p.B + (w0 >> 2)];
       } else {
@@ -233,12 +246,12 @@ __global__ __launch_bounds__(TB_THREADS) void mfma_tile_kernel(
   auto stage = [&](const Slot& sl, int buf, int kt) {  // registers -> LDS, weights expanded
     const int k0 = kt * TB_K;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int id = i * TB_THREADS + tid, row = id >> 3, kc = id & 7;
+    for (int i = 0; i < XCH; ++i) {
+      const int id = i * THREADS + tid, row = id >> 3, kc = id & 7;
       *(u4*)(xs[buf] + row * TB_LD + kc * 8) = sl.xg[i];
     }
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < WPT; ++j) {
       h2 d[4], nat[4];
       if (MX) {
         dq_mx(sl.wq[j], mx_scale(sl.wsb[0]), nat);
@@ -246,16 +259,16 @@ __global__ __launch_bounds__(TB_THREADS) void mfma_tile_kernel(
         const int i = NS == 1 ? 0 : j;
         int z = 8;
         if (FMT == 1) {
-          const int g = (k0 + wq4 * 16 + 8 * j) / p.gs;
+          const int g = (k0 + (wpart * WPT + j) * 8) / p.gs;
           z = (int)((sl.wzw[i] >> (4 * (g & 7))) & 0xFu);
         }
         dq_w4(sl.wq[j], w4_group((uint16_t)sl.wsb[i], z), d);
         to_natural(d, nat);
       }
       const u4 v = u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
-      *(u4*)(ws[buf] + wrow * TB_LD + wq4 * 16 + j * 8) = v;
+      *(u4*)(ws[buf] + wrow * TB_LD + (wpart * WPT + j) * 8) = v;
       if (hook && n0 + wrow < p.N)
-        *(u4*)(w_out + (size_t)(n0 + wrow) * p.K + k0 + wq4 * 16 + j * 8) = v;
+        *(u4*)(w_out + (size_t)(n0 + wrow) * p.K + k0 + (wpart * WPT + j) * 8) = v;
     }
   };
 
@@ -269,25 +282,26 @@ __global__ __launch_bounds__(TB_THREADS) void mfma_tile_kernel(
       const int kt = kt0 + d;
       const int buf = kt & 1;
       fetch(ring[d], kt + DEPTH);  // slot d held k-step kt, which is already in LDS
-#pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        h8 a[4], b[4];
-        const int koff = kk * 32 + (lane >> 4) * 8;
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          a[j] = *(const h8*)(ws[buf] + (wn + j * 16 + (lane & 15)) * TB_LD + koff);
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          b[i] = *(const h8*)(xs[buf] + (wm + i * 16 + (lane & 15)) * TB_LD + koff);
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j], b[i], acc[i][j], 0, 0, 0);
-      }
+      __builtin_amdgcn_iglp_opt(0);  // let the scheduler weave LDS traffic between the MFMAs
       // k-step kt+1 goes to the other buffer (a surplus copy of the last k-step
       // on the final iteration: nobody reads it)
       stage(ring[(d + 1) % DEPTH], buf ^ 1, min(kt + 1, nk - 1));
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) {
+        h8 a[TJ], b[TI];
+        const int koff = kk * 32 + (lane >> 4) * 8;
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+          a[j] = *(const h8*)(ws[buf] + (wn + j * 16 + (lane & 15)) * TB_LD + koff);
+#pragma unroll
+        for (int i = 0; i < TI; ++i)
+          b[i] = *(const h8*)(xs[buf] + (wm + i * 16 + (lane & 15)) * TB_LD + koff);
+#pragma unroll
+        for (int i = 0; i < TI; ++i)
+#pragma unroll
+          for (int j = 0; j < TJ; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j], b[i], acc[i][j], 0, 0, 0);
+      }
       __syncthreads();
     }
   }
@@ -295,11 +309,11 @@ __global__ __launch_bounds__(TB_THREADS) void mfma_tile_kernel(
   // lane holds c[m][n .. n+4) for m = tile row (lane & 15), n = 4 * (lane >> 4)
   const bool vec_ok = (p.N & 3) == 0 && (((uintptr_t)c & 7) == 0);
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < TI; ++i) {
     const int m = m0 + wm + i * 16 + (lane & 15);
     if (m >= M) continue;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < TJ; ++j) {
       const int n = n0 + wn + j * 16 + 4 * (lane >> 4);
       uint16_t hv[4];
 #pragma unroll
@@ -319,24 +333,32 @@ __global__ __launch_bounds__(TB_THREADS) void mfma_tile_kernel(
   }
 }
 
-template <int FMT, bool HOOK, bool GS16, int DEPTH>
+// 4 x 2 waves (64 x 64 outputs each), 4 k-steps in flight: the fastest of the
+// (WM, WN, DEPTH) combinations measured at M = 2048 and 4096, N = K = 4096.
+#define W4_TILE_WM 4
+#define W4_TILE_WN 2
+#define W4_TILE_DEPTH 4
+
+template <int FMT, bool HOOK, bool GSOK, int DEPTH>
 static hipError_t launch_tile(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                               w4_half* w_out, int tiles_m, int tiles_n, unsigned grid) {
-  mfma_tile_kernel<FMT, HOOK, GS16, DEPTH>
-      <<<grid, TB_THREADS, 0, s>>>(v, x, c, M, w_out, tiles_m, tiles_n);
+  mfma_tile_kernel<FMT, HOOK, GSOK, DEPTH, W4_TILE_WM, W4_TILE_WN>
+      <<<grid, W4_TILE_WM * W4_TILE_WN * 64, 0, s>>>(v, x, c, M, w_out, tiles_m, tiles_n);
   return hipGetLastError();
 }
 
 template <int FMT>
 static hipError_t launch_tile_fmt(const WView& v, const w4_half* x, w4_half* c, int M,
                                   hipStream_t s, w4_half* w_out, int tm, int tn, unsigned grid) {
-  const bool gs16 = v.mx || v.gs % 16 == 0;
+  constexpr int WPT = TB_N * 8 / (W4_TILE_WM * W4_TILE_WN * 64);
+  const bool gsok = v.mx || v.gs % (8 * WPT) == 0;  // one group per thread's words
   const int nk = v.K / TB_K;
   if (w_out)
-    return gs16 ? launch_tile<FMT, true, true, 1>(v, x, c, M, s, w_out, tm, tn, grid)
+    return gsok ? launch_tile<FMT, true, true, 1>(v, x, c, M, s, w_out, tm, tn, grid)
                 : launch_tile<FMT, true, false, 1>(v, x, c, M, s, w_out, tm, tn, grid);
-  if (!gs16) return launch_tile<FMT, false, false, 1>(v, x, c, M, s, w_out, tm, tn, grid);
-  if (nk % 4 == 0) return launch_tile<FMT, false, true, 4>(v, x, c, M, s, w_out, tm, tn, grid);
+  if (!gsok) return launch_tile<FMT, false, false, 1>(v, x, c, M, s, w_out, tm, tn, grid);
+  if (nk % W4_TILE_DEPTH == 0)
+    return launch_tile<FMT, false, true, W4_TILE_DEPTH>(v, x, c, M, s, w_out, tm, tn, grid);
   if (nk % 2 == 0) return launch_tile<FMT, false, true, 2>(v, x, c, M, s, w_out, tm, tn, grid);
   return launch_tile<FMT, false, true, 1>(v, x, c, M, s, w_out, tm, tn, grid);
 }

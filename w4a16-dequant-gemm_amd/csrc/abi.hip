@@ -37,9 +37,11 @@ int done(const char* what, hipError_t e) {
   return e == hipSuccess ? W4_OK : runtime(what, e);
 }
 
-// Measured on MI355X: the matrix-core kernel overtakes the vector kernel from
-// this activation-row count on.
-constexpr int DISPATCH_MMA_MIN_M = 2;
+// Measured on MI355X (N = 4096 and 11008, K = 4096, gs = 128): the vector kernel
+// wins through M = 4 (5.8 vs 6.2 us and 12.7 vs 13.9 us at M = 4) and loses from
+// M = 5 on, where it needs a second pass over the activations (11.8 vs 6.5 us and
+// 34 vs 16 us at M = 8).
+constexpr int DISPATCH_MMA_MIN_M = 5;
 
 // Largest M the reference's launch grids accept; kept so callers see the same
 // rejections (fused.cuh:187-194, mma.cuh:253-254).

@@ -149,6 +149,372 @@ __global__ __launch_bounds__(MMA_WAVES * 64) void mfma_skinny_kernel(
   }
 }
 
+// ---- decode-batch kernel (2 <= M < 96, 16-byte aligned rows) ----------------------
+// A workgroup of 8 waves owns 16 * NT weight rows and 16 * MT activation rows;
+// the waves split K in runs of CH chunks of 128 k and combine through LDS in a
+// fixed order.  A round of a wave issues every load it needs before consuming
+// any: scales and zero-points, then the activations (B operands, 64 contiguous
+// bytes per lane and chunk, served by L2), then the packed weights (A operands,
+// the only HBM stream) -- loads return in issue order, so the weights arrive
+// last and nothing waits behind them.  Chunks past K are clamped to k = 0 and
+// their activations zeroed, which keeps the round branch-free.
+constexpr int DEC_WAVES = 8;
+
+template <int FMT, int MT, int NT, int CH, bool HOOK, bool GS32>
+__global__ __launch_bounds__(DEC_WAVES * 64) void mfma_decode_kernel(
+    const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
+    w4_half* __restrict__ w_out, const int gs_shift) {
+  constexpr bool MX = FMT == 2;
+  constexpr int NS = (MX || GS32) ? 1 : 4;  // group lookups per lane and chunk
+  __shared__ f4 red[DEC_WAVES][NT * MT][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, b = lane >> 4;
+  const int n0 = blockIdx.x * (16 * NT), m0 = blockIdx.y * (16 * MT);
+  const int wpr = p.K >> 3;
+  const int wg = MX ? 0 : words(p.G);
+  const int nchunks = (p.K + MMA_CHUNK - 1) / MMA_CHUNK;
+  const bool hook = HOOK && blockIdx.y == 0;
+
+  size_t nrow[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) nrow[t] = (size_t)min(n0 + 16 * t + r, p.N - 1);
+  const uint16_t* xrow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) xrow[mt] = x + (size_t)min(m0 + 16 * mt + r, M - 1) * p.K;
+
+  f4 acc[NT][MT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f4{0.f, 0.f, 0.f, 0.f};
+
+  for (int c0 = wave * CH; c0 < nchunks; c0 += DEC_WAVES * CH) {
+    int kl[CH];
+    bool ok[CH];
+    uint32_t sc[CH][NT][NS], zw[CH][NT][NS], zsh[CH][NS];
+    u4 xv[CH][MT][4], qw[CH][NT];
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int k = (c0 + i) * MMA_CHUNK + b * 32;
+      ok[i] = k < p.K;
+      kl[i] = ok[i] ? k : 0;
+    }
+#pragma unroll
+    for (int i = 0; i < CH; ++i)
+#pragma unroll
+      for (int e = 0; e < NS; ++e) {
+        const int kk = kl[i] + 8 * e;
+        const int g = MX ? (kk >> 5) : gs_shift >= 0 ? (kk >> gs_shift) : kk / p.gs;
+        zsh[i][e] = 4u * (uint32_t)(g & 7);
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          if (MX) {
+            sc[i][t][e] = ((const uint8_t*)p.scales)[nrow[t] * p.B + g];
+          } else {
+            sc[i][t][e] = ((const uint16_t*)p.scales)[nrow[t] * p.G + g];
+            if (FMT == 1) zw[i][t][e] = p.zeros[nrow[t] * wg + (g >> 3)];
+          }
+        }
+      }
+#pragma unroll
+    for (int i = 0; i < CH; ++i)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xv[i][mt][j] = *(const u4*)(xrow[mt] + kl[i] + 8 * j);
+#pragma unroll
+    for (int i = 0; i < CH; ++i)
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        qw[i][t] = __builtin_nontemporal_load((const u4*)(p.q + nrow[t] * wpr + (kl[i] >> 3)));
+
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (!ok[i]) xv[i][mt][j] = u4{0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          h2 d[4], nat[4];
+          const int e = NS == 1 ? 0 : j;
+          if (MX) {
+            dq_mx(qw[i][t][j], mx_scale(sc[i][t][0]), nat);
+          } else {
+            const int z = FMT == 1 ? (int)((zw[i][t][e] >> zsh[i][e]) & 0xFu) : 8;
+            dq_w4(qw[i][t][j], w4_group((uint16_t)sc[i][t][e], z), d);
+            to_natural(d, nat);
+          }
+          if (hook && ok[i] && n0 + 16 * t + r < p.N)
+            *(u4*)(w_out + nrow[t] * p.K + kl[i] + 8 * j) =
+                u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
+          const h8 a = pack_h8(nat);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                a, __builtin_bit_cast(h8, xv[i][mt][j]), acc[t][mt], 0, 0, 0);
+        }
+    }
+  }
+
+  // Fixed-order combine of the 8 K slices: wave w sums output tile w.
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) red[wave][t * MT + mt][lane] = acc[t][mt];
+  __syncthreads();
+  if (wave < NT * MT) {
+    f4 s = red[0][wave][lane];
+#pragma unroll
+    for (int w = 1; w < DEC_WAVES; ++w) s += red[w][wave][lane];
+    const int t = wave / MT, mt = wave % MT;
+    const int m = m0 + 16 * mt + r;       // activation row of this lane
+    const int nn = n0 + 16 * t + 4 * b;   // first of its 4 weight rows
+    if (m < M) {
+      uint16_t hv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const _Float16 h = (_Float16)s[i];
+        hv[i] = __builtin_bit_cast(uint16_t, h);
+      }
+      uint16_t* dst = c + (size_t)m * p.N + nn;
+      if (nn + 3 < p.N && (p.N & 3) == 0 && (((uintptr_t)c & 7) == 0)) {
+        *(u2*)dst = u2{hv[0] | ((uint32_t)hv[1] << 16), hv[2] | ((uint32_t)hv[3] << 16)};
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (nn + i < p.N) dst[i] = hv[i];
+      }
+    }
+  }
+}
+
+// One chunk per wave and round, one row tile per workgroup: the fastest of the
+// (NT, CH) combinations measured for M <= 16 (N = 4096 .. 14336, K = 4096 .. 11008).
+template <int FMT, int MT>
+static hipError_t launch_decode_mt(const WView& v, const w4_half* x, w4_half* c, int M,
+                                   hipStream_t s, w4_half* w_out) {
+  const bool gs32 = v.mx || v.gs % 32 == 0;
+  int gs_shift = -1;
+  if (!v.mx && (v.gs & (v.gs - 1)) == 0) gs_shift = __builtin_ctz((unsigned)v.gs);
+  const dim3 grid((unsigned)((v.N + 15) / 16), (unsigned)((M + 16 * MT - 1) / (16 * MT)));
+#define W4_GO(HOOK, GS) \
+  mfma_decode_kernel<FMT, MT, 1, 1, HOOK, GS><<<grid, DEC_WAVES * 64, 0, s>>>(v, x, c, M, w_out, gs_shift)
+  if (w_out) {
+    if (gs32) W4_GO(true, true); else W4_GO(true, false);
+  } else {
+    if (gs32) W4_GO(false, true); else W4_GO(false, false);
+  }
+#undef W4_GO
+  return hipGetLastError();
+}
+
+template <int FMT>
+static hipError_t launch_decode(const WView& v, const w4_half* x, w4_half* c, int M,
+                                hipStream_t s, w4_half* w_out) {
+  return launch_decode_mt<FMT, 1>(v, x, c, M, s, w_out);  // M <= 16
+}
+
+// ---- streaming decode-batch kernel --------------------------------------------------
+// 8 waves = NW row tiles x KW slices of K.  The waves of one K slice share the
+// activations of that slice through LDS (staged 128 k at a time, double
+// buffered, one barrier per step), so x crosses L2 -> CU once per workgroup
+// instead of once per wave; each wave streams its own 16 weight rows straight
+// into registers as MFMA A operands, DEPTH steps ahead.  Steps past the end of a
+// slice, and k past K, fetch from clamped addresses and stage zeros.
+template <int FMT, int MT, int NW, int KW, int DEPTH, bool HOOK, bool GS32>
+__global__ __launch_bounds__(512) void mfma_stream_kernel(
+    const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
+    w4_half* __restrict__ w_out, const int gs_shift) {
+  static_assert(NW * KW == 8, "8 waves");
+  constexpr bool MX = FMT == 2;
+  constexpr int NS = (MX || GS32) ? 1 : 4;
+  constexpr int ROWS = 16 * MT;
+  constexpr int LD = MMA_CHUNK + 8;           // halves per staged row: 16-lane reads hit 16 bank groups
+  constexpr int PIECES = KW * ROWS * 16;      // 16-byte pieces staged per step
+  constexpr int XP = (PIECES + 511) / 512;    // ... per thread
+  constexpr int XS_HALVES = 2 * KW * ROWS * LD;
+  constexpr int RED_HALVES = KW * NW * MT * 64 * 8;
+  __shared__ __attribute__((aligned(16))) uint16_t smem[XS_HALVES > RED_HALVES ? XS_HALVES : RED_HALVES];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, b = lane >> 4;
+  const int nw = wave % NW, kw = wave / NW;
+  const int n0 = blockIdx.x * (16 * NW) + 16 * nw, m0 = blockIdx.y * ROWS;
+  const int wpr = p.K >> 3;
+  const int wg = MX ? 0 : words(p.G);
+  const int nchunks = (p.K + MMA_CHUNK - 1) / MMA_CHUNK;
+  const int cpk = (nchunks + KW - 1) / KW;                  // chunks per K slice
+  const int steps = (cpk + DEPTH - 1) / DEPTH * DEPTH;
+  const bool hook = HOOK && blockIdx.y == 0 && n0 + r < p.N;
+  const size_t nrow = (size_t)min(n0 + r, p.N - 1);
+  const uint32_t* qrow = p.q + nrow * wpr;
+
+  // the pieces of x this thread stages every step
+  const uint16_t* xsrc[XP];  // start of the activation row
+  int xk0[XP], xdst[XP];     // first k of the piece at step 0; where it goes in a staging buffer
+#pragma unroll
+  for (int i = 0; i < XP; ++i) {
+    const int id = i * 512 + tid;
+    const int pk = (id / (ROWS * 16)) % KW, prow = (id >> 4) % ROWS, seg = (id & 15) * 8;
+    xsrc[i] = x + (size_t)min(m0 + prow, M - 1) * p.K;
+    xk0[i] = pk * cpk * MMA_CHUNK + seg;
+    xdst[i] = pk * (ROWS * LD) + prow * LD + seg;
+  }
+
+  struct Slot {
+    u4 q;
+    uint32_t sc[NS], zw[NS];
+    u4 xg[XP];
+  };
+  Slot ring[DEPTH];
+  auto group_of = [&](int kk) { return MX ? (kk >> 5) : gs_shift >= 0 ? (kk >> gs_shift) : kk / p.gs; };
+  auto lane_k = [&](int s) { return (kw * cpk + s) * MMA_CHUNK + b * 32; };
+  auto fetch = [&](Slot& sl, int s) {
+    const int k = lane_k(s);
+    const int kc = (s < cpk && k < p.K) ? k : 0;
+#pragma unroll
+    for (int e = 0; e < NS; ++e) {
+      const int g = group_of(kc + 8 * e);
+      if (MX) {
+        sl.sc[e] = ((const uint8_t*)p.scales)[nrow * p.B + g];
+      } else {
+        sl.sc[e] = ((const uint16_t*)p.scales)[nrow * p.G + g];
+        if (FMT == 1) sl.zw[e] = p.zeros[nrow * wg + (g >> 3)];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < XP; ++i) {
+      const int kx = xk0[i] + s * MMA_CHUNK;
+      sl.xg[i] = *(const u4*)(xsrc[i] + ((s < cpk && kx < p.K) ? kx : 0));
+    }
+    sl.q = __builtin_nontemporal_load((const u4*)(qrow + (kc >> 3)));
+  };
+  auto stage = [&](const Slot& sl, int buf, int s) {
+    uint16_t* base = smem + buf * (KW * ROWS * LD);
+#pragma unroll
+    for (int i = 0; i < XP; ++i) {
+      const int kx = xk0[i] + s * MMA_CHUNK;
+      const bool okx = s < cpk && kx < p.K;
+      if (XP * 512 == PIECES || i * 512 + tid < PIECES)
+        *(u4*)(base + xdst[i]) = okx ? sl.xg[i] : u4{0u, 0u, 0u, 0u};
+    }
+  };
+
+  f4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d) fetch(ring[d], d);
+  stage(ring[0], 0, 0);
+  __syncthreads();
+  for (int s0 = 0; s0 < steps; s0 += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      const int s = s0 + d, buf = s & 1;
+      const u4 q = ring[d].q;
+      uint32_t sc[NS], zw[NS];
+#pragma unroll
+      for (int e = 0; e < NS; ++e) sc[e] = ring[d].sc[e], zw[e] = ring[d].zw[e];
+      fetch(ring[d], s + DEPTH);  // slot d: weights copied out, activations staged one step ago
+      stage(ring[(d + 1) % DEPTH], buf ^ 1, s + 1);
+      const int k = lane_k(s);
+      const bool okw = s < cpk && k < p.K;
+      const int kc = okw ? k : 0;
+      const uint16_t* xb = smem + buf * (KW * ROWS * LD) + kw * (ROWS * LD) + r * LD + b * 32;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        h2 dq[4], nat[4];
+        const int e = NS == 1 ? 0 : j;
+        if (MX) {
+          dq_mx(q[j], mx_scale(sc[0]), nat);
+        } else {
+          int z = 8;
+          if (FMT == 1) z = (int)((zw[e] >> (4 * (group_of(kc + 8 * e) & 7))) & 0xFu);
+          dq_w4(q[j], w4_group((uint16_t)sc[e], z), dq);
+          to_natural(dq, nat);
+        }
+        if (hook && okw)
+          *(u4*)(w_out + nrow * p.K + kc + 8 * j) =
+              u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
+        const h8 a = pack_h8(nat);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const h8 bx = *(const h8*)(xb + mt * 16 * LD + j * 8);
+          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bx, acc[mt], 0, 0, 0);
+        }
+      }
+      __syncthreads();
+    }
+  }
+
+  // Fixed-order combine of the KW slices (the staging buffers are free now).
+  f4* red = (f4*)smem;  // [KW][NW * MT][64]
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) red[(kw * (NW * MT) + nw * MT + mt) * 64 + lane] = acc[mt];
+  __syncthreads();
+  for (int tile = wave; tile < NW * MT; tile += 8) {
+    f4 sum = red[tile * 64 + lane];
+#pragma unroll
+    for (int w = 1; w < KW; ++w) sum += red[(w * (NW * MT) + tile) * 64 + lane];
+    const int m = m0 + 16 * (tile % MT) + r;                              // activation row of this lane
+    const int nn = blockIdx.x * (16 * NW) + 16 * (tile / MT) + 4 * b;    // first of its 4 weight rows
+    if (m < M) {
+      uint16_t hv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const _Float16 h = (_Float16)sum[i];
+        hv[i] = __builtin_bit_cast(uint16_t, h);
+      }
+      uint16_t* dst = c + (size_t)m * p.N + nn;
+      if (nn + 3 < p.N && (p.N & 3) == 0 && (((uintptr_t)c & 7) == 0)) {
+        *(u2*)dst = u2{hv[0] | ((uint32_t)hv[1] << 16), hv[2] | ((uint32_t)hv[3] << 16)};
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (nn + i < p.N) dst[i] = hv[i];
+      }
+    }
+  }
+}
+
+// 4 row tiles x 2 K slices, 4 steps in flight (deeper rings measured slower).
+
+template <int FMT, int MT>
+static hipError_t launch_stream_mt(const WView& v, const w4_half* x, w4_half* c, int M,
+                                   hipStream_t s, w4_half* w_out) {
+  const bool gs32 = v.mx || v.gs % 32 == 0;
+  int gs_shift = -1;
+  if (!v.mx && (v.gs & (v.gs - 1)) == 0) gs_shift = __builtin_ctz((unsigned)v.gs);
+  constexpr int NW = 4, KW = 2, DEPTH = 4;
+  const dim3 grid((unsigned)((v.N + 16 * NW - 1) / (16 * NW)), (unsigned)((M + 16 * MT - 1) / (16 * MT)));
+  const int cpk = ((v.K + MMA_CHUNK - 1) / MMA_CHUNK + KW - 1) / KW;
+#define W4_GO(D, HOOK, GS) \
+  mfma_stream_kernel<FMT, MT, NW, KW, D, HOOK, GS><<<grid, 512, 0, s>>>(v, x, c, M, w_out, gs_shift)
+  if (w_out) {
+    if (gs32) W4_GO(1, true, true); else W4_GO(1, true, false);
+  } else if (!gs32) {
+    W4_GO(1, false, false);
+  } else if (cpk >= DEPTH) {
+    W4_GO(DEPTH, false, true);
+  } else {
+    W4_GO(1, false, true);
+  }
+#undef W4_GO
+  return hipGetLastError();
+}
+
+template <int FMT>
+static hipError_t launch_stream(const WView& v, const w4_half* x, w4_half* c, int M,
+                                hipStream_t s, w4_half* w_out) {
+  if (M <= 16) return launch_stream_mt<FMT, 1>(v, x, c, M, s, w_out);
+  if (M <= 32) return launch_stream_mt<FMT, 2>(v, x, c, M, s, w_out);
+  return launch_stream_mt<FMT, 4>(v, x, c, M, s, w_out);
+}
+
 // ---- large-M kernel -----------------------------------------------------------
 // Workgroup tile 256 (m) x 128 (n), k-step 64, WM x WN waves each owning a
 // (256/WM) x (128/WN) sub-tile of 16x16 MFMA tiles.  Both
@@ -402,6 +768,21 @@ static hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M
                              hipStream_t s, w4_half* w_out) {
   hipError_t terr = hipSuccess;
   if (try_tile<MX>(v, x, c, M, s, w_out, &terr)) return terr;
+  const bool aligned = (v.K % 32 == 0) && (((uintptr_t)v.q | (uintptr_t)x) & 15) == 0 &&
+                       (w_out == nullptr || ((uintptr_t)w_out & 15) == 0);
+  if (aligned) {
+    // Measured on N = 4096 .. 14336, K = 4096 .. 11008: the K-split kernel wins for
+    // M <= 16 unless N is large enough to give the streaming kernel a full grid.
+    const bool ksplit = M <= 8 || (M <= 16 && v.N < 8192);
+    if (ksplit) {
+      if (MX) return launch_decode<2>(v, x, c, M, s, w_out);
+      return v.symmetric ? launch_decode<0>(v, x, c, M, s, w_out)
+                         : launch_decode<1>(v, x, c, M, s, w_out);
+    }
+    if (MX) return launch_stream<2>(v, x, c, M, s, w_out);
+    return v.symmetric ? launch_stream<0>(v, x, c, M, s, w_out)
+                       : launch_stream<1>(v, x, c, M, s, w_out);
+  }
   if (M <= 16) return launch_tiles<MX, 1>(v, x, c, M, s, w_out);
   if (M <= 32) return launch_tiles<MX, 2>(v, x, c, M, s, w_out);
   return launch_tiles<MX, 4>(v, x, c, M, s, w_out);

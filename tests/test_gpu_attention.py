@@ -18,7 +18,10 @@ pytestmark = pytest.mark.gpu
 TOL, CROSS = 1e-3, 2e-3
 
 ATT = [(1, 1, 64, 32), (2, 7, 64, 8), (4, 128, 128, 128), (2, 300, 96, 32), (3, 65, 40, 8),
-       (1, 4096, 64, 64)]
+       (1, 4096, 64, 64),
+       # head dimension 128 takes the matrix-core kernel: one position, ragged tiles, gs 32 / 64,
+       # and gs = 8 (D = 128 on the general kernel)
+       (2, 1, 128, 32), (3, 33, 128, 32), (2, 129, 128, 64), (1, 777, 128, 32), (1, 300, 128, 8)]
 BIG = [(2, 5000, 64, 32), (1, 9000, 128, 64)]
 
 
@@ -73,14 +76,21 @@ def test_w4_flash_long(i, sym):
     _check_w4(c4, q)
 
 
-@pytest.mark.parametrize("group", [2, 3, 4, 7])
+@pytest.mark.parametrize("group", [2, 3, 4, 7, 16, 17, 40])
 def test_w4_flash_grouped_query(group):
-    c4, q = _w4_case(3, 700, 128, 32, True, 0x6A11 + group, group)
+    """Query heads sharing one slab; more than 16 heads take several passes."""
+    c4, q = _w4_case(3 if group < 16 else 2, 700, 128, 32, group % 2 == 0, 0x6A11 + group, group)
+    _check_w4(c4, q, group)
+
+
+@pytest.mark.parametrize("group", [3, 5])
+def test_w4_flash_grouped_query_general_kernel(group):
+    c4, q = _w4_case(2, 333, 64, 32, True, 0x6B22 + group, group)
     _check_w4(c4, q, group)
 
 
 F8 = [(1, 1, 64, 32), (2, 7, 64, 8), (4, 128, 128, 128), (2, 300, 96, 32), (3, 65, 40, 8),
-      (1, 9000, 128, 64)]
+      (1, 9000, 128, 64), (2, 1, 128, 32), (2, 100, 128, 32), (1, 300, 128, 16)]
 
 
 @pytest.mark.parametrize("i", range(len(F8)))
@@ -146,8 +156,35 @@ def test_f8_every_code_and_slab_scale():
     assert orc.rel_l2(f64(out), ref) <= TOL
 
 
+def test_f8_slab_scale_head_dim_128():
+    c = w4amd.capi()
+    H, S, D, gs, group = 2, 500, 128, 128, 4
+    rng = np.random.default_rng(5)
+    kk = rng.standard_normal(H * S * D)
+    c8 = orc.quantize_cache_f8(kk, kk[::-1].copy(), H, S, D, gs)
+    slab_k = np.array([0x2000, 0x2400], np.uint16)
+    slab_v = np.array([0x2200, 0x1C00], np.uint16)
+    c8b = orc.KVCacheF8()
+    c8b.__dict__.update(c8.__dict__)
+    c8b.s_k, c8b.s_v = np.repeat(slab_k, S * c8.G), np.repeat(slab_v, S * c8.G)
+    q = orc.normal_activations(H * group * D, 78)
+    ref = orc.attention_reference_f8(q, c8b, heads_per_slab=group)
+    d8 = DevKVF8(c8, slab_k, slab_v)
+    out = halves(H * group * D, 0x7E00)
+    ko, vo = halves(H * S * D, 0x7E00), halves(H * S * D, 0x7E00)
+    c.attention_f8_flash(d8.view, ptr(to_dev(q)), ptr(out), 0, ptr(ko), ptr(vo), group=group, scale_mode=1)
+    assert np.array_equal(bits(ko), orc.dequant_cache_f8(c8b, False).ravel())
+    assert np.array_equal(bits(vo), orc.dequant_cache_f8(c8b, True).ravel())
+    assert orc.rel_l2(f64(out), ref) <= TOL
+    out2 = halves(H * group * D, 0x7E00)
+    c.attention_f8_flash(d8.view, ptr(to_dev(q)), ptr(out2), group=group, scale_mode=1)
+    assert np.array_equal(bits(out2), bits(out))
+
+
 PAGED = [(2, 300, 96, 32, 16), (2, 520, 64, 32, 16), (1, 1000, 128, 64, 64), (3, 65, 40, 8, 32),
-         (1, 5000, 64, 32, 256)]
+         (1, 5000, 64, 32, 256),
+         # matrix-core kernel: page 16, a page size that is no multiple of 16, one-row pages
+         (2, 700, 128, 32, 16), (1, 530, 128, 32, 24), (1, 100, 128, 128, 1), (2, 2000, 128, 32, 256)]
 
 
 def _paged_pool(c4, page, bt):
@@ -183,11 +220,12 @@ def test_paged_equals_contiguous(i, sym):
     assert np.array_equal(bits(ko), kd.ravel()) and np.array_equal(bits(vo), vd.ravel())
 
 
-def test_paged_batched_prefix_sharing():
+@pytest.mark.parametrize("D", [64, 128])
+def test_paged_batched_prefix_sharing(D):
     """Four sequences over one pool; the first three share their leading pages.
     Each sequence's output equals the contiguous kernel run on its logical cache."""
     c = w4amd.capi()
-    Hkv, D, gs, page, group = 2, 64, 32, 16, 2
+    Hkv, gs, page, group = 2, 32, 16, 2
     S, prefix = 520, 208                     # 13 shared pages
     nseq = 4
     lp = (S + page - 1) // page

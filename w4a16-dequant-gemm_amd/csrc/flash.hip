@@ -24,7 +24,6 @@ constexpr int FL_TILE = 256;   // positions per tile
 constexpr int FL_WAVES = 4;
 constexpr int FL_MAXGQ = 4;    // query heads handled per pass
 
-enum { KIND_F16 = 0, KIND_W4 = 1, KIND_F8 = 2 };
 
 // Offset within a lane's E-element chunk of register pair p, half hf.
 template <int KIND>
@@ -284,35 +283,82 @@ __global__ __launch_bounds__(FL_WAVES * 64) void flash_phase1(const FlashArgs a,
 }
 
 // Phase 2: out[d] = sum_t exp(m_t - M) acc_t[d] / sum_t exp(m_t - M) l_t.
-__global__ __launch_bounds__(128) void flash_phase2(const float* __restrict__ part,
-                                                    w4_half* __restrict__ out, const int T,
-                                                    const int D) {
+// One workgroup per query head.  The split weights are computed once, in
+// parallel over t, and kept in LDS; the sum over t for each d is cut into up to
+// four runs of consecutive t handled by different threads and added in run
+// order.  Every reduction is a fixed tree, so the result depends only on the
+// partials.
+constexpr int P2_THREADS = 256;
+constexpr int P2_MAXT = 2048;  // flash_plan never makes more splits
+
+__device__ __forceinline__ float block_reduce(float v, float* tmp, bool is_max) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float o = __shfl_xor(v, off, 64);
+    v = is_max ? fmaxf(v, o) : v + o;
+  }
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) tmp[wave] = v;
+  __syncthreads();
+  float r = tmp[0];
+#pragma unroll
+  for (int w = 1; w < P2_THREADS / 64; ++w) r = is_max ? fmaxf(r, tmp[w]) : r + tmp[w];
+  __syncthreads();
+  return r;
+}
+
+__global__ __launch_bounds__(P2_THREADS) void flash_phase2(const float* __restrict__ part,
+                                                           w4_half* __restrict__ out,
+                                                           const int T, const int D) {
+  __shared__ float wts[P2_MAXT];
+  __shared__ float tmp[P2_THREADS / 64];
+  __shared__ float runs[3][256];
   const long long hq = blockIdx.x;
-  const float* hb = part + hq * T * (D + 2);
-  float M = -INFINITY;
-  for (int t = 0; t < T; ++t) M = fmaxf(M, hb[(long long)t * (D + 2)]);
+  const int stride = D + 2;
+  const float* hb = part + hq * T * stride;
+  float m = -INFINITY;
+  for (int t = threadIdx.x; t < T; t += P2_THREADS) m = fmaxf(m, hb[(long long)t * stride]);
+  const float M = block_reduce(m, tmp, true);
   float den = 0.0f;
-  for (int t = 0; t < T; ++t)
-    den += __expf(hb[(long long)t * (D + 2)] - M) * hb[(long long)t * (D + 2) + 1];
+  for (int t = threadIdx.x; t < T; t += P2_THREADS) {
+    const float w = __expf(hb[(long long)t * stride] - M);
+    wts[t] = w;
+    den += w * hb[(long long)t * stride + 1];
+  }
+  den = block_reduce(den, tmp, false);  // also orders the wts writes before the reads below
   const float inv = 1.0f / den;
-  for (int d = threadIdx.x; d < D; d += 128) {
+  const int dpad = (D + 63) & ~63;
+  if (dpad <= 256) {
+    const int nrun = P2_THREADS / dpad;  // 4, 2 or 1 runs of consecutive t
+    const int run = threadIdx.x / dpad, d = threadIdx.x - run * dpad;
+    const int per = (T + nrun - 1) / nrun;
+    const int ta = min(T, run * per), tb = min(T, ta + per);
     float acc = 0.0f;
-    for (int t = 0; t < T; ++t) {
-      const float* pb = hb + (long long)t * (D + 2);
-      acc += __expf(pb[0] - M) * pb[2 + d];
+    if (run < nrun && d < D) {
+#pragma unroll 4
+      for (int t = ta; t < tb; ++t) acc += wts[t] * hb[(long long)t * stride + 2 + d];
     }
-    const _Float16 h = (_Float16)(acc * inv);
-    out[hq * D + d] = __builtin_bit_cast(uint16_t, h);
+    if (run > 0 && run < nrun && d < D) runs[run - 1][d] = acc;
+    __syncthreads();
+    if (run == 0 && d < D) {
+      for (int r = 1; r < nrun; ++r) acc += runs[r - 1][d];
+      const _Float16 h = (_Float16)(acc * inv);
+      out[hq * D + d] = __builtin_bit_cast(uint16_t, h);
+    }
+  } else {
+    for (int d = threadIdx.x; d < D; d += P2_THREADS) {
+      float acc = 0.0f;
+#pragma unroll 4
+      for (int t = 0; t < T; ++t) acc += wts[t] * hb[(long long)t * stride + 2 + d];
+      const _Float16 h = (_Float16)(acc * inv);
+      out[hq * D + d] = __builtin_bit_cast(uint16_t, h);
+    }
   }
 }
 
 // ---- host side -------------------------------------------------------------
 
-struct FlashPlan {
-  int split_len, nsplit;
-};
-
-static FlashPlan plan_of(const FlashArgs& a) {
+FlashPlan flash_plan(const FlashArgs& a) {
   // Enough workgroups to fill 256 CUs several times over, but splits no shorter
   // than one tile; a longer split writes fewer partials.
   const int tiles = (a.S + FL_TILE - 1) / FL_TILE;
@@ -327,7 +373,7 @@ static FlashPlan plan_of(const FlashArgs& a) {
 }
 
 size_t flash_scratch_floats(const FlashArgs& a) {
-  const FlashPlan p = plan_of(a);
+  const FlashPlan p = flash_plan(a);
   return (size_t)a.H * a.group * p.nsplit * (a.D + 2);
 }
 
@@ -370,8 +416,14 @@ static hipError_t go_heads(const FlashArgs& a, const FlashPlan& pl, float* scrat
 }
 
 hipError_t launch_flash(const FlashArgs& a, float* scratch, hipStream_t s) {
-  const FlashPlan pl = plan_of(a);
+  const FlashPlan pl = flash_plan(a);
+  if (pl.nsplit > P2_MAXT) return hipErrorInvalidValue;
   hipError_t e;
+  if (try_flash_mfma(a, pl, scratch, s, &e)) {
+    if (e != hipSuccess) return e;
+    flash_phase2<<<(unsigned)(a.H * a.group), P2_THREADS, 0, s>>>(scratch, a.out, pl.nsplit, a.D);
+    return hipGetLastError();
+  }
   const bool al16 = (((uintptr_t)a.k | (uintptr_t)a.v) & 15) == 0;
   if (a.kind == KIND_F16) {
     if (a.D % 8 == 0 && al16) e = go_heads<KIND_F16, 8, true>(a, pl, scratch, s);
@@ -384,7 +436,7 @@ hipError_t launch_flash(const FlashArgs& a, float* scratch, hipStream_t s) {
     else e = go_heads<KIND_F8, 8, false>(a, pl, scratch, s);
   }
   if (e != hipSuccess) return e;
-  flash_phase2<<<(unsigned)(a.H * a.group), 128, 0, s>>>(scratch, a.out, pl.nsplit, a.D);
+  flash_phase2<<<(unsigned)(a.H * a.group), P2_THREADS, 0, s>>>(scratch, a.out, pl.nsplit, a.D);
   return hipGetLastError();
 }
 

@@ -1,0 +1,391 @@
+// Split-S flash-decode phase 1 on the matrix cores, head dimension 128.
+//
+// A wave walks tiles of 32 cache positions.  Per tile:
+//   scores   S[t][h] = sum_d K[t][d] q[h][d]  -- two groups of four
+//            v_mfma_f32_16x16x32_f16, A = K rows (lane: position l%16, 32 of the
+//            128 d), B = the query heads of the pass (up to 16 share one slab
+//            read).  A lane's A operand is exactly what it loads: one dwordx4 of
+//            packed codes (W4), two of bytes (FP8), four of halves (FP16).
+//   softmax  the result leaves lane (h = l%16, r = l/16) with the scores of head
+//            h at positions {4r..4r+3, 16+4r..16+4r+3} of the tile; running
+//            max / rescale are per lane, the tile max needs two lane exchanges.
+//   output   O^T[d][h] += sum_t V[t][d] p[t][h]  -- eight MFMAs contracting over
+//            the 32 positions, B = the probabilities straight from the score
+//            registers (FP16), A = V transposed: lane (i = l%16, r = l/16) loads
+//            the 8 cache elements d = 8i..8i+7 of its 8 positions (one packed
+//            word, 8 bytes, or 16 bytes each), expands them and regroups the
+//            8x8 block with v_perm so that MFMA e takes element e of every
+//            position.  A ninth MFMA with A = 1 accumulates the denominators.
+// Dequantisation is the bit-exact register step of dq.cuh (the k_out / v_out
+// hooks store those values); only the order of the FP32 sums differs from the
+// vector kernel.  The four waves of a workgroup interleave tiles of one split
+// and merge their (m, l, O) through LDS in wave order, so a split yields one
+// partial and every sum has a fixed order: paged and contiguous caches give the
+// same bytes.
+#include "dq.cuh"
+#include "kernels.h"
+
+namespace w4k {
+
+constexpr int FM_D = 128;
+constexpr int FM_TILE = 32;   // positions per wave tile
+constexpr int FM_WAVES = 4;
+constexpr int FM_DEPTH = 2;   // tiles in flight per wave
+constexpr int FM_HEADS = 16;  // query heads per pass
+
+// What one lane fetches for one tile, before expansion.
+template <int KIND>
+struct TileRaw;
+template <>
+struct TileRaw<KIND_W4> {
+  u4 k[2];
+  uint32_t ks[2], kz[2];
+  uint32_t v[8], vs[8], vz[8];
+};
+template <>
+struct TileRaw<KIND_F16> {
+  u4 k[2][4];
+  u4 v[8];
+};
+template <>
+struct TileRaw<KIND_F8> {
+  u4 k[2][2];
+  uint32_t ks[2];
+  u2 v[8];
+  uint32_t vs[8];
+};
+
+// Position of element e (0..7) of an expanded 8-element block: register and half.
+template <int KIND>
+__device__ __forceinline__ constexpr int reg_of(int e) {
+  return KIND == KIND_W4 ? (e & 3) : KIND == KIND_F16 ? (e >> 1) : 2 * (e >> 2) + (e & 1);
+}
+template <int KIND>
+__device__ __forceinline__ constexpr int half_of(int e) {
+  return KIND == KIND_W4 ? (e >> 2) : KIND == KIND_F16 ? (e & 1) : ((e & 3) >> 1);
+}
+// Logical element held by (register p, half hf) of an expanded block.
+template <int KIND>
+__device__ __forceinline__ constexpr int elem_of(int p, int hf) {
+  return KIND == KIND_W4 ? p + 4 * hf : KIND == KIND_F16 ? 2 * p + hf : 4 * (p >> 1) + (p & 1) + 2 * hf;
+}
+
+__device__ __forceinline__ h8 pack8(const h2 v[4]) {
+  return h8{v[0][0], v[0][1], v[1][0], v[1][1], v[2][0], v[2][1], v[3][0], v[3][1]};
+}
+
+// PAGED: 0 contiguous slabs, 1 pages of a multiple of 16 rows (both halves of a
+// tile lie in one page each), 2 any page size.
+template <int KIND, bool HOOK, int PAGED, bool ASYM>
+__global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashArgs a,
+                                                                   const int qh0,
+                                                                   const int split_len,
+                                                                   float* __restrict__ part) {
+  constexpr int LDW = FM_D + 4;  // floats per (wave, head) merge row: O[128], l, m
+  __shared__ float wo[FM_WAVES][FM_HEADS * LDW];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c16 = lane & 15, q4 = lane >> 4;
+  const int split = blockIdx.x, slab = blockIdx.y, nsplit = gridDim.x;
+  const int nh = min(FM_HEADS, a.group - qh0);
+  const float inv_sqrt_d = 1.0f / sqrtf((float)FM_D);
+  const int G = a.G, wg = words(a.G);
+  const int gk = KIND == KIND_F16 ? 0 : (32 * q4) / a.gs;  // group of this lane's K elements
+  const int gv = KIND == KIND_F16 ? 0 : (8 * c16) / a.gs;  // ... and of its V elements
+
+  const int* bt = nullptr;
+  long long rows0;
+  if (PAGED) {
+    bt = a.bt + (long long)(slab / a.Hkv) * a.bt_stride;
+    rows0 = (long long)(slab % a.Hkv) * a.pool_rows;
+  } else {
+    rows0 = (long long)slab * a.S;
+  }
+  uint32_t slab_sk = 0, slab_sv = 0;
+  if (KIND == KIND_F8 && a.scale_mode == 1) slab_sk = a.s_k[slab], slab_sv = a.s_v[slab];
+
+  const int s0 = split * split_len;
+  const int s1 = min(a.S, s0 + split_len);
+  const long long hook_base = (long long)slab * a.S;
+  const bool hook_k = HOOK && a.k_out && qh0 == 0, hook_v = HOOK && a.v_out && qh0 == 0;
+
+  // Query operands: lane (head c16, k-block q4) of MFMA c holds
+  // q[head][32 q4 + 8 c + elem_of(p, hf)].
+  h8 qop[4];
+  {
+    const uint16_t* qp = a.q + ((long long)slab * a.group + qh0 + min(c16, nh - 1)) * FM_D + 32 * q4;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      h2 t[4];
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const uint32_t lo = qp[8 * c + elem_of<KIND>(p, 0)], hi = qp[8 * c + elem_of<KIND>(p, 1)];
+        t[p] = as_h2(c16 < nh ? (lo | (hi << 16)) : 0u);
+      }
+      qop[c] = pack8(t);
+    }
+  }
+
+  // physical cache row of logical position t (t < S)
+  auto phys = [&](int t, int pg_lo, long long base_lo, int pg_hi, long long base_hi, bool hi) -> long long {
+    if (PAGED == 0) return rows0 + t;
+    if (PAGED == 1) return (hi ? base_hi : base_lo) + (t - (hi ? pg_hi : pg_lo) * a.page);
+    const int pg = t / a.page;
+    return rows0 + (long long)bt[pg] * a.page + (t - pg * a.page);
+  };
+
+  auto fetch = [&](TileRaw<KIND>& raw, int t0) {
+    int pg_lo = 0, pg_hi = 0;
+    long long base_lo = 0, base_hi = 0;
+    if (PAGED == 1) {  // wave-uniform lookups: the page of each 16-position half
+      pg_lo = min(t0, s1 - 1) / a.page;
+      pg_hi = min(t0 + 16, s1 - 1) / a.page;
+      base_lo = rows0 + (long long)bt[pg_lo] * a.page;
+      base_hi = rows0 + (long long)bt[pg_hi] * a.page;
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int t = min(t0 + 16 * j + c16, s1 - 1);
+      const long long row = phys(t, pg_lo, base_lo, pg_hi, base_hi, j == 1);
+      if constexpr (KIND == KIND_W4) {
+        raw.k[j] = __builtin_nontemporal_load((const u4*)((const uint32_t*)a.k + row * 16 + 4 * q4));
+        raw.ks[j] = a.s_k[row * G + gk];
+        if (ASYM) raw.kz[j] = a.z_k[row * wg + (gk >> 3)];
+      } else if constexpr (KIND == KIND_F16) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          raw.k[j][c] = __builtin_nontemporal_load(
+              (const u4*)((const uint16_t*)a.k + row * FM_D + 32 * q4 + 8 * c));
+      } else {
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+          raw.k[j][c] = __builtin_nontemporal_load(
+              (const u4*)((const uint8_t*)a.k + row * FM_D + 32 * q4 + 16 * c));
+        raw.ks[j] = a.scale_mode == 0 ? (uint32_t)a.s_k[row * G + gk] : slab_sk;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int t = min(t0 + 16 * (k >> 2) + 4 * q4 + (k & 3), s1 - 1);
+      const long long row = phys(t, pg_lo, base_lo, pg_hi, base_hi, k >= 4);
+      if constexpr (KIND == KIND_W4) {
+        raw.v[k] = __builtin_nontemporal_load((const uint32_t*)a.v + row * 16 + c16);
+        raw.vs[k] = a.s_v[row * G + gv];
+        if (ASYM) raw.vz[k] = a.z_v[row * wg + (gv >> 3)];
+      } else if constexpr (KIND == KIND_F16) {
+        raw.v[k] = __builtin_nontemporal_load((const u4*)((const uint16_t*)a.v + row * FM_D + 8 * c16));
+      } else {
+        raw.v[k] = __builtin_nontemporal_load((const u2*)((const uint8_t*)a.v + row * FM_D + 8 * c16));
+        raw.vs[k] = a.scale_mode == 0 ? (uint32_t)a.s_v[row * G + gv] : slab_sv;
+      }
+    }
+  };
+
+  f4 o[8], lsum = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o[e] = f4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY;
+  const h8 ones = h8{1, 1, 1, 1, 1, 1, 1, 1};
+
+  auto store16 = [&](uint16_t* dst, const h2 nat[4]) {
+    *(u4*)dst = u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
+  };
+
+  auto compute = [&](const TileRaw<KIND>& raw, int t0) {
+    // ---- scores
+    f4 sc[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      sc[j] = f4{0.f, 0.f, 0.f, 0.f};
+      const int t = t0 + 16 * j + c16;
+      uint16_t* kdst = HOOK ? a.k_out + (hook_base + t) * FM_D + 32 * q4 : nullptr;
+      const bool kst = hook_k && t < s1;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        h2 d[4];
+        if constexpr (KIND == KIND_W4) {
+          const int z = ASYM ? (int)((raw.kz[j] >> (4 * (gk & 7))) & 0xFu) : 8;
+          dq_w4(raw.k[j][c], w4_group((uint16_t)raw.ks[j], z), d);
+          if (kst) {
+            h2 nat[4];
+            to_natural(d, nat);
+            store16(kdst + 8 * c, nat);
+          }
+        } else if constexpr (KIND == KIND_F16) {
+#pragma unroll
+          for (int p = 0; p < 4; ++p) d[p] = as_h2(raw.k[j][c][p]);
+          if (kst) store16(kdst + 8 * c, d);
+        } else {
+          const h2 s = splat_bits(raw.ks[j]);
+          dq_f8(raw.k[j][c >> 1][2 * (c & 1)], s, d);
+          dq_f8(raw.k[j][c >> 1][2 * (c & 1) + 1], s, d + 2);
+          if (kst) {
+            h2 nat[4];
+            to_natural_f8(d, nat);
+            to_natural_f8(d + 2, nat + 2);
+            store16(kdst + 8 * c, nat);
+          }
+        }
+        sc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pack8(d), qop[c], sc[j], 0, 0, 0);
+      }
+    }
+    // ---- online softmax for head c16 over this lane's 8 positions
+    float x[8];
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int t = t0 + 16 * (k >> 2) + 4 * q4 + (k & 3);
+      x[k] = t < s1 ? sc[k >> 2][k & 3] * inv_sqrt_d : -INFINITY;
+      tmax = fmaxf(tmax, x[k]);
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m_run, tmax);
+    const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+    if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {  // wave-uniform
+      const float alpha = __expf(m_run - m_use);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) o[e] *= alpha;
+      lsum *= alpha;
+    }
+    m_run = m_new;
+    h2 pr[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      pr[k] = h2{(_Float16)__expf(x[2 * k] - m_use), (_Float16)__expf(x[2 * k + 1] - m_use)};
+    const h8 pop = pack8(pr);
+    lsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pop, lsum, 0, 0, 0);
+    // ---- V: expand the 8 positions x 8 elements of this lane, regroup, accumulate
+    h2 vt[8][4];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int t = t0 + 16 * (k >> 2) + 4 * q4 + (k & 3);
+      const bool vst = hook_v && t < s1;
+      uint16_t* vdst = HOOK ? a.v_out + (hook_base + t) * FM_D + 8 * c16 : nullptr;
+      if constexpr (KIND == KIND_W4) {
+        const int z = ASYM ? (int)((raw.vz[k] >> (4 * (gv & 7))) & 0xFu) : 8;
+        dq_w4(raw.v[k], w4_group((uint16_t)raw.vs[k], z), vt[k]);
+        if (vst) {
+          h2 nat[4];
+          to_natural(vt[k], nat);
+          store16(vdst, nat);
+        }
+      } else if constexpr (KIND == KIND_F16) {
+#pragma unroll
+        for (int p = 0; p < 4; ++p) vt[k][p] = as_h2(raw.v[k][p]);
+        if (vst) store16(vdst, vt[k]);
+      } else {
+        const h2 s = splat_bits(raw.vs[k]);
+        dq_f8(raw.v[k][0], s, vt[k]);
+        dq_f8(raw.v[k][1], s, vt[k] + 2);
+        if (vst) {
+          h2 nat[4];
+          to_natural_f8(vt[k], nat);
+          to_natural_f8(vt[k] + 2, nat + 2);
+          store16(vdst, nat);
+        }
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      constexpr uint32_t LO = 0x05040100u, HI = 0x07060302u;
+      const int rg = reg_of<KIND>(e);
+      const uint32_t sel = half_of<KIND>(e) ? HI : LO;
+      h2 at[4];
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk)
+        at[kk] = as_h2(__builtin_amdgcn_perm(as_u32(vt[2 * kk + 1][rg]), as_u32(vt[2 * kk][rg]), sel));
+      o[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pack8(at), pop, o[e], 0, 0, 0);
+    }
+  };
+
+  // tiles of this wave: s0 + 32 * (wave + 4 * it)
+  const int nit = (s1 - s0 + FM_WAVES * FM_TILE - 1) / (FM_WAVES * FM_TILE);
+  auto tile_start = [&](int it) { return s0 + FM_TILE * (wave + FM_WAVES * it); };
+  TileRaw<KIND> ring[FM_DEPTH];
+#pragma unroll
+  for (int d = 0; d < FM_DEPTH; ++d) fetch(ring[d], tile_start(d));
+  for (int it0 = 0; it0 < nit; it0 += FM_DEPTH) {
+#pragma unroll
+    for (int d = 0; d < FM_DEPTH; ++d) {
+      const TileRaw<KIND> raw = ring[d];
+      fetch(ring[d], tile_start(it0 + d + FM_DEPTH));
+      compute(raw, tile_start(it0 + d));
+    }
+  }
+
+  // ---- merge the four waves in wave order: lane (head c16, q4) holds
+  // O[head][32 q4 + 8 r + e] in o[e][r]
+  float* mine = wo[wave] + c16 * LDW;
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) mine[32 * q4 + 8 * r + e] = o[e][r];
+  if (q4 == 0) {
+    mine[FM_D] = lsum[0];
+    mine[FM_D + 1] = m_run;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < nh * (FM_D + 1); i += FM_WAVES * 64) {
+    const int h = i / (FM_D + 1), j = i - h * (FM_D + 1);  // j < 128: O[j]; j == 128: l
+    float mw[FM_WAVES], M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < FM_WAVES; ++w) {
+      mw[w] = wo[w][h * LDW + FM_D + 1];
+      M = fmaxf(M, mw[w]);
+    }
+    float sum = 0.0f;
+#pragma unroll
+    for (int w = 0; w < FM_WAVES; ++w) sum += __expf(mw[w] - M) * wo[w][h * LDW + j];
+    float* dst = part + (((long long)slab * a.group + qh0 + h) * nsplit + split) * (FM_D + 2);
+    if (j < FM_D) {
+      dst[2 + j] = sum;
+    } else {
+      dst[1] = sum;
+      dst[0] = M;
+    }
+  }
+}
+
+template <int KIND, bool HOOK, int PAGED>
+static hipError_t go_asym(const FlashArgs& a, int qh0, const FlashPlan& pl, float* part,
+                          hipStream_t s) {
+  const dim3 grid((unsigned)pl.nsplit, (unsigned)a.H);
+  if (KIND == KIND_W4 && !a.symmetric)
+    flash_mfma_phase1<KIND, HOOK, PAGED, true><<<grid, FM_WAVES * 64, 0, s>>>(a, qh0, pl.split_len, part);
+  else
+    flash_mfma_phase1<KIND, HOOK, PAGED, false><<<grid, FM_WAVES * 64, 0, s>>>(a, qh0, pl.split_len, part);
+  return hipGetLastError();
+}
+
+template <int KIND>
+static hipError_t go_kind(const FlashArgs& a, int qh0, const FlashPlan& pl, float* part,
+                          hipStream_t s) {
+  const bool hook = a.k_out || a.v_out;
+  if constexpr (KIND == KIND_W4) {
+    if (a.bt) {
+      if (a.page % 16 == 0)
+        return hook ? go_asym<KIND, true, 1>(a, qh0, pl, part, s) : go_asym<KIND, false, 1>(a, qh0, pl, part, s);
+      return hook ? go_asym<KIND, true, 2>(a, qh0, pl, part, s) : go_asym<KIND, false, 2>(a, qh0, pl, part, s);
+    }
+  }
+  return hook ? go_asym<KIND, true, 0>(a, qh0, pl, part, s) : go_asym<KIND, false, 0>(a, qh0, pl, part, s);
+}
+
+bool try_flash_mfma(const FlashArgs& a, const FlashPlan& pl, float* part, hipStream_t s,
+                    hipError_t* err) {
+  if (a.D != FM_D) return false;
+  if (a.kind != KIND_F16 && a.gs % 32) return false;  // one group per lane's 32 K elements
+  if ((((uintptr_t)a.k | (uintptr_t)a.v) & 15) || (((uintptr_t)a.k_out | (uintptr_t)a.v_out) & 15))
+    return false;
+  if (pl.split_len % (FM_WAVES * FM_TILE)) return false;
+  *err = hipSuccess;
+  for (int qh0 = 0; qh0 < a.group && *err == hipSuccess; qh0 += FM_HEADS) {
+    if (a.kind == KIND_F16) *err = go_kind<KIND_F16>(a, qh0, pl, part, s);
+    else if (a.kind == KIND_W4) *err = go_kind<KIND_W4>(a, qh0, pl, part, s);
+    else *err = go_kind<KIND_F8>(a, qh0, pl, part, s);
+  }
+  return true;
+}
+
+}  // namespace w4k

@@ -62,6 +62,18 @@ struct FlashArgs {
   w4_half* k_out;
   w4_half* v_out;
 };
+enum { KIND_F16 = 0, KIND_W4 = 1, KIND_F8 = 2 };  // FlashArgs::kind
+
+// Split of the sequence over workgroups (shared by both phase-1 kernels).
+struct FlashPlan {
+  int split_len, nsplit;
+};
+FlashPlan flash_plan(const FlashArgs& a);
+// flash_mfma.hip: matrix-core phase 1 for D = 128; false when the arguments need
+// the general kernel (nothing is launched then).
+bool try_flash_mfma(const FlashArgs& a, const FlashPlan& pl, float* part, hipStream_t s,
+                    hipError_t* err);
+
 // Floats of scratch the split-S partials need for these arguments.
 size_t flash_scratch_floats(const FlashArgs& a);
 hipError_t launch_flash(const FlashArgs& a, float* scratch, hipStream_t s);

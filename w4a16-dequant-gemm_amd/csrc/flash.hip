@@ -359,10 +359,13 @@ __global__ __launch_bounds__(P2_THREADS) void flash_phase2(const float* __restri
 // ---- host side -------------------------------------------------------------
 
 FlashPlan flash_plan(const FlashArgs& a) {
-  // Enough workgroups to fill 256 CUs several times over, but splits no shorter
-  // than one tile; a longer split writes fewer partials.
+  // Enough workgroups to fill 256 CUs, but splits no shorter than one tile; a
+  // longer split writes fewer partials.  Measured at 64 slabs x 32768 positions:
+  // the matrix-core kernel is fastest with 2 workgroups per CU (512 in all; 256,
+  // 768, 1024, 2048 and 4096 were slower), the vector kernel with 8.
   const int tiles = (a.S + FL_TILE - 1) / FL_TILE;
-  int want = (8 * 256 + a.H - 1) / a.H;  // splits per slab for ~2048 workgroups
+  const int per_cu = flash_mfma_applies(a) ? 2 : 8;
+  int want = (per_cu * 256 + a.H - 1) / a.H;  // splits per slab
   if (want < 1) want = 1;
   if (want > tiles) want = tiles;
   const int tiles_per = (tiles + want - 1) / want;

@@ -372,13 +372,16 @@ static hipError_t go_kind(const FlashArgs& a, int qh0, const FlashPlan& pl, floa
   return hook ? go_asym<KIND, true, 0>(a, qh0, pl, part, s) : go_asym<KIND, false, 0>(a, qh0, pl, part, s);
 }
 
-bool try_flash_mfma(const FlashArgs& a, const FlashPlan& pl, float* part, hipStream_t s,
-                    hipError_t* err) {
+bool flash_mfma_applies(const FlashArgs& a) {
   if (a.D != FM_D) return false;
   if (a.kind != KIND_F16 && a.gs % 32) return false;  // one group per lane's 32 K elements
-  if ((((uintptr_t)a.k | (uintptr_t)a.v) & 15) || (((uintptr_t)a.k_out | (uintptr_t)a.v_out) & 15))
-    return false;
-  if (pl.split_len % (FM_WAVES * FM_TILE)) return false;
+  return ((((uintptr_t)a.k | (uintptr_t)a.v) & 15) == 0) &&
+         ((((uintptr_t)a.k_out | (uintptr_t)a.v_out) & 15) == 0);
+}
+
+bool try_flash_mfma(const FlashArgs& a, const FlashPlan& pl, float* part, hipStream_t s,
+                    hipError_t* err) {
+  if (!flash_mfma_applies(a) || pl.split_len % (FM_WAVES * FM_TILE)) return false;
   *err = hipSuccess;
   for (int qh0 = 0; qh0 < a.group && *err == hipSuccess; qh0 += FM_HEADS) {
     if (a.kind == KIND_F16) *err = go_kind<KIND_F16>(a, qh0, pl, part, s);

@@ -69,8 +69,10 @@ struct FlashPlan {
   int split_len, nsplit;
 };
 FlashPlan flash_plan(const FlashArgs& a);
-// flash_mfma.hip: matrix-core phase 1 for D = 128; false when the arguments need
-// the general kernel (nothing is launched then).
+// flash_mfma.hip: whether the matrix-core phase 1 (D = 128) takes these arguments.
+bool flash_mfma_applies(const FlashArgs& a);
+// Launches it; false when the arguments need the general kernel (nothing is
+// launched then).
 bool try_flash_mfma(const FlashArgs& a, const FlashPlan& pl, float* part, hipStream_t s,
                     hipError_t* err);
 

@@ -313,57 +313,86 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_generic_kernel(
 
 // Fully unrolled form of the fast kernel for the shapes decode GEMMs have:
 // K = STEPS * 2048, one group per 32-k lane slice, whole workgroups of rows, no
-// hook.  Every load of a wave (activations first, then the STEPS * R weight
-// dwordx4 and their scales) is issued before anything is consumed, and the
+// hook.  Every load of a wave (activations first, then the scales, then the
+// STEPS * R weight dwordx4) is issued before anything is consumed, and the
 // waits are retired in that order.
-template <int MX, int MT, int R, int STEPS>
+template <int MX, int MT, int R, int STEPS, bool ASYM>
 __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_unrolled_kernel(
     const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M) {
-  __shared__ u4 xs[MT * STEPS * 256];
+  // One activation row: every lane fetches its own 32-k slices of x straight from
+  // L2 (no LDS, no barrier: 0.3 us at N = K = 4096).  More rows: staged once per
+  // workgroup in LDS.
+  constexpr bool XDIRECT = MT == 1;
+  __shared__ u4 xs[XDIRECT ? 1 : MT * STEPS * 256];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n0 = (blockIdx.x * SIMT_WAVES + wave) * R;
   const int m0 = blockIdx.y * MT;
   constexpr int K = STEPS * 2048, WPR = K / 8;
-  constexpr int XL = (MT * STEPS * 256) / (SIMT_WAVES * 64);
+  constexpr int XL = XDIRECT ? STEPS * 4 : (MT * STEPS * 256) / (SIMT_WAVES * 64);
   const int wg = MX ? 0 : words(p.G);
 
-  u4 xv[XL];
+  const u4* xsrc[XL];
 #pragma unroll
   for (int t = 0; t < XL; ++t) {
-    const int i = t * SIMT_WAVES * 64 + threadIdx.x;
-    const int m = i / (STEPS * 256), g8 = i % (STEPS * 256);
-    xv[t] = (m0 + m < M) ? *(const u4*)(x + (size_t)(m0 + m) * K + g8 * 8) : u4{0u, 0u, 0u, 0u};
+    if (XDIRECT) {
+      xsrc[t] = (const u4*)(x + (size_t)m0 * K + (t >> 2) * 2048 + lane * 32 + (t & 3) * 8);
+    } else {
+      const int i = t * SIMT_WAVES * 64 + threadIdx.x;
+      const int m = min(i / (STEPS * 256), M - 1 - m0), g8 = i % (STEPS * 256);
+      xsrc[t] = (const u4*)(x + (size_t)(m0 + m) * K + g8 * 8);  // rows past M: a valid row, never stored
+    }
   }
-  uint32_t sc[STEPS][R], zp[STEPS][R];
+  const uint16_t* ssrc[STEPS][R];
+  const uint32_t* zsrc[STEPS][R];
+  uint32_t zsh[STEPS];
+  const u4* qsrc[STEPS][R];
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    const int k0 = s * 2048 + lane * 32;
+    const int g = MX ? (k0 >> 5) : k0 / p.gs;
+    zsh[s] = 4u * (uint32_t)(g & 7);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const size_t n = (size_t)(n0 + r);
+      ssrc[s][r] = MX ? (const uint16_t*)((const uint8_t*)p.scales + n * p.B + g)
+                      : (const uint16_t*)p.scales + n * p.G + g;
+      zsrc[s][r] = ASYM ? p.zeros + n * wg + (g >> 3) : nullptr;
+      qsrc[s][r] = (const u4*)(p.q + n * WPR + s * 256 + lane * 4);
+    }
+  }
+  u4 xv[XL];
+  uint32_t sc[STEPS][R], zw[STEPS][R];
   u4 qw[STEPS][R];
+#pragma unroll
+  for (int t = 0; t < XL; ++t) xv[t] = *xsrc[t];
 #pragma unroll
   for (int s = 0; s < STEPS; ++s)
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const int n = n0 + r, k0 = s * 2048 + lane * 32;
-      if (MX) {
-        sc[s][r] = ((const uint8_t*)p.scales)[(size_t)n * p.B + (k0 >> 5)];
-        zp[s][r] = 0;
-      } else {
-        const int g = k0 / p.gs;
-        sc[s][r] = ((const uint16_t*)p.scales)[(size_t)n * p.G + g];
-        zp[s][r] = (uint32_t)zero_point(p, n, g, wg);
-      }
+      sc[s][r] = MX ? (uint32_t) * (const uint8_t*)ssrc[s][r] : (uint32_t)*ssrc[s][r];
+      zw[s][r] = ASYM ? *zsrc[s][r] : 0u;
     }
 #pragma unroll
   for (int s = 0; s < STEPS; ++s)
 #pragma unroll
-    for (int r = 0; r < R; ++r)
-      qw[s][r] = __builtin_nontemporal_load(
-          (const u4*)(p.q + (size_t)(n0 + r) * WPR + s * 256 + lane * 4));
+    for (int r = 0; r < R; ++r) qw[s][r] = __builtin_nontemporal_load(qsrc[s][r]);
+  // With LDS staging every request goes out before the barrier.  With direct
+  // activations the compiler is left free to weave address arithmetic between
+  // the requests and to start on the first rows while the last request is still
+  // being formed: measured 3.8 us against 4.2 us with all requests forced up
+  // front (N = K = 4096) -- at kernel start the 16 waves of a CU all compete for
+  // the vector ALUs, so what matters is how few instructions precede each request.
+  if (!XDIRECT) __builtin_amdgcn_sched_barrier(0);
+  if (!XDIRECT) {
 #pragma unroll
-  for (int t = 0; t < XL; ++t) {
-    const int i = t * SIMT_WAVES * 64 + threadIdx.x;
-    const int m = i / (STEPS * 256), g8 = i % (STEPS * 256);
-    const int slot = (g8 & ~255) + (g8 & 3) * 64 + ((g8 & 255) >> 2);
-    xs[m * STEPS * 256 + slot] = MX ? xv[t] : pair_strided(xv[t]);
+    for (int t = 0; t < XL; ++t) {
+      const int i = t * SIMT_WAVES * 64 + threadIdx.x;
+      const int m = i / (STEPS * 256), g8 = i % (STEPS * 256);
+      const int slot = (g8 & ~255) + (g8 & 3) * 64 + ((g8 & 255) >> 2);
+      xs[m * STEPS * 256 + slot] = MX ? xv[t] : pair_strided(xv[t]);
+    }
+    __syncthreads();
   }
-  __syncthreads();
 
   float acc[R][MT];
 #pragma unroll
@@ -376,10 +405,14 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_unrolled_kernel(
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) xr[m][j] = xs[m * STEPS * 256 + s * 256 + j * 64 + lane];
+      for (int j = 0; j < 4; ++j) {
+        if (XDIRECT) xr[m][j] = MX ? xv[s * 4 + j] : pair_strided(xv[s * 4 + j]);
+        else xr[m][j] = xs[m * STEPS * 256 + s * 256 + j * 64 + lane];
+      }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const W4Group grp = w4_group((uint16_t)sc[s][r], (int)zp[s][r]);
+      const W4Group grp =
+          w4_group((uint16_t)sc[s][r], ASYM ? (int)((zw[s][r] >> zsh[s]) & 0xFu) : 8);
       const float mxs = mx_scale(sc[s][r]);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -421,7 +454,10 @@ template <int MX, int MT, int STEPS>
 static hipError_t launch_unrolled(const WView& v, const w4_half* x, w4_half* c, int M,
                                   hipStream_t s) {
   const dim3 grid((unsigned)(v.N / (SIMT_WAVES * SIMT_R)), (unsigned)((M + MT - 1) / MT));
-  simt_unrolled_kernel<MX, MT, SIMT_R, STEPS><<<grid, SIMT_WAVES * 64, 0, s>>>(v, x, c, M);
+  if (!MX && !v.symmetric)
+    simt_unrolled_kernel<MX, MT, SIMT_R, STEPS, true><<<grid, SIMT_WAVES * 64, 0, s>>>(v, x, c, M);
+  else
+    simt_unrolled_kernel<MX, MT, SIMT_R, STEPS, false><<<grid, SIMT_WAVES * 64, 0, s>>>(v, x, c, M);
   return hipGetLastError();
 }
 

@@ -24,6 +24,8 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         # shapes of the unrolled decode kernel (K = 2048, 4096, 8192; whole workgroups of rows)
         # shapes of the large-M matrix-core kernel (ragged M and N tiles, gs % 32 != 0)
         (300, 200, 512, 128), (96, 136, 256, 48), (257, 128, 192, 64),
+        # odd and even numbers of k-steps, ragged M and N tiles
+        (130, 260, 384, 32), (128, 256, 256, 64), (200, 300, 1024, 128), (97, 72, 128, 96),
         (2, 64, 2048, 64), (1, 128, 8192, 128), (4, 72, 4096, 32), (3, 40, 6144, 128), (8, 16, 2048, 128)]
 TOL, CROSS = 1e-3, 2e-3  # rel L2 vs the FP64 oracle; between two gated paths
 

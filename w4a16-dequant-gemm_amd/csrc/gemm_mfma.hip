@@ -151,8 +151,8 @@ __global__ __launch_bounds__(MMA_WAVES * 64) void mfma_skinny_kernel(
 
 // ---- decode-batch kernel (2 <= M < 96, 16-byte aligned rows) ----------------------
 // A workgroup of 8 waves owns 16 * NT weight rows and 16 * MT activation rows;
-// the waves split K in runs of CH chunks of 128 k and combine through LDS in a
-// fixed order.  A round of a wave issues every load it needs before consuming
+// wave w owns the w-th eighth of the 128-k chunks of K, walks it CH chunks at a
+// time, and the waves combine through LDS in wave order.  A round of a wave issues every load it needs before consuming
 // any: scales and zero-points, then the activations (B operands, 64 contiguous
 // bytes per lane and chunk, served by L2), then the packed weights (A operands,
 // the only HBM stream) -- loads return in issue order, so the weights arrive
@@ -188,7 +188,10 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void mfma_decode_kernel(
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f4{0.f, 0.f, 0.f, 0.f};
 
-  for (int c0 = wave * CH; c0 < nchunks; c0 += DEC_WAVES * CH) {
+  // wave w owns the chunks [w * cpw, (w + 1) * cpw), walked CH at a time
+  const int cpw = (nchunks + DEC_WAVES - 1) / DEC_WAVES;
+  const int cend = min(nchunks, (wave + 1) * cpw);
+  for (int c0 = wave * cpw; c0 < cend; c0 += CH) {
     int kl[CH];
     bool ok[CH];
     uint32_t sc[CH][NT][NS], zw[CH][NT][NS], zsh[CH][NS];
@@ -196,7 +199,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void mfma_decode_kernel(
 #pragma unroll
     for (int i = 0; i < CH; ++i) {
       const int k = (c0 + i) * MMA_CHUNK + b * 32;
-      ok[i] = k < p.K;
+      ok[i] = c0 + i < cend && k < p.K;
       kl[i] = ok[i] ? k : 0;
     }
 #pragma unroll
@@ -292,6 +295,102 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void mfma_decode_kernel(
   }
 }
 
+// Unrolled form of the kernel above for the common decode shapes: M <= 16,
+// K = 1024 * CH (one round: wave w owns k in [128 CH w, 128 CH (w + 1))), whole
+// row tiles, one group per lane slice, no hook.  No bounds logic at all, so few
+// instructions stand between the start of a wave and its requests.
+template <int FMT, int CH, bool POW2>
+__global__ __launch_bounds__(DEC_WAVES * 64) void mfma_decode_unrolled_kernel(
+    const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
+    const int gs_shift) {
+  constexpr bool MX = FMT == 2;
+  constexpr int K = 1024 * CH, WPR = K / 8;
+  __shared__ f4 red[DEC_WAVES][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, b = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int kw = wave * (128 * CH) + 32 * b;  // first k of this lane
+  const size_t n = (size_t)(n0 + r);
+  const uint16_t* xr = x + (size_t)min(r, M - 1) * K + kw;
+  const uint32_t* qr = p.q + n * WPR + (kw >> 3);
+
+  u4 xv[CH][4], qw[CH];
+  uint32_t sc[CH], zw[CH], zsh[CH];
+#pragma unroll
+  for (int i = 0; i < CH; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xv[i][j] = *(const u4*)(xr + 128 * i + 8 * j);
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int k = kw + 128 * i;
+    const int g = MX ? (k >> 5) : POW2 ? (k >> gs_shift) : k / p.gs;
+    zsh[i] = 4u * (uint32_t)(g & 7);
+    if (MX) {
+      sc[i] = ((const uint8_t*)p.scales)[n * p.B + g];
+    } else {
+      sc[i] = ((const uint16_t*)p.scales)[n * p.G + g];
+      if (FMT == 1) zw[i] = p.zeros[n * words(p.G) + (g >> 3)];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < CH; ++i) qw[i] = __builtin_nontemporal_load((const u4*)(qr + 16 * i));
+
+  f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < CH; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      h2 d[4], nat[4];
+      if (MX) {
+        dq_mx(qw[i][j], mx_scale(sc[i]), nat);
+      } else {
+        const int z = FMT == 1 ? (int)((zw[i] >> zsh[i]) & 0xFu) : 8;
+        dq_w4(qw[i][j], w4_group((uint16_t)sc[i], z), d);
+        to_natural(d, nat);
+      }
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(pack_h8(nat), __builtin_bit_cast(h8, xv[i][j]),
+                                                   acc, 0, 0, 0);
+    }
+  red[wave][lane] = acc;
+  __syncthreads();
+  if (wave == 0) {
+    f4 s = red[0][lane];
+#pragma unroll
+    for (int w = 1; w < DEC_WAVES; ++w) s += red[w][lane];
+    if (r < M) {  // lane: activation row r, weight rows n0 + 4 b .. + 3
+      uint16_t hv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const _Float16 h = (_Float16)s[i];
+        hv[i] = __builtin_bit_cast(uint16_t, h);
+      }
+      *(u2*)(c + (size_t)r * p.N + n0 + 4 * b) =
+          u2{hv[0] | ((uint32_t)hv[1] << 16), hv[2] | ((uint32_t)hv[3] << 16)};
+    }
+  }
+}
+
+template <int FMT>
+static bool try_decode_unrolled(const WView& v, const w4_half* x, w4_half* c, int M,
+                                hipStream_t s, w4_half* w_out, hipError_t* err) {
+  if (w_out || M > 16 || v.N % 16 || ((uintptr_t)c & 7)) return false;
+  if (!v.mx && v.gs % 32) return false;
+  if (v.K != 2048 && v.K != 4096) return false;
+  const bool pow2 = !v.mx && (v.gs & (v.gs - 1)) == 0;
+  const int sh = pow2 ? __builtin_ctz((unsigned)v.gs) : 0;
+  const unsigned grid = (unsigned)(v.N / 16);
+#define W4_GO(CH, P2) \
+  mfma_decode_unrolled_kernel<FMT, CH, P2><<<grid, DEC_WAVES * 64, 0, s>>>(v, x, c, M, sh)
+  if (v.K == 4096) {
+    if (pow2) W4_GO(4, true); else W4_GO(4, false);
+  } else {
+    if (pow2) W4_GO(2, true); else W4_GO(2, false);
+  }
+#undef W4_GO
+  *err = hipGetLastError();
+  return true;
+}
+
 // One chunk per wave and round, one row tile per workgroup: the fastest of the
 // (NT, CH) combinations measured for M <= 16 (N = 4096 .. 14336, K = 4096 .. 11008).
 template <int FMT, int MT>
@@ -325,7 +424,7 @@ static hipError_t launch_decode(const WView& v, const w4_half* x, w4_half* c, in
 // instead of once per wave; each wave streams its own 16 weight rows straight
 // into registers as MFMA A operands, DEPTH steps ahead.  Steps past the end of a
 // slice, and k past K, fetch from clamped addresses and stage zeros.
-template <int FMT, int MT, int NW, int KW, int DEPTH, bool HOOK, bool GS32>
+template <int FMT, int MT, int NW, int KW, int CPS, int DEPTH, bool HOOK, bool GS32>
 __global__ __launch_bounds__(512) void mfma_stream_kernel(
     const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
     w4_half* __restrict__ w_out, const int gs_shift) {
@@ -333,8 +432,10 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
   constexpr bool MX = FMT == 2;
   constexpr int NS = (MX || GS32) ? 1 : 4;
   constexpr int ROWS = 16 * MT;
-  constexpr int LD = MMA_CHUNK + 8;           // halves per staged row: 16-lane reads hit 16 bank groups
-  constexpr int PIECES = KW * ROWS * 16;      // 16-byte pieces staged per step
+  constexpr int BK = MMA_CHUNK * CPS;         // k per step
+  constexpr int SEGS = BK / 8;                // 16-byte pieces per staged row
+  constexpr int LD = BK + 8;                  // halves per staged row: 16-lane reads hit 16 bank groups
+  constexpr int PIECES = KW * ROWS * SEGS;    // pieces staged per step
   constexpr int XP = (PIECES + 511) / 512;    // ... per thread
   constexpr int XS_HALVES = 2 * KW * ROWS * LD;
   constexpr int RED_HALVES = KW * NW * MT * 64 * 8;
@@ -345,8 +446,8 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
   const int n0 = blockIdx.x * (16 * NW) + 16 * nw, m0 = blockIdx.y * ROWS;
   const int wpr = p.K >> 3;
   const int wg = MX ? 0 : words(p.G);
-  const int nchunks = (p.K + MMA_CHUNK - 1) / MMA_CHUNK;
-  const int cpk = (nchunks + KW - 1) / KW;                  // chunks per K slice
+  const int nblocks = (p.K + BK - 1) / BK;
+  const int cpk = (nblocks + KW - 1) / KW;                  // steps per K slice
   const int steps = (cpk + DEPTH - 1) / DEPTH * DEPTH;
   const bool hook = HOOK && blockIdx.y == 0 && n0 + r < p.N;
   const size_t nrow = (size_t)min(n0 + r, p.N - 1);
@@ -358,45 +459,53 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
 #pragma unroll
   for (int i = 0; i < XP; ++i) {
     const int id = i * 512 + tid;
-    const int pk = (id / (ROWS * 16)) % KW, prow = (id >> 4) % ROWS, seg = (id & 15) * 8;
+    const int pk = (id / (ROWS * SEGS)) % KW, prow = (id / SEGS) % ROWS, seg = (id % SEGS) * 8;
     xsrc[i] = x + (size_t)min(m0 + prow, M - 1) * p.K;
-    xk0[i] = pk * cpk * MMA_CHUNK + seg;
+    xk0[i] = pk * cpk * BK + seg;
     xdst[i] = pk * (ROWS * LD) + prow * LD + seg;
   }
 
   struct Slot {
-    u4 q;
-    uint32_t sc[NS], zw[NS];
+    u4 q[CPS];
+    uint32_t sc[CPS][NS], zw[CPS][NS];
     u4 xg[XP];
   };
   Slot ring[DEPTH];
   auto group_of = [&](int kk) { return MX ? (kk >> 5) : gs_shift >= 0 ? (kk >> gs_shift) : kk / p.gs; };
-  auto lane_k = [&](int s) { return (kw * cpk + s) * MMA_CHUNK + b * 32; };
+  auto lane_k = [&](int s, int ch) { return (kw * cpk + s) * BK + ch * MMA_CHUNK + b * 32; };
   auto fetch = [&](Slot& sl, int s) {
-    const int k = lane_k(s);
-    const int kc = (s < cpk && k < p.K) ? k : 0;
 #pragma unroll
-    for (int e = 0; e < NS; ++e) {
-      const int g = group_of(kc + 8 * e);
-      if (MX) {
-        sl.sc[e] = ((const uint8_t*)p.scales)[nrow * p.B + g];
-      } else {
-        sl.sc[e] = ((const uint16_t*)p.scales)[nrow * p.G + g];
-        if (FMT == 1) sl.zw[e] = p.zeros[nrow * wg + (g >> 3)];
+    for (int ch = 0; ch < CPS; ++ch) {
+      const int k = lane_k(s, ch);
+      const int kc = (s < cpk && k < p.K) ? k : 0;
+#pragma unroll
+      for (int e = 0; e < NS; ++e) {
+        const int g = group_of(kc + 8 * e);
+        if (MX) {
+          sl.sc[ch][e] = ((const uint8_t*)p.scales)[nrow * p.B + g];
+        } else {
+          sl.sc[ch][e] = ((const uint16_t*)p.scales)[nrow * p.G + g];
+          if (FMT == 1) sl.zw[ch][e] = p.zeros[nrow * wg + (g >> 3)];
+        }
       }
     }
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
-      const int kx = xk0[i] + s * MMA_CHUNK;
+      const int kx = xk0[i] + s * BK;
       sl.xg[i] = *(const u4*)(xsrc[i] + ((s < cpk && kx < p.K) ? kx : 0));
     }
-    sl.q = __builtin_nontemporal_load((const u4*)(qrow + (kc >> 3)));
+#pragma unroll
+    for (int ch = 0; ch < CPS; ++ch) {
+      const int k = lane_k(s, ch);
+      const int kc = (s < cpk && k < p.K) ? k : 0;
+      sl.q[ch] = __builtin_nontemporal_load((const u4*)(qrow + (kc >> 3)));
+    }
   };
   auto stage = [&](const Slot& sl, int buf, int s) {
     uint16_t* base = smem + buf * (KW * ROWS * LD);
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
-      const int kx = xk0[i] + s * MMA_CHUNK;
+      const int kx = xk0[i] + s * BK;
       const bool okx = s < cpk && kx < p.K;
       if (XP * 512 == PIECES || i * 512 + tid < PIECES)
         *(u4*)(base + xdst[i]) = okx ? sl.xg[i] : u4{0u, 0u, 0u, 0u};
@@ -415,36 +524,43 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       const int s = s0 + d, buf = s & 1;
-      const u4 q = ring[d].q;
-      uint32_t sc[NS], zw[NS];
+      u4 q[CPS];
+      uint32_t sc[CPS][NS], zw[CPS][NS];
 #pragma unroll
-      for (int e = 0; e < NS; ++e) sc[e] = ring[d].sc[e], zw[e] = ring[d].zw[e];
+      for (int ch = 0; ch < CPS; ++ch) {
+        q[ch] = ring[d].q[ch];
+#pragma unroll
+        for (int e = 0; e < NS; ++e) sc[ch][e] = ring[d].sc[ch][e], zw[ch][e] = ring[d].zw[ch][e];
+      }
       fetch(ring[d], s + DEPTH);  // slot d: weights copied out, activations staged one step ago
       stage(ring[(d + 1) % DEPTH], buf ^ 1, s + 1);
-      const int k = lane_k(s);
-      const bool okw = s < cpk && k < p.K;
-      const int kc = okw ? k : 0;
       const uint16_t* xb = smem + buf * (KW * ROWS * LD) + kw * (ROWS * LD) + r * LD + b * 32;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        h2 dq[4], nat[4];
-        const int e = NS == 1 ? 0 : j;
-        if (MX) {
-          dq_mx(q[j], mx_scale(sc[0]), nat);
-        } else {
-          int z = 8;
-          if (FMT == 1) z = (int)((zw[e] >> (4 * (group_of(kc + 8 * e) & 7))) & 0xFu);
-          dq_w4(q[j], w4_group((uint16_t)sc[e], z), dq);
-          to_natural(dq, nat);
-        }
-        if (hook && okw)
-          *(u4*)(w_out + nrow * p.K + kc + 8 * j) =
-              u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
-        const h8 a = pack_h8(nat);
+      for (int ch = 0; ch < CPS; ++ch) {
+        const int k = lane_k(s, ch);
+        const bool okw = s < cpk && k < p.K;
+        const int kc = okw ? k : 0;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-          const h8 bx = *(const h8*)(xb + mt * 16 * LD + j * 8);
-          acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bx, acc[mt], 0, 0, 0);
+        for (int j = 0; j < 4; ++j) {
+          h2 dq[4], nat[4];
+          const int e = NS == 1 ? 0 : j;
+          if (MX) {
+            dq_mx(q[ch][j], mx_scale(sc[ch][0]), nat);
+          } else {
+            int z = 8;
+            if (FMT == 1) z = (int)((zw[ch][e] >> (4 * (group_of(kc + 8 * e) & 7))) & 0xFu);
+            dq_w4(q[ch][j], w4_group((uint16_t)sc[ch][e], z), dq);
+            to_natural(dq, nat);
+          }
+          if (hook && okw)
+            *(u4*)(w_out + nrow * p.K + kc + 8 * j) =
+                u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
+          const h8 a = pack_h8(nat);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            const h8 bx = *(const h8*)(xb + mt * 16 * LD + ch * MMA_CHUNK + j * 8);
+            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bx, acc[mt], 0, 0, 0);
+          }
         }
       }
       __syncthreads();
@@ -481,7 +597,7 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
   }
 }
 
-// 4 row tiles x 2 K slices, 4 steps in flight (deeper rings measured slower).
+// 4 row tiles x 2 K slices (deeper rings and more chunks per step measured slower).
 
 template <int FMT, int MT>
 static hipError_t launch_stream_mt(const WView& v, const w4_half* x, w4_half* c, int M,
@@ -489,11 +605,14 @@ static hipError_t launch_stream_mt(const WView& v, const w4_half* x, w4_half* c,
   const bool gs32 = v.mx || v.gs % 32 == 0;
   int gs_shift = -1;
   if (!v.mx && (v.gs & (v.gs - 1)) == 0) gs_shift = __builtin_ctz((unsigned)v.gs);
-  constexpr int NW = 4, KW = 2, DEPTH = 4;
+  constexpr int NW = 4, KW = 2;
+  // two chunks per step, two steps in flight; MT = 4 fills the LDS with one chunk per step
+  constexpr int CPS = MT == 4 ? 1 : 2;
+  constexpr int DEPTH = MT == 4 ? 4 : 2;
   const dim3 grid((unsigned)((v.N + 16 * NW - 1) / (16 * NW)), (unsigned)((M + 16 * MT - 1) / (16 * MT)));
-  const int cpk = ((v.K + MMA_CHUNK - 1) / MMA_CHUNK + KW - 1) / KW;
+  const int cpk = ((v.K + MMA_CHUNK * CPS - 1) / (MMA_CHUNK * CPS) + KW - 1) / KW;
 #define W4_GO(D, HOOK, GS) \
-  mfma_stream_kernel<FMT, MT, NW, KW, D, HOOK, GS><<<grid, 512, 0, s>>>(v, x, c, M, w_out, gs_shift)
+  mfma_stream_kernel<FMT, MT, NW, KW, CPS, D, HOOK, GS><<<grid, 512, 0, s>>>(v, x, c, M, w_out, gs_shift)
   if (w_out) {
     if (gs32) W4_GO(1, true, true); else W4_GO(1, true, false);
   } else if (!gs32) {
@@ -774,6 +893,11 @@ static hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M
     // Measured on N = 4096 .. 14336, K = 4096 .. 11008: the K-split kernel wins for
     // M <= 16 unless N is large enough to give the streaming kernel a full grid.
     const bool ksplit = M <= 8 || (M <= 16 && v.N < 8192);
+    if (ksplit &&
+        (MX ? try_decode_unrolled<2>(v, x, c, M, s, w_out, &terr)
+            : v.symmetric ? try_decode_unrolled<0>(v, x, c, M, s, w_out, &terr)
+                          : try_decode_unrolled<1>(v, x, c, M, s, w_out, &terr)))
+      return terr;
     if (ksplit) {
       if (MX) return launch_decode<2>(v, x, c, M, s, w_out);
       return v.symmetric ? launch_decode<0>(v, x, c, M, s, w_out)

@@ -316,9 +316,10 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_generic_kernel(
 // hook.  Every load of a wave (activations first, then the scales, then the
 // STEPS * R weight dwordx4) is issued before anything is consumed, and the
 // waits are retired in that order.
-template <int MX, int MT, int R, int STEPS, bool ASYM>
+template <int MX, int MT, int R, int STEPS, bool ASYM, bool POW2>
 __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_unrolled_kernel(
-    const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M) {
+    const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
+    const int gs_shift) {
   // One activation row: every lane fetches its own 32-k slices of x straight from
   // L2 (no LDS, no barrier: 0.3 us at N = K = 4096).  More rows: staged once per
   // workgroup in LDS.
@@ -349,7 +350,7 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_unrolled_kernel(
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
     const int k0 = s * 2048 + lane * 32;
-    const int g = MX ? (k0 >> 5) : k0 / p.gs;
+    const int g = MX ? (k0 >> 5) : POW2 ? (k0 >> gs_shift) : k0 / p.gs;
     zsh[s] = 4u * (uint32_t)(g & 7);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -454,10 +455,16 @@ template <int MX, int MT, int STEPS>
 static hipError_t launch_unrolled(const WView& v, const w4_half* x, w4_half* c, int M,
                                   hipStream_t s) {
   const dim3 grid((unsigned)(v.N / (SIMT_WAVES * SIMT_R)), (unsigned)((M + MT - 1) / MT));
-  if (!MX && !v.symmetric)
-    simt_unrolled_kernel<MX, MT, SIMT_R, STEPS, true><<<grid, SIMT_WAVES * 64, 0, s>>>(v, x, c, M);
-  else
-    simt_unrolled_kernel<MX, MT, SIMT_R, STEPS, false><<<grid, SIMT_WAVES * 64, 0, s>>>(v, x, c, M);
+  const bool pow2 = !MX && (v.gs & (v.gs - 1)) == 0;  // group index by shift instead of division
+  const int sh = pow2 ? __builtin_ctz((unsigned)v.gs) : 0;
+#define W4_GO(ASYM, POW2) \
+  simt_unrolled_kernel<MX, MT, SIMT_R, STEPS, ASYM, POW2><<<grid, SIMT_WAVES * 64, 0, s>>>(v, x, c, M, sh)
+  if (!MX && !v.symmetric) {
+    if (pow2) W4_GO(true, true); else W4_GO(true, false);
+  } else {
+    if (pow2) W4_GO(false, true); else W4_GO(false, false);
+  }
+#undef W4_GO
   return hipGetLastError();
 }
 

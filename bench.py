@@ -27,12 +27,12 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 PREWARM_LAUNCHES = 2000
 # HBM bytes one launch of the headline kernel moves, from rocprofv3 --pmc runs of
-# `python3 bench.py --extras none --steps 50 --warmup 5`: FETCH_SIZE 4291.5 and
+# `python3 bench.py --extras none --steps 50 --warmup 5`: FETCH_SIZE 4287.5 and
 # WRITE_SIZE 16.0 per dispatch, scaled by what the same counters read for the
 # 1 GiB stream_copy kernel of this file's yardstick (FETCH_SIZE 524298 and
-# WRITE_SIZE 1048593 for 1048576 KiB each way, i.e. factors 2.0 and 1.0):
-# 8583 KiB fetched + 16 KiB written, against 8 667 136 algorithmic bytes.
-HEADLINE_TRAFFIC_BYTES = int((4291.5 * 2.0 + 16.0 * 1.0) * 1024)
+# WRITE_SIZE 1048591 for 1048576 KiB each way, i.e. factors 2.0 and 1.0):
+# 8575 KiB fetched + 16 KiB written, against 8 667 136 algorithmic bytes.
+HEADLINE_TRAFFIC_BYTES = int((4287.5 * 2.0 + 16.0 * 1.0) * 1024)
 
 
 def _pkg():

@@ -69,6 +69,7 @@ struct DeviceKVF8 {
   const __half* s_v;
 };
 
+constexpr int KV_MAX_S = 4096;   // kvattention.cuh:36
 constexpr int KV_MAX_D = 512;    // kvattention.cuh:37
 constexpr int FLASH_TILE = 256;  // kvflash.cuh:35
 
@@ -188,6 +189,22 @@ inline void attention_fp16_flash(const __half* q, const __half* k16, const __hal
                                  __half* out, int H, int S, int D, hipStream_t stream = 0) {
   detail::raise(w4_attention_fp16_flash(detail::h(q), detail::h(k16), detail::h(v16),
                                         detail::h(out), H, S, D, stream));
+}
+
+// The single-pass entry points of kvattention.cuh:226-249.  There is one
+// attention kernel family here, so they run the split-S path; the sequence
+// bound of the reference's shared-memory score buffer is kept so that callers
+// see the same rejections.
+inline void attention_fp16(const __half* q, const __half* k16, const __half* v16, __half* out,
+                           int H, int S, int D, hipStream_t stream = 0) {
+  if (S > KV_MAX_S) throw std::invalid_argument("kv fp16: S exceeds the shared-memory bound");
+  attention_fp16_flash(q, k16, v16, out, H, S, D, stream);
+}
+inline void attention_w4(const DeviceKVW4& p, const __half* q, __half* out,
+                         hipStream_t stream = 0, __half* k_out = nullptr,
+                         __half* v_out = nullptr) {
+  if (p.S > KV_MAX_S) throw std::invalid_argument("kv: S exceeds the shared-memory bound");
+  attention_w4_flash(p, q, out, stream, k_out, v_out);
 }
 
 // kvflash.cuh:572-590

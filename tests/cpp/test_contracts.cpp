@@ -100,6 +100,10 @@ int main() {
     t.throws_invalid([&] { attention_w4_flash_gqa(v, 4, P, P); }, "kv flash gqa view");
     t.throws_invalid([&] { attention_w4_flash_paged(v, BT, 16, 1 << 20, P, P); }, "kv paged view");
   }
+  t.throws_invalid([&] { attention_w4(withk([](auto& v) { v.S = KV_MAX_S + 1; }), P, P); }, "kv single-pass S bound");
+  t.throws_invalid([&] { attention_w4(okv, nullptr, P); }, "kv single-pass q null");
+  t.throws_invalid([&] { attention_fp16(P, P, P, P, 1, KV_MAX_S + 1, 64); }, "kv fp16 single-pass S bound");
+  t.throws_invalid([&] { attention_fp16(P, P, nullptr, P, 1, 64, 64); }, "kv fp16 single-pass null");
   t.throws_invalid([&] { attention_w4_flash(okv, nullptr, P); }, "kv flash q null");
   t.throws_invalid([&] { attention_w4_flash(okv, P, nullptr); }, "kv flash out null");
   t.throws_invalid([&] { attention_w4_flash_gqa(okv, 0, P, P); }, "kv flash group=0");

@@ -180,6 +180,13 @@ std::vector<__half> w4_flash_gates(Checks& t, const kv::KVCacheW4& c, const std:
   const auto of = o16.get();
   oracle_gate(t, of, ref, "FP16 flash vs FP64 reference");
   t.expect(cross(o, of, ref) <= 2e-3, "W4 flash vs FP16 flash");
+  if (c.S <= KV_MAX_S) {  // the single-pass entry points (kvattention.cuh:226-249) accept this length
+    Dev<__half> o1((size_t)c.H * c.D), o2((size_t)c.H * c.D);
+    attention_w4(d.view, qd.p, o1.p);
+    attention_fp16(qd.p, k16.p, v16.p, o2.p, c.H, c.S, c.D);
+    oracle_gate(t, o1.get(), ref, "W4 single-pass entry vs FP64 reference");
+    t.expect(cross(o1.get(), o2.get(), ref) <= 2e-3, "W4 vs FP16 single-pass entries");
+  }
   return o;
 }
 

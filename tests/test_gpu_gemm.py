@@ -26,7 +26,13 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         (300, 200, 512, 128), (96, 136, 256, 48), (257, 128, 192, 64),
         # odd and even numbers of k-steps, ragged M and N tiles
         (130, 260, 384, 32), (128, 256, 256, 64), (200, 300, 1024, 128), (97, 72, 128, 96),
-        (2, 64, 2048, 64), (1, 128, 8192, 128), (4, 72, 4096, 32), (3, 40, 6144, 128), (8, 16, 2048, 128)]
+        (2, 64, 2048, 64), (1, 128, 8192, 128), (4, 72, 4096, 32), (3, 40, 6144, 128), (8, 16, 2048, 128),
+        # group sizes that are no multiple of 32 (a lane's 32-k slice spans several groups) on the
+        # unrolled and streaming kernels
+        (1, 64, 2048, 8), (2, 16, 4096, 48), (3, 24, 2048, 24), (12, 48, 2048, 40), (20, 64, 2048, 48),
+        (40, 32, 1024, 8),
+        # K % 8 == 0 but K % 32 != 0: whole words, rows of packed words not 16-byte aligned
+        (9, 64, 4104, 8), (40, 48, 1032, 24), (3, 32, 520, 8), (100, 40, 264, 16)]
 TOL, CROSS = 1e-3, 2e-3  # rel L2 vs the FP64 oracle; between two gated paths
 
 

@@ -160,7 +160,20 @@ __global__ __launch_bounds__(MMA_WAVES * 64) void mfma_skinny_kernel(
 // their activations zeroed, which keeps the round branch-free.
 constexpr int DEC_WAVES = 8;
 
-template <int FMT, int MT, int NT, int CH, bool HOOK, bool GS32>
+// The four packed words of a lane's 32-k slice starting at word w0 of a row of
+// wpr words: one dwordx4 when rows are 16-byte aligned (K % 32 == 0), else four
+// dword loads with the index clamped to the row (K % 8 == 0; words past K meet
+// zero activations).
+template <bool WVEC>
+__device__ __forceinline__ u4 load_words4(const uint32_t* __restrict__ row, int w0, int wpr) {
+  if (WVEC) return __builtin_nontemporal_load((const u4*)(row + w0));
+  u4 v;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) v[j] = __builtin_nontemporal_load(row + min(w0 + j, wpr - 1));
+  return v;
+}
+
+template <int FMT, int MT, int NT, int CH, bool HOOK, bool GS32, bool WVEC>
 __global__ __launch_bounds__(DEC_WAVES * 64) void mfma_decode_kernel(
     const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
     w4_half* __restrict__ w_out, const int gs_shift) {
@@ -203,11 +216,13 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void mfma_decode_kernel(
       kl[i] = ok[i] ? k : 0;
     }
 #pragma unroll
-    for (int i = 0; i < CH; ++i)
+    for (int i = 0; i < CH; ++i) {
+      int g4[4];
+      if (NS == 1) g4[0] = MX ? (kl[i] >> 5) : gs_shift >= 0 ? (kl[i] >> gs_shift) : kl[i] / p.gs;
+      else groups_of_slice(kl[i], p.gs, gs_shift, g4);
 #pragma unroll
       for (int e = 0; e < NS; ++e) {
-        const int kk = kl[i] + 8 * e;
-        const int g = MX ? (kk >> 5) : gs_shift >= 0 ? (kk >> gs_shift) : kk / p.gs;
+        const int g = g4[e];
         zsh[i][e] = 4u * (uint32_t)(g & 7);
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
@@ -219,17 +234,19 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void mfma_decode_kernel(
           }
         }
       }
+    }
 #pragma unroll
     for (int i = 0; i < CH; ++i)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) xv[i][mt][j] = *(const u4*)(xrow[mt] + kl[i] + 8 * j);
+        for (int j = 0; j < 4; ++j)
+          xv[i][mt][j] = *(const u4*)(xrow[mt] + ((WVEC || kl[i] + 8 * j < p.K) ? kl[i] + 8 * j : 0));
 #pragma unroll
     for (int i = 0; i < CH; ++i)
 #pragma unroll
       for (int t = 0; t < NT; ++t)
-        qw[i][t] = __builtin_nontemporal_load((const u4*)(p.q + nrow[t] * wpr + (kl[i] >> 3)));
+        qw[i][t] = load_words4<WVEC>(p.q + nrow[t] * wpr, kl[i] >> 3, wpr);
 
 #pragma unroll
     for (int i = 0; i < CH; ++i) {
@@ -237,7 +254,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void mfma_decode_kernel(
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          if (!ok[i]) xv[i][mt][j] = u4{0u, 0u, 0u, 0u};
+          if (!ok[i] || (!WVEC && kl[i] + 8 * j >= p.K)) xv[i][mt][j] = u4{0u, 0u, 0u, 0u};
 #pragma unroll
       for (int t = 0; t < NT; ++t)
 #pragma unroll
@@ -251,7 +268,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void mfma_decode_kernel(
             dq_w4(qw[i][t][j], w4_group((uint16_t)sc[i][t][e], z), d);
             to_natural(d, nat);
           }
-          if (hook && ok[i] && n0 + 16 * t + r < p.N)
+          if (hook && ok[i] && (WVEC || kl[i] + 8 * j < p.K) && n0 + 16 * t + r < p.N)
             *(u4*)(w_out + nrow[t] * p.K + kl[i] + 8 * j) =
                 u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
           const h8 a = pack_h8(nat);
@@ -395,13 +412,20 @@ static bool try_decode_unrolled(const WView& v, const w4_half* x, w4_half* c, in
 // (NT, CH) combinations measured for M <= 16 (N = 4096 .. 14336, K = 4096 .. 11008).
 template <int FMT, int MT>
 static hipError_t launch_decode_mt(const WView& v, const w4_half* x, w4_half* c, int M,
-                                   hipStream_t s, w4_half* w_out) {
+                                   hipStream_t s, w4_half* w_out, bool wvec) {
   const bool gs32 = v.mx || v.gs % 32 == 0;
   int gs_shift = -1;
   if (!v.mx && (v.gs & (v.gs - 1)) == 0) gs_shift = __builtin_ctz((unsigned)v.gs);
   const dim3 grid((unsigned)((v.N + 15) / 16), (unsigned)((M + 16 * MT - 1) / (16 * MT)));
-#define W4_GO(HOOK, GS) \
-  mfma_decode_kernel<FMT, MT, 1, 1, HOOK, GS><<<grid, DEC_WAVES * 64, 0, s>>>(v, x, c, M, w_out, gs_shift)
+#define W4_GO(HOOK, GS)                                                                       \
+  do {                                                                                        \
+    if (wvec)                                                                                 \
+      mfma_decode_kernel<FMT, MT, 1, 1, HOOK, GS, true>                                       \
+          <<<grid, DEC_WAVES * 64, 0, s>>>(v, x, c, M, w_out, gs_shift);                      \
+    else                                                                                      \
+      mfma_decode_kernel<FMT, MT, 1, 1, HOOK, GS, false>                                      \
+          <<<grid, DEC_WAVES * 64, 0, s>>>(v, x, c, M, w_out, gs_shift);                      \
+  } while (0)
   if (w_out) {
     if (gs32) W4_GO(true, true); else W4_GO(true, false);
   } else {
@@ -413,8 +437,8 @@ static hipError_t launch_decode_mt(const WView& v, const w4_half* x, w4_half* c,
 
 template <int FMT>
 static hipError_t launch_decode(const WView& v, const w4_half* x, w4_half* c, int M,
-                                hipStream_t s, w4_half* w_out) {
-  return launch_decode_mt<FMT, 1>(v, x, c, M, s, w_out);  // M <= 16
+                                hipStream_t s, w4_half* w_out, bool wvec) {
+  return launch_decode_mt<FMT, 1>(v, x, c, M, s, w_out, wvec);  // M <= 16
 }
 
 // ---- streaming decode-batch kernel --------------------------------------------------
@@ -424,7 +448,7 @@ static hipError_t launch_decode(const WView& v, const w4_half* x, w4_half* c, in
 // instead of once per wave; each wave streams its own 16 weight rows straight
 // into registers as MFMA A operands, DEPTH steps ahead.  Steps past the end of a
 // slice, and k past K, fetch from clamped addresses and stage zeros.
-template <int FMT, int MT, int NW, int KW, int CPS, int DEPTH, bool HOOK, bool GS32>
+template <int FMT, int MT, int NW, int KW, int CPS, int DEPTH, bool HOOK, bool GS32, bool WVEC>
 __global__ __launch_bounds__(512) void mfma_stream_kernel(
     const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
     w4_half* __restrict__ w_out, const int gs_shift) {
@@ -467,7 +491,7 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
 
   struct Slot {
     u4 q[CPS];
-    uint32_t sc[CPS][NS], zw[CPS][NS];
+    uint32_t sc[CPS][NS], zw[CPS][NS], zsh[CPS][NS];
     u4 xg[XP];
   };
   Slot ring[DEPTH];
@@ -478,14 +502,19 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
     for (int ch = 0; ch < CPS; ++ch) {
       const int k = lane_k(s, ch);
       const int kc = (s < cpk && k < p.K) ? k : 0;
+      int g[4];
+      if (NS == 1) g[0] = group_of(kc);
+      else groups_of_slice(kc, p.gs, gs_shift, g);
 #pragma unroll
       for (int e = 0; e < NS; ++e) {
-        const int g = group_of(kc + 8 * e);
         if (MX) {
-          sl.sc[ch][e] = ((const uint8_t*)p.scales)[nrow * p.B + g];
+          sl.sc[ch][e] = ((const uint8_t*)p.scales)[nrow * p.B + g[e]];
         } else {
-          sl.sc[ch][e] = ((const uint16_t*)p.scales)[nrow * p.G + g];
-          if (FMT == 1) sl.zw[ch][e] = p.zeros[nrow * wg + (g >> 3)];
+          sl.sc[ch][e] = ((const uint16_t*)p.scales)[nrow * p.G + g[e]];
+          if (FMT == 1) {
+            sl.zw[ch][e] = p.zeros[nrow * wg + (g[e] >> 3)];
+            sl.zsh[ch][e] = 4u * (uint32_t)(g[e] & 7);
+          }
         }
       }
     }
@@ -498,7 +527,7 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
     for (int ch = 0; ch < CPS; ++ch) {
       const int k = lane_k(s, ch);
       const int kc = (s < cpk && k < p.K) ? k : 0;
-      sl.q[ch] = __builtin_nontemporal_load((const u4*)(qrow + (kc >> 3)));
+      sl.q[ch] = load_words4<WVEC>(qrow, kc >> 3, wpr);
     }
   };
   auto stage = [&](const Slot& sl, int buf, int s) {
@@ -525,12 +554,13 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
     for (int d = 0; d < DEPTH; ++d) {
       const int s = s0 + d, buf = s & 1;
       u4 q[CPS];
-      uint32_t sc[CPS][NS], zw[CPS][NS];
+      uint32_t sc[CPS][NS], zw[CPS][NS], zsh[CPS][NS];
 #pragma unroll
       for (int ch = 0; ch < CPS; ++ch) {
         q[ch] = ring[d].q[ch];
 #pragma unroll
-        for (int e = 0; e < NS; ++e) sc[ch][e] = ring[d].sc[ch][e], zw[ch][e] = ring[d].zw[ch][e];
+        for (int e = 0; e < NS; ++e)
+          sc[ch][e] = ring[d].sc[ch][e], zw[ch][e] = ring[d].zw[ch][e], zsh[ch][e] = ring[d].zsh[ch][e];
       }
       fetch(ring[d], s + DEPTH);  // slot d: weights copied out, activations staged one step ago
       stage(ring[(d + 1) % DEPTH], buf ^ 1, s + 1);
@@ -548,11 +578,11 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
             dq_mx(q[ch][j], mx_scale(sc[ch][0]), nat);
           } else {
             int z = 8;
-            if (FMT == 1) z = (int)((zw[ch][e] >> (4 * (group_of(kc + 8 * e) & 7))) & 0xFu);
+            if (FMT == 1) z = (int)((zw[ch][e] >> zsh[ch][e]) & 0xFu);
             dq_w4(q[ch][j], w4_group((uint16_t)sc[ch][e], z), dq);
             to_natural(dq, nat);
           }
-          if (hook && okw)
+          if (hook && okw && (WVEC || kc + 8 * j < p.K))
             *(u4*)(w_out + nrow * p.K + kc + 8 * j) =
                 u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
           const h8 a = pack_h8(nat);
@@ -601,7 +631,7 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
 
 template <int FMT, int MT>
 static hipError_t launch_stream_mt(const WView& v, const w4_half* x, w4_half* c, int M,
-                                   hipStream_t s, w4_half* w_out) {
+                                   hipStream_t s, w4_half* w_out, bool wvec) {
   const bool gs32 = v.mx || v.gs % 32 == 0;
   int gs_shift = -1;
   if (!v.mx && (v.gs & (v.gs - 1)) == 0) gs_shift = __builtin_ctz((unsigned)v.gs);
@@ -611,16 +641,21 @@ static hipError_t launch_stream_mt(const WView& v, const w4_half* x, w4_half* c,
   constexpr int DEPTH = MT == 4 ? 4 : 2;
   const dim3 grid((unsigned)((v.N + 16 * NW - 1) / (16 * NW)), (unsigned)((M + 16 * MT - 1) / (16 * MT)));
   const int cpk = ((v.K + MMA_CHUNK * CPS - 1) / (MMA_CHUNK * CPS) + KW - 1) / KW;
-#define W4_GO(D, HOOK, GS) \
-  mfma_stream_kernel<FMT, MT, NW, KW, CPS, D, HOOK, GS><<<grid, 512, 0, s>>>(v, x, c, M, w_out, gs_shift)
+#define W4_GO(D, HOOK, GS)                                                                    \
+  do {                                                                                        \
+    if (wvec)                                                                                 \
+      mfma_stream_kernel<FMT, MT, NW, KW, CPS, D, HOOK, GS, true>                             \
+          <<<grid, 512, 0, s>>>(v, x, c, M, w_out, gs_shift);                                 \
+    else                                                                                      \
+      mfma_stream_kernel<FMT, MT, NW, KW, CPS, D, HOOK, GS, false>                            \
+          <<<grid, 512, 0, s>>>(v, x, c, M, w_out, gs_shift);                                 \
+  } while (0)
   if (w_out) {
     if (gs32) W4_GO(1, true, true); else W4_GO(1, true, false);
-  } else if (!gs32) {
-    W4_GO(1, false, false);
   } else if (cpk >= DEPTH) {
-    W4_GO(DEPTH, false, true);
+    if (gs32) W4_GO(DEPTH, false, true); else W4_GO(DEPTH, false, false);
   } else {
-    W4_GO(1, false, true);
+    if (gs32) W4_GO(1, false, true); else W4_GO(1, false, false);
   }
 #undef W4_GO
   return hipGetLastError();
@@ -628,10 +663,10 @@ static hipError_t launch_stream_mt(const WView& v, const w4_half* x, w4_half* c,
 
 template <int FMT>
 static hipError_t launch_stream(const WView& v, const w4_half* x, w4_half* c, int M,
-                                hipStream_t s, w4_half* w_out) {
-  if (M <= 16) return launch_stream_mt<FMT, 1>(v, x, c, M, s, w_out);
-  if (M <= 32) return launch_stream_mt<FMT, 2>(v, x, c, M, s, w_out);
-  return launch_stream_mt<FMT, 4>(v, x, c, M, s, w_out);
+                                hipStream_t s, w4_half* w_out, bool wvec) {
+  if (M <= 16) return launch_stream_mt<FMT, 1>(v, x, c, M, s, w_out, wvec);
+  if (M <= 32) return launch_stream_mt<FMT, 2>(v, x, c, M, s, w_out, wvec);
+  return launch_stream_mt<FMT, 4>(v, x, c, M, s, w_out, wvec);
 }
 
 // ---- large-M kernel -----------------------------------------------------------
@@ -887,25 +922,28 @@ static hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M
                              hipStream_t s, w4_half* w_out) {
   hipError_t terr = hipSuccess;
   if (try_tile<MX>(v, x, c, M, s, w_out, &terr)) return terr;
-  const bool aligned = (v.K % 32 == 0) && (((uintptr_t)v.q | (uintptr_t)x) & 15) == 0 &&
+  // Rows of packed words are 16-byte aligned when K % 32 == 0 (one dwordx4 per lane
+  // slice); K % 8 == 0 still gives whole words and 16-byte aligned activation rows.
+  const bool wvec = (v.K % 32 == 0) && (((uintptr_t)v.q) & 15) == 0;
+  const bool aligned = (v.K % 8 == 0) && (((uintptr_t)x) & 15) == 0 &&
                        (w_out == nullptr || ((uintptr_t)w_out & 15) == 0);
   if (aligned) {
     // Measured on N = 4096 .. 14336, K = 4096 .. 11008: the K-split kernel wins for
     // M <= 16 unless N is large enough to give the streaming kernel a full grid.
     const bool ksplit = M <= 8 || (M <= 16 && v.N < 8192);
-    if (ksplit &&
+    if (ksplit && wvec &&
         (MX ? try_decode_unrolled<2>(v, x, c, M, s, w_out, &terr)
             : v.symmetric ? try_decode_unrolled<0>(v, x, c, M, s, w_out, &terr)
                           : try_decode_unrolled<1>(v, x, c, M, s, w_out, &terr)))
       return terr;
     if (ksplit) {
-      if (MX) return launch_decode<2>(v, x, c, M, s, w_out);
-      return v.symmetric ? launch_decode<0>(v, x, c, M, s, w_out)
-                         : launch_decode<1>(v, x, c, M, s, w_out);
+      if (MX) return launch_decode<2>(v, x, c, M, s, w_out, wvec);
+      return v.symmetric ? launch_decode<0>(v, x, c, M, s, w_out, wvec)
+                         : launch_decode<1>(v, x, c, M, s, w_out, wvec);
     }
-    if (MX) return launch_stream<2>(v, x, c, M, s, w_out);
-    return v.symmetric ? launch_stream<0>(v, x, c, M, s, w_out)
-                       : launch_stream<1>(v, x, c, M, s, w_out);
+    if (MX) return launch_stream<2>(v, x, c, M, s, w_out, wvec);
+    return v.symmetric ? launch_stream<0>(v, x, c, M, s, w_out, wvec)
+                       : launch_stream<1>(v, x, c, M, s, w_out, wvec);
   }
   if (M <= 16) return launch_tiles<MX, 1>(v, x, c, M, s, w_out);
   if (M <= 32) return launch_tiles<MX, 2>(v, x, c, M, s, w_out);

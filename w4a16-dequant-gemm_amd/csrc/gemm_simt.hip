@@ -316,7 +316,7 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_generic_kernel(
 // hook.  Every load of a wave (activations first, then the scales, then the
 // STEPS * R weight dwordx4) is issued before anything is consumed, and the
 // waits are retired in that order.
-template <int MX, int MT, int R, int STEPS, bool ASYM, bool POW2>
+template <int MX, int MT, int R, int STEPS, bool ASYM, bool POW2, bool GS32>
 __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_unrolled_kernel(
     const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
     const int gs_shift) {
@@ -343,36 +343,45 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_unrolled_kernel(
       xsrc[t] = (const u4*)(x + (size_t)(m0 + m) * K + g8 * 8);  // rows past M: a valid row, never stored
     }
   }
-  const uint16_t* ssrc[STEPS][R];
-  const uint32_t* zsrc[STEPS][R];
-  uint32_t zsh[STEPS];
+  constexpr int NS = (MX || GS32) ? 1 : 4;  // group lookups per lane slice
+  const uint16_t* ssrc[STEPS][R][NS];
+  const uint32_t* zsrc[STEPS][R][NS];
+  uint32_t zsh[STEPS][NS];
   const u4* qsrc[STEPS][R];
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
     const int k0 = s * 2048 + lane * 32;
-    const int g = MX ? (k0 >> 5) : POW2 ? (k0 >> gs_shift) : k0 / p.gs;
-    zsh[s] = 4u * (uint32_t)(g & 7);
+    int g[4];
+    if (NS == 1) g[0] = MX ? (k0 >> 5) : POW2 ? (k0 >> gs_shift) : k0 / p.gs;
+    else groups_of_slice(k0, p.gs, gs_shift, g);
+#pragma unroll
+    for (int e = 0; e < NS; ++e) zsh[s][e] = 4u * (uint32_t)(g[e] & 7);
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const size_t n = (size_t)(n0 + r);
-      ssrc[s][r] = MX ? (const uint16_t*)((const uint8_t*)p.scales + n * p.B + g)
-                      : (const uint16_t*)p.scales + n * p.G + g;
-      zsrc[s][r] = ASYM ? p.zeros + n * wg + (g >> 3) : nullptr;
+#pragma unroll
+      for (int e = 0; e < NS; ++e) {
+        ssrc[s][r][e] = MX ? (const uint16_t*)((const uint8_t*)p.scales + n * p.B + g[e])
+                           : (const uint16_t*)p.scales + n * p.G + g[e];
+        zsrc[s][r][e] = ASYM ? p.zeros + n * wg + (g[e] >> 3) : nullptr;
+      }
       qsrc[s][r] = (const u4*)(p.q + n * WPR + s * 256 + lane * 4);
     }
   }
   u4 xv[XL];
-  uint32_t sc[STEPS][R], zw[STEPS][R];
+  uint32_t sc[STEPS][R][NS], zw[STEPS][R][NS];
   u4 qw[STEPS][R];
 #pragma unroll
   for (int t = 0; t < XL; ++t) xv[t] = *xsrc[t];
 #pragma unroll
   for (int s = 0; s < STEPS; ++s)
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      sc[s][r] = MX ? (uint32_t) * (const uint8_t*)ssrc[s][r] : (uint32_t)*ssrc[s][r];
-      zw[s][r] = ASYM ? *zsrc[s][r] : 0u;
-    }
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int e = 0; e < NS; ++e) {
+        sc[s][r][e] = MX ? (uint32_t) * (const uint8_t*)ssrc[s][r][e] : (uint32_t)*ssrc[s][r][e];
+        zw[s][r][e] = ASYM ? *zsrc[s][r][e] : 0u;
+      }
 #pragma unroll
   for (int s = 0; s < STEPS; ++s)
 #pragma unroll
@@ -412,14 +421,16 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_unrolled_kernel(
       }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const W4Group grp =
-          w4_group((uint16_t)sc[s][r], ASYM ? (int)((zw[s][r] >> zsh[s]) & 0xFu) : 8);
-      const float mxs = mx_scale(sc[s][r]);
+      const float mxs = mx_scale(sc[s][r][0]);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
+        const int e = NS == 1 ? 0 : j;
         h2 d[4];
-        if (MX) dq_mx(qw[s][r][j], mxs, d);
-        else dq_w4(qw[s][r][j], grp, d);
+        if (MX)
+          dq_mx(qw[s][r][j], mxs, d);
+        else
+          dq_w4(qw[s][r][j],
+                w4_group((uint16_t)sc[s][r][e], ASYM ? (int)((zw[s][r][e] >> zsh[s][e]) & 0xFu) : 8), d);
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
@@ -457,12 +468,16 @@ static hipError_t launch_unrolled(const WView& v, const w4_half* x, w4_half* c, 
   const dim3 grid((unsigned)(v.N / (SIMT_WAVES * SIMT_R)), (unsigned)((M + MT - 1) / MT));
   const bool pow2 = !MX && (v.gs & (v.gs - 1)) == 0;  // group index by shift instead of division
   const int sh = pow2 ? __builtin_ctz((unsigned)v.gs) : 0;
-#define W4_GO(ASYM, POW2) \
-  simt_unrolled_kernel<MX, MT, SIMT_R, STEPS, ASYM, POW2><<<grid, SIMT_WAVES * 64, 0, s>>>(v, x, c, M, sh)
-  if (!MX && !v.symmetric) {
-    if (pow2) W4_GO(true, true); else W4_GO(true, false);
+  const bool gs32 = MX || v.gs % 32 == 0;  // else a lane's 32-k slice spans several groups
+#define W4_GO(ASYM, POW2, GS32) \
+  simt_unrolled_kernel<MX, MT, SIMT_R, STEPS, ASYM, POW2, GS32> \
+      <<<grid, SIMT_WAVES * 64, 0, s>>>(v, x, c, M, pow2 ? sh : -1)
+  if (!gs32) {
+    if (!v.symmetric) W4_GO(true, false, false); else W4_GO(false, false, false);
+  } else if (!MX && !v.symmetric) {
+    if (pow2) W4_GO(true, true, true); else W4_GO(true, false, true);
   } else {
-    if (pow2) W4_GO(false, true); else W4_GO(false, false);
+    if (pow2) W4_GO(false, true, true); else W4_GO(false, false, true);
   }
 #undef W4_GO
   return hipGetLastError();
@@ -473,7 +488,6 @@ template <int MX, int MT>
 static bool try_unrolled(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                          w4_half* w_out, hipError_t* err) {
   if (w_out || v.K % 2048 || v.N % (SIMT_WAVES * SIMT_R)) return false;
-  if (!v.mx && v.gs % 32) return false;
   if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)c & 3)) return false;
   const int steps = v.K / 2048;
   if (steps * MT > 8) return false;  // LDS: MT * K halves, at most 32 KiB

@@ -331,10 +331,13 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void mfma_decode_unrolled_kernel(
   const uint16_t* xr = x + (size_t)min(r, M - 1) * K + kw;
   const uint32_t* qr = p.q + n * WPR + (kw >> 3);
 
-  u4 xv[CH][4], qw[CH];
+  // Activations are requested in two halves that share registers, so that enough
+  // workgroups fit on a CU for the whole grid to be resident at once.
+  constexpr int HALF = CH / 2;
+  u4 xv[HALF][4], qw[CH];
   uint32_t sc[CH], zw[CH], zsh[CH];
 #pragma unroll
-  for (int i = 0; i < CH; ++i)
+  for (int i = 0; i < HALF; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) xv[i][j] = *(const u4*)(xr + 128 * i + 8 * j);
 #pragma unroll
@@ -354,20 +357,32 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void mfma_decode_unrolled_kernel(
 
   f4 acc = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int i = 0; i < CH; ++i)
+  for (int half = 0; half < 2; ++half) {
+    if (half == 1) {
+      __builtin_amdgcn_sched_barrier(0);  // the second half reuses the registers of the first
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      h2 d[4], nat[4];
-      if (MX) {
-        dq_mx(qw[i][j], mx_scale(sc[i]), nat);
-      } else {
-        const int z = FMT == 1 ? (int)((zw[i] >> zsh[i]) & 0xFu) : 8;
-        dq_w4(qw[i][j], w4_group((uint16_t)sc[i], z), d);
-        to_natural(d, nat);
-      }
-      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(pack_h8(nat), __builtin_bit_cast(h8, xv[i][j]),
-                                                   acc, 0, 0, 0);
+      for (int i = 0; i < HALF; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) xv[i][j] = *(const u4*)(xr + 128 * (HALF + i) + 8 * j);
     }
+#pragma unroll
+    for (int ii = 0; ii < HALF; ++ii) {
+      const int i = half * HALF + ii;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        h2 d[4], nat[4];
+        if (MX) {
+          dq_mx(qw[i][j], mx_scale(sc[i]), nat);
+        } else {
+          const int z = FMT == 1 ? (int)((zw[i] >> zsh[i]) & 0xFu) : 8;
+          dq_w4(qw[i][j], w4_group((uint16_t)sc[i], z), d);
+          to_natural(d, nat);
+        }
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(pack_h8(nat), __builtin_bit_cast(h8, xv[ii][j]),
+                                                     acc, 0, 0, 0);
+      }
+    }
+  }
   red[wave][lane] = acc;
   __syncthreads();
   if (wave == 0) {

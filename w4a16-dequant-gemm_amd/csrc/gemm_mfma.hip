@@ -463,11 +463,16 @@ static hipError_t launch_decode(const WView& v, const w4_half* x, w4_half* c, in
 // instead of once per wave; each wave streams its own 16 weight rows straight
 // into registers as MFMA A operands, DEPTH steps ahead.  Steps past the end of a
 // slice, and k past K, fetch from clamped addresses and stage zeros.
-template <int FMT, int MT, int NW, int KW, int CPS, int DEPTH, bool HOOK, bool GS32, bool WVEC>
-__global__ __launch_bounds__(512) void mfma_stream_kernel(
+// LEAN: K is a whole number of steps per slice and of ring rounds, N a whole
+// number of workgroups, the group size a power of two: every bounds test and
+// its branch disappears from the loop (the kernel is bound by instruction issue).
+template <int FMT, int MT, int NW, int KW, int CPS, int DEPTH, bool HOOK, bool GS32, bool WVEC,
+          bool LEAN>
+__global__ __launch_bounds__(64 * NW * KW) void mfma_stream_kernel(
     const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
     w4_half* __restrict__ w_out, const int gs_shift) {
-  static_assert(NW * KW == 8, "8 waves");
+  constexpr int THREADS = 64 * NW * KW;
+  static_assert(!LEAN || (GS32 && WVEC), "lean form: one group per lane slice, aligned rows");
   constexpr bool MX = FMT == 2;
   constexpr int NS = (MX || GS32) ? 1 : 4;
   constexpr int ROWS = 16 * MT;
@@ -475,7 +480,7 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
   constexpr int SEGS = BK / 8;                // 16-byte pieces per staged row
   constexpr int LD = BK + 8;                  // halves per staged row: 16-lane reads hit 16 bank groups
   constexpr int PIECES = KW * ROWS * SEGS;    // pieces staged per step
-  constexpr int XP = (PIECES + 511) / 512;    // ... per thread
+  constexpr int XP = (PIECES + THREADS - 1) / THREADS;  // ... per thread
   constexpr int XS_HALVES = 2 * KW * ROWS * LD;
   constexpr int RED_HALVES = KW * NW * MT * 64 * 8;
   __shared__ __attribute__((aligned(16))) uint16_t smem[XS_HALVES > RED_HALVES ? XS_HALVES : RED_HALVES];
@@ -487,9 +492,9 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
   const int wg = MX ? 0 : words(p.G);
   const int nblocks = (p.K + BK - 1) / BK;
   const int cpk = (nblocks + KW - 1) / KW;                  // steps per K slice
-  const int steps = (cpk + DEPTH - 1) / DEPTH * DEPTH;
+  const int steps = LEAN ? cpk : (cpk + DEPTH - 1) / DEPTH * DEPTH;
   const bool hook = HOOK && blockIdx.y == 0 && n0 + r < p.N;
-  const size_t nrow = (size_t)min(n0 + r, p.N - 1);
+  const size_t nrow = LEAN ? (size_t)(n0 + r) : (size_t)min(n0 + r, p.N - 1);
   const uint32_t* qrow = p.q + nrow * wpr;
 
   // the pieces of x this thread stages every step
@@ -497,7 +502,7 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
   int xk0[XP], xdst[XP];     // first k of the piece at step 0; where it goes in a staging buffer
 #pragma unroll
   for (int i = 0; i < XP; ++i) {
-    const int id = i * 512 + tid;
+    const int id = i * THREADS + tid;
     const int pk = (id / (ROWS * SEGS)) % KW, prow = (id / SEGS) % ROWS, seg = (id % SEGS) * 8;
     xsrc[i] = x + (size_t)min(m0 + prow, M - 1) * p.K;
     xk0[i] = pk * cpk * BK + seg;
@@ -510,13 +515,16 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
     u4 xg[XP];
   };
   Slot ring[DEPTH];
-  auto group_of = [&](int kk) { return MX ? (kk >> 5) : gs_shift >= 0 ? (kk >> gs_shift) : kk / p.gs; };
+  auto group_of = [&](int kk) {
+    return MX ? (kk >> 5) : (LEAN || gs_shift >= 0) ? (kk >> gs_shift) : kk / p.gs;
+  };
   auto lane_k = [&](int s, int ch) { return (kw * cpk + s) * BK + ch * MMA_CHUNK + b * 32; };
   auto fetch = [&](Slot& sl, int s) {
+    if (LEAN) s = min(s, cpk - 1);  // the ring runs past the end of the slice: refetch the last step
 #pragma unroll
     for (int ch = 0; ch < CPS; ++ch) {
       const int k = lane_k(s, ch);
-      const int kc = (s < cpk && k < p.K) ? k : 0;
+      const int kc = (LEAN || (s < cpk && k < p.K)) ? k : 0;
       int g[4];
       if (NS == 1) g[0] = group_of(kc);
       else groups_of_slice(kc, p.gs, gs_shift, g);
@@ -536,12 +544,12 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
       const int kx = xk0[i] + s * BK;
-      sl.xg[i] = *(const u4*)(xsrc[i] + ((s < cpk && kx < p.K) ? kx : 0));
+      sl.xg[i] = *(const u4*)(xsrc[i] + ((LEAN || (s < cpk && kx < p.K)) ? kx : 0));
     }
 #pragma unroll
     for (int ch = 0; ch < CPS; ++ch) {
       const int k = lane_k(s, ch);
-      const int kc = (s < cpk && k < p.K) ? k : 0;
+      const int kc = (LEAN || (s < cpk && k < p.K)) ? k : 0;
       sl.q[ch] = load_words4<WVEC>(qrow, kc >> 3, wpr);
     }
   };
@@ -550,9 +558,11 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
       const int kx = xk0[i] + s * BK;
-      const bool okx = s < cpk && kx < p.K;
-      if (XP * 512 == PIECES || i * 512 + tid < PIECES)
-        *(u4*)(base + xdst[i]) = okx ? sl.xg[i] : u4{0u, 0u, 0u, 0u};
+      const bool okx = LEAN || (s < cpk && kx < p.K);
+      // W4: staged in the (k, k+4) pairing the expansion step produces, so the
+      // weights need no re-pairing on their way into the MFMA
+      if (XP * THREADS == PIECES || i * THREADS + tid < PIECES)
+        *(u4*)(base + xdst[i]) = okx ? (MX ? sl.xg[i] : pair_strided(sl.xg[i])) : u4{0u, 0u, 0u, 0u};
     }
   };
 
@@ -583,24 +593,31 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
 #pragma unroll
       for (int ch = 0; ch < CPS; ++ch) {
         const int k = lane_k(s, ch);
-        const bool okw = s < cpk && k < p.K;
+        const bool okw = LEAN || (s < cpk && k < p.K);
         const int kc = okw ? k : 0;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          h2 dq[4], nat[4];
+          h2 dq[4];  // MX: natural pairs; W4: (k, k+4) pairs, like the staged activations
           const int e = NS == 1 ? 0 : j;
           if (MX) {
-            dq_mx(q[ch][j], mx_scale(sc[ch][0]), nat);
+            dq_mx(q[ch][j], mx_scale(sc[ch][0]), dq);
           } else {
             int z = 8;
             if (FMT == 1) z = (int)((zw[ch][e] >> zsh[ch][e]) & 0xFu);
             dq_w4(q[ch][j], w4_group((uint16_t)sc[ch][e], z), dq);
-            to_natural(dq, nat);
           }
-          if (hook && okw && (WVEC || kc + 8 * j < p.K))
+          if (hook && okw && (WVEC || kc + 8 * j < p.K)) {
+            h2 nat[4];
+            if (MX) {
+#pragma unroll
+              for (int t = 0; t < 4; ++t) nat[t] = dq[t];
+            } else {
+              to_natural(dq, nat);
+            }
             *(u4*)(w_out + nrow * p.K + kc + 8 * j) =
                 u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
-          const h8 a = pack_h8(nat);
+          }
+          const h8 a = pack_h8(dq);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) {
             const h8 bx = *(const h8*)(xb + mt * 16 * LD + ch * MMA_CHUNK + j * 8);
@@ -617,7 +634,7 @@ __global__ __launch_bounds__(512) void mfma_stream_kernel(
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) red[(kw * (NW * MT) + nw * MT + mt) * 64 + lane] = acc[mt];
   __syncthreads();
-  for (int tile = wave; tile < NW * MT; tile += 8) {
+  for (int tile = wave; tile < NW * MT; tile += NW * KW) {
     f4 sum = red[tile * 64 + lane];
 #pragma unroll
     for (int w = 1; w < KW; ++w) sum += red[(w * (NW * MT) + tile) * 64 + lane];
@@ -650,7 +667,7 @@ static hipError_t launch_stream_mt(const WView& v, const w4_half* x, w4_half* c,
   const bool gs32 = v.mx || v.gs % 32 == 0;
   int gs_shift = -1;
   if (!v.mx && (v.gs & (v.gs - 1)) == 0) gs_shift = __builtin_ctz((unsigned)v.gs);
-  constexpr int NW = 4, KW = 2;
+  constexpr int NW = 4, KW = 2;  // 16 waves (KW = 4) measured slower
   // two chunks per step, two steps in flight; MT = 4 fills the LDS with one chunk per step
   constexpr int CPS = MT == 4 ? 1 : 2;
   constexpr int DEPTH = MT == 4 ? 4 : 2;
@@ -659,13 +676,24 @@ static hipError_t launch_stream_mt(const WView& v, const w4_half* x, w4_half* c,
 #define W4_GO(D, HOOK, GS)                                                                    \
   do {                                                                                        \
     if (wvec)                                                                                 \
-      mfma_stream_kernel<FMT, MT, NW, KW, CPS, D, HOOK, GS, true>                             \
-          <<<grid, 512, 0, s>>>(v, x, c, M, w_out, gs_shift);                                 \
+      mfma_stream_kernel<FMT, MT, NW, KW, CPS, D, HOOK, GS, true, false>                      \
+          <<<grid, 64 * NW * KW, 0, s>>>(v, x, c, M, w_out, gs_shift);                                 \
     else                                                                                      \
-      mfma_stream_kernel<FMT, MT, NW, KW, CPS, D, HOOK, GS, false>                            \
-          <<<grid, 512, 0, s>>>(v, x, c, M, w_out, gs_shift);                                 \
+      mfma_stream_kernel<FMT, MT, NW, KW, CPS, D, HOOK, GS, false, false>                     \
+          <<<grid, 64 * NW * KW, 0, s>>>(v, x, c, M, w_out, gs_shift);                                 \
   } while (0)
-  if (w_out) {
+  // the lean form: whole steps, whole ring rounds, whole workgroups, shift for the group index.
+  // Measured at N = 11008, K = 4096: 23.7 vs 25.6 us with four activation tiles (M = 64), but
+  // 18.4 vs 15.2 us with one (M = 16) and 19.8 vs 18.4 us with two, so only MT = 4 takes it.
+  const bool lean = MT == 4 && wvec && gs32 && (v.mx || gs_shift >= 0) && v.K % (MMA_CHUNK * CPS * KW) == 0 &&
+                    v.N % (16 * NW) == 0;
+  if (lean && w_out) {
+    mfma_stream_kernel<FMT, MT, NW, KW, CPS, 1, true, true, true, true>
+        <<<grid, 64 * NW * KW, 0, s>>>(v, x, c, M, w_out, gs_shift);
+  } else if (lean && cpk % DEPTH == 0) {
+    mfma_stream_kernel<FMT, MT, NW, KW, CPS, DEPTH, false, true, true, true>
+        <<<grid, 64 * NW * KW, 0, s>>>(v, x, c, M, w_out, gs_shift);
+  } else if (w_out) {
     if (gs32) W4_GO(1, true, true); else W4_GO(1, true, false);
   } else if (cpk >= DEPTH) {
     if (gs32) W4_GO(DEPTH, false, true); else W4_GO(DEPTH, false, false);

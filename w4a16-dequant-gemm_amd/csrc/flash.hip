@@ -4,7 +4,7 @@
 // S rows of D elements; `group` query heads read the same slab (grouped-query
 // attention), so the slab is streamed from HBM once for all of them.
 //
-// Phase 1: grid (split, slab).  A workgroup walks its split of the sequence in
+// Phase 1: grid (slab, split).  A workgroup walks its split of the sequence in
 // tiles of 256 positions: K pass -> scaled scores in LDS, tile max, then V pass
 // accumulating exp(s - m) * v in FP32 registers; a running (m, l, acc) is
 // rescaled once per tile.  Lanes own a fixed slice of D (E elements) and a
@@ -135,8 +135,8 @@ __global__ __launch_bounds__(FL_WAVES * 64) void flash_phase1(const FlashArgs a,
   __shared__ float sc[GQ][FL_TILE];
   __shared__ float wred[FL_WAVES][GQ][512 + 2];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int split = blockIdx.x, slab = blockIdx.y;
-  const int nsplit = gridDim.x;
+  const int split = blockIdx.y, slab = blockIdx.x;  // slabs on x: no 65535 bound
+  const int nsplit = gridDim.y;
   const int PW = 64 / LP;             // position slots per wave
   const int sub = lane & (LP - 1);    // which E-chunk of the row
   const int slot = lane / LP;
@@ -386,7 +386,7 @@ static hipError_t go(const FlashArgs& a, int qh0, const FlashPlan& pl, float* sc
   const int chunks = (a.D + E - 1) / E;
   int LP = 1;
   while (LP < chunks) LP <<= 1;
-  const dim3 grid((unsigned)pl.nsplit, (unsigned)a.H);
+  const dim3 grid((unsigned)a.H, (unsigned)pl.nsplit);
   if (a.k_out || a.v_out)
     flash_phase1<KIND, E, GQ, true, FASTLD>
         <<<grid, FL_WAVES * 64, 0, s>>>(a, qh0, LP, pl.split_len, scratch);

@@ -86,7 +86,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c16 = lane & 15, q4 = lane >> 4;
-  const int split = blockIdx.x, slab = blockIdx.y, nsplit = gridDim.x;
+  const int split = blockIdx.y, slab = blockIdx.x, nsplit = gridDim.y;  // slabs on x: no 65535 bound
   const int nh = min(FM_HEADS, a.group - qh0);
   const float inv_sqrt_d = 1.0f / sqrtf((float)FM_D);
   const int G = a.G, wg = words(a.G);
@@ -350,7 +350,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
 template <int KIND, bool HOOK, int PAGED>
 static hipError_t go_asym(const FlashArgs& a, int qh0, const FlashPlan& pl, float* part,
                           hipStream_t s) {
-  const dim3 grid((unsigned)pl.nsplit, (unsigned)a.H);
+  const dim3 grid((unsigned)a.H, (unsigned)pl.nsplit);
   if (KIND == KIND_W4 && !a.symmetric)
     flash_mfma_phase1<KIND, HOOK, PAGED, true><<<grid, FM_WAVES * 64, 0, s>>>(a, qh0, pl.split_len, part);
   else

@@ -21,7 +21,9 @@ ATT = [(1, 1, 64, 32), (2, 7, 64, 8), (4, 128, 128, 128), (2, 300, 96, 32), (3, 
        (1, 4096, 64, 64),
        # head dimension 128 takes the matrix-core kernel: one position, ragged tiles, gs 32 / 64,
        # and gs = 8 (D = 128 on the general kernel)
-       (2, 1, 128, 32), (3, 33, 128, 32), (2, 129, 128, 64), (1, 777, 128, 32), (1, 300, 128, 8)]
+       (2, 1, 128, 32), (3, 33, 128, 32), (2, 129, 128, 64), (1, 777, 128, 32), (1, 300, 128, 8),
+       # head dimension 64 on the matrix-core kernel (gs a multiple of 16)
+       (2, 100, 64, 16), (1, 1, 64, 64), (3, 257, 64, 32)]
 BIG = [(2, 5000, 64, 32), (1, 9000, 128, 64)]
 
 
@@ -91,12 +93,19 @@ def test_w4_flash_grouped_query(group):
 
 @pytest.mark.parametrize("group", [3, 5])
 def test_w4_flash_grouped_query_general_kernel(group):
-    c4, q = _w4_case(2, 333, 64, 32, True, 0x6B22 + group, group)
+    c4, q = _w4_case(2, 333, 96, 32, True, 0x6B22 + group, group)
+    _check_w4(c4, q, group)
+
+
+@pytest.mark.parametrize("group", [4, 17])
+def test_w4_flash_grouped_query_head_dim_64(group):
+    c4, q = _w4_case(2, 400, 64, 32, group == 4, 0x6C33 + group, group)
     _check_w4(c4, q, group)
 
 
 F8 = [(1, 1, 64, 32), (2, 7, 64, 8), (4, 128, 128, 128), (2, 300, 96, 32), (3, 65, 40, 8),
-      (1, 9000, 128, 64), (2, 1, 128, 32), (2, 100, 128, 32), (1, 300, 128, 16)]
+      (1, 9000, 128, 64), (2, 1, 128, 32), (2, 100, 128, 32), (1, 300, 128, 16), (2, 200, 64, 16),
+      (1, 2500, 64, 64)]
 
 
 @pytest.mark.parametrize("i", range(len(F8)))
@@ -190,7 +199,8 @@ def test_f8_slab_scale_head_dim_128():
 PAGED = [(2, 300, 96, 32, 16), (2, 520, 64, 32, 16), (1, 1000, 128, 64, 64), (3, 65, 40, 8, 32),
          (1, 5000, 64, 32, 256),
          # matrix-core kernel: page 16, a page size that is no multiple of 16, one-row pages
-         (2, 700, 128, 32, 16), (1, 530, 128, 32, 24), (1, 100, 128, 128, 1), (2, 2000, 128, 32, 256)]
+         (2, 700, 128, 32, 16), (1, 530, 128, 32, 24), (1, 100, 128, 128, 1), (2, 2000, 128, 32, 256),
+         (2, 300, 64, 16, 40), (1, 900, 64, 32, 48)]
 
 
 def _paged_pool(c4, page, bt):

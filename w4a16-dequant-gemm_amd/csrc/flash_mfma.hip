@@ -1,11 +1,12 @@
-// Split-S flash-decode phase 1 on the matrix cores, head dimension 128.
+// Split-S flash-decode phase 1 on the matrix cores, head dimension 128 or 64.
 //
 // A wave walks tiles of 32 cache positions.  Per tile:
 //   scores   S[t][h] = sum_d K[t][d] q[h][d]  -- two groups of four
 //            v_mfma_f32_16x16x32_f16, A = K rows (lane: position l%16, 32 of the
 //            128 d), B = the query heads of the pass (up to 16 share one slab
 //            read).  A lane's A operand is exactly what it loads: one dwordx4 of
-//            packed codes (W4), two of bytes (FP8), four of halves (FP16).
+//            packed codes (W4), two of bytes (FP8), four of halves (FP16); half of
+//            that for D = 64, where a group is two MFMAs.
 //   softmax  the result leaves lane (h = l%16, r = l/16) with the scores of head
 //            h at positions {4r..4r+3, 16+4r..16+4r+3} of the tile; running
 //            max / rescale are per lane, the tile max needs two lane exchanges.
@@ -16,6 +17,8 @@
 //            word, 8 bytes, or 16 bytes each), expands them and regroups the
 //            8x8 block with v_perm so that MFMA e takes element e of every
 //            position.  A ninth MFMA with A = 1 accumulates the denominators.
+//            (D = 64 has only 8 element blocks: lanes i >= 8 repeat blocks 0..7
+//            and their output rows are dropped.)
 // Dequantisation is the bit-exact register step of dq.cuh (the k_out / v_out
 // hooks store those values); only the order of the FP32 sums differs from the
 // vector kernel.  The four waves of a workgroup interleave tiles of one split
@@ -27,29 +30,29 @@
 
 namespace w4k {
 
-constexpr int FM_D = 128;
 constexpr int FM_TILE = 32;   // positions per wave tile
 constexpr int FM_WAVES = 4;
 constexpr int FM_DEPTH = 2;   // tiles in flight per wave
 constexpr int FM_HEADS = 16;  // query heads per pass
 
 // What one lane fetches for one tile, before expansion.
-template <int KIND>
+// NC = D / 32: MFMAs per group of 16 positions = packed words (W4) per lane.
+template <int KIND, int NC>
 struct TileRaw;
-template <>
-struct TileRaw<KIND_W4> {
-  u4 k[2];
+template <int NC>
+struct TileRaw<KIND_W4, NC> {
+  uint32_t k[2][NC];
   uint32_t ks[2], kz[2];
   uint32_t v[8], vs[8], vz[8];
 };
-template <>
-struct TileRaw<KIND_F16> {
-  u4 k[2][4];
+template <int NC>
+struct TileRaw<KIND_F16, NC> {
+  u4 k[2][NC];
   u4 v[8];
 };
-template <>
-struct TileRaw<KIND_F8> {
-  u4 k[2][2];
+template <int NC>
+struct TileRaw<KIND_F8, NC> {
+  u2 k[2][NC];
   uint32_t ks[2];
   u2 v[8];
   uint32_t vs[8];
@@ -76,12 +79,16 @@ __device__ __forceinline__ h8 pack8(const h2 v[4]) {
 
 // PAGED: 0 contiguous slabs, 1 pages of a multiple of 16 rows (both halves of a
 // tile lie in one page each), 2 any page size.
-template <int KIND, bool HOOK, int PAGED, bool ASYM>
+template <int KIND, int DH, bool HOOK, int PAGED, bool ASYM>
 __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashArgs a,
                                                                    const int qh0,
                                                                    const int split_len,
                                                                    float* __restrict__ part) {
-  constexpr int LDW = FM_D + 4;  // floats per (wave, head) merge row: O[128], l, m
+  constexpr int FM_D = DH;       // head dimension
+  constexpr int NC = DH / 32;    // MFMAs per score group; a lane's K slice is 8 * NC elements
+  constexpr int NB = DH / 8;     // 8-element blocks per row
+  constexpr int WD = DH / 8;     // packed words per W4 row
+  constexpr int LDW = FM_D + 4;  // floats per (wave, head) merge row: O[D], l, m
   __shared__ float wo[FM_WAVES][FM_HEADS * LDW];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -90,8 +97,9 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
   const int nh = min(FM_HEADS, a.group - qh0);
   const float inv_sqrt_d = 1.0f / sqrtf((float)FM_D);
   const int G = a.G, wg = words(a.G);
-  const int gk = KIND == KIND_F16 ? 0 : (32 * q4) / a.gs;  // group of this lane's K elements
-  const int gv = KIND == KIND_F16 ? 0 : (8 * c16) / a.gs;  // ... and of its V elements
+  const int vb = c16 & (NB - 1);                               // this lane's V element block
+  const int gk = KIND == KIND_F16 ? 0 : (8 * NC * q4) / a.gs;  // group of this lane's K elements
+  const int gv = KIND == KIND_F16 ? 0 : (8 * vb) / a.gs;       // ... and of its V elements
 
   const int* bt = nullptr;
   long long rows0;
@@ -110,12 +118,13 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
   const bool hook_k = HOOK && a.k_out && qh0 == 0, hook_v = HOOK && a.v_out && qh0 == 0;
 
   // Query operands: lane (head c16, k-block q4) of MFMA c holds
-  // q[head][32 q4 + 8 c + elem_of(p, hf)].
-  h8 qop[4];
+  // q[head][8 NC q4 + 8 c + elem_of(p, hf)].
+  h8 qop[NC];
   {
-    const uint16_t* qp = a.q + ((long long)slab * a.group + qh0 + min(c16, nh - 1)) * FM_D + 32 * q4;
+    const uint16_t* qp =
+        a.q + ((long long)slab * a.group + qh0 + min(c16, nh - 1)) * FM_D + 8 * NC * q4;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
+    for (int c = 0; c < NC; ++c) {
       h2 t[4];
 #pragma unroll
       for (int p = 0; p < 4; ++p) {
@@ -134,7 +143,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     return rows0 + (long long)bt[pg] * a.page + (t - pg * a.page);
   };
 
-  auto fetch = [&](TileRaw<KIND>& raw, int t0) {
+  auto fetch = [&](TileRaw<KIND, NC>& raw, int t0) {
     int pg_lo = 0, pg_hi = 0;
     long long base_lo = 0, base_hi = 0;
     if (PAGED == 1) {  // wave-uniform lookups: the page of each 16-position half
@@ -148,19 +157,37 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
       const int t = min(t0 + 16 * j + c16, s1 - 1);
       const long long row = phys(t, pg_lo, base_lo, pg_hi, base_hi, j == 1);
       if constexpr (KIND == KIND_W4) {
-        raw.k[j] = __builtin_nontemporal_load((const u4*)((const uint32_t*)a.k + row * 16 + 4 * q4));
+        const uint32_t* src = (const uint32_t*)a.k + row * WD + NC * q4;
+        if constexpr (NC == 4) {
+          const u4 t4 = __builtin_nontemporal_load((const u4*)src);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) raw.k[j][c] = t4[c];
+        } else {
+          const u2 t2 = __builtin_nontemporal_load((const u2*)src);
+          raw.k[j][0] = t2[0];
+          raw.k[j][1] = t2[1];
+        }
         raw.ks[j] = a.s_k[row * G + gk];
         if (ASYM) raw.kz[j] = a.z_k[row * wg + (gk >> 3)];
       } else if constexpr (KIND == KIND_F16) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c)
+        for (int c = 0; c < NC; ++c)
           raw.k[j][c] = __builtin_nontemporal_load(
-              (const u4*)((const uint16_t*)a.k + row * FM_D + 32 * q4 + 8 * c));
+              (const u4*)((const uint16_t*)a.k + row * FM_D + 8 * NC * q4 + 8 * c));
       } else {
+        const uint8_t* src = (const uint8_t*)a.k + row * FM_D + 8 * NC * q4;
+        if constexpr (NC == 4) {
 #pragma unroll
-        for (int c = 0; c < 2; ++c)
-          raw.k[j][c] = __builtin_nontemporal_load(
-              (const u4*)((const uint8_t*)a.k + row * FM_D + 32 * q4 + 16 * c));
+          for (int c = 0; c < 2; ++c) {
+            const u4 t4 = __builtin_nontemporal_load((const u4*)(src + 16 * c));
+            raw.k[j][2 * c] = u2{t4[0], t4[1]};
+            raw.k[j][2 * c + 1] = u2{t4[2], t4[3]};
+          }
+        } else {
+          const u4 t4 = __builtin_nontemporal_load((const u4*)src);
+          raw.k[j][0] = u2{t4[0], t4[1]};
+          raw.k[j][1] = u2{t4[2], t4[3]};
+        }
         raw.ks[j] = a.scale_mode == 0 ? (uint32_t)a.s_k[row * G + gk] : slab_sk;
       }
     }
@@ -169,13 +196,13 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
       const int t = min(t0 + 16 * (k >> 2) + 4 * q4 + (k & 3), s1 - 1);
       const long long row = phys(t, pg_lo, base_lo, pg_hi, base_hi, k >= 4);
       if constexpr (KIND == KIND_W4) {
-        raw.v[k] = __builtin_nontemporal_load((const uint32_t*)a.v + row * 16 + c16);
+        raw.v[k] = __builtin_nontemporal_load((const uint32_t*)a.v + row * WD + vb);
         raw.vs[k] = a.s_v[row * G + gv];
         if (ASYM) raw.vz[k] = a.z_v[row * wg + (gv >> 3)];
       } else if constexpr (KIND == KIND_F16) {
-        raw.v[k] = __builtin_nontemporal_load((const u4*)((const uint16_t*)a.v + row * FM_D + 8 * c16));
+        raw.v[k] = __builtin_nontemporal_load((const u4*)((const uint16_t*)a.v + row * FM_D + 8 * vb));
       } else {
-        raw.v[k] = __builtin_nontemporal_load((const u2*)((const uint8_t*)a.v + row * FM_D + 8 * c16));
+        raw.v[k] = __builtin_nontemporal_load((const u2*)((const uint8_t*)a.v + row * FM_D + 8 * vb));
         raw.vs[k] = a.scale_mode == 0 ? (uint32_t)a.s_v[row * G + gv] : slab_sv;
       }
     }
@@ -191,17 +218,17 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     *(u4*)dst = u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
   };
 
-  auto compute = [&](const TileRaw<KIND>& raw, int t0) {
+  auto compute = [&](const TileRaw<KIND, NC>& raw, int t0) {
     // ---- scores
     f4 sc[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       sc[j] = f4{0.f, 0.f, 0.f, 0.f};
       const int t = t0 + 16 * j + c16;
-      uint16_t* kdst = HOOK ? a.k_out + (hook_base + t) * FM_D + 32 * q4 : nullptr;
+      uint16_t* kdst = HOOK ? a.k_out + (hook_base + t) * FM_D + 8 * NC * q4 : nullptr;
       const bool kst = hook_k && t < s1;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
+      for (int c = 0; c < NC; ++c) {
         h2 d[4];
         if constexpr (KIND == KIND_W4) {
           const int z = ASYM ? (int)((raw.kz[j] >> (4 * (gk & 7))) & 0xFu) : 8;
@@ -217,8 +244,8 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
           if (kst) store16(kdst + 8 * c, d);
         } else {
           const h2 s = splat_bits(raw.ks[j]);
-          dq_f8(raw.k[j][c >> 1][2 * (c & 1)], s, d);
-          dq_f8(raw.k[j][c >> 1][2 * (c & 1) + 1], s, d + 2);
+          dq_f8(raw.k[j][c][0], s, d);
+          dq_f8(raw.k[j][c][1], s, d + 2);
           if (kst) {
             h2 nat[4];
             to_natural_f8(d, nat);
@@ -260,8 +287,8 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       const int t = t0 + 16 * (k >> 2) + 4 * q4 + (k & 3);
-      const bool vst = hook_v && t < s1;
-      uint16_t* vdst = HOOK ? a.v_out + (hook_base + t) * FM_D + 8 * c16 : nullptr;
+      const bool vst = hook_v && t < s1 && c16 < NB;
+      uint16_t* vdst = HOOK ? a.v_out + (hook_base + t) * FM_D + 8 * vb : nullptr;
       if constexpr (KIND == KIND_W4) {
         const int z = ASYM ? (int)((raw.vz[k] >> (4 * (gv & 7))) & 0xFu) : 8;
         dq_w4(raw.v[k], w4_group((uint16_t)raw.vs[k], z), vt[k]);
@@ -302,25 +329,26 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
   // tiles of this wave: s0 + 32 * (wave + 4 * it)
   const int nit = (s1 - s0 + FM_WAVES * FM_TILE - 1) / (FM_WAVES * FM_TILE);
   auto tile_start = [&](int it) { return s0 + FM_TILE * (wave + FM_WAVES * it); };
-  TileRaw<KIND> ring[FM_DEPTH];
+  TileRaw<KIND, NC> ring[FM_DEPTH];
 #pragma unroll
   for (int d = 0; d < FM_DEPTH; ++d) fetch(ring[d], tile_start(d));
   for (int it0 = 0; it0 < nit; it0 += FM_DEPTH) {
 #pragma unroll
     for (int d = 0; d < FM_DEPTH; ++d) {
-      const TileRaw<KIND> raw = ring[d];
+      const TileRaw<KIND, NC> raw = ring[d];
       fetch(ring[d], tile_start(it0 + d + FM_DEPTH));
       compute(raw, tile_start(it0 + d));
     }
   }
 
   // ---- merge the four waves in wave order: lane (head c16, q4) holds
-  // O[head][32 q4 + 8 r + e] in o[e][r]
+  // O[head][32 q4 + 8 r + e] in o[e][r] (output rows past D / 8 are repeats: dropped)
   float* mine = wo[wave] + c16 * LDW;
 #pragma unroll
   for (int e = 0; e < 8; ++e)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) mine[32 * q4 + 8 * r + e] = o[e][r];
+    for (int r = 0; r < 4; ++r)
+      if (4 * q4 + r < NB) mine[32 * q4 + 8 * r + e] = o[e][r];
   if (q4 == 0) {
     mine[FM_D] = lsum[0];
     mine[FM_D + 1] = m_run;
@@ -351,10 +379,15 @@ template <int KIND, bool HOOK, int PAGED>
 static hipError_t go_asym(const FlashArgs& a, int qh0, const FlashPlan& pl, float* part,
                           hipStream_t s) {
   const dim3 grid((unsigned)a.H, (unsigned)pl.nsplit);
-  if (KIND == KIND_W4 && !a.symmetric)
-    flash_mfma_phase1<KIND, HOOK, PAGED, true><<<grid, FM_WAVES * 64, 0, s>>>(a, qh0, pl.split_len, part);
-  else
-    flash_mfma_phase1<KIND, HOOK, PAGED, false><<<grid, FM_WAVES * 64, 0, s>>>(a, qh0, pl.split_len, part);
+  const bool asym = KIND == KIND_W4 && !a.symmetric;
+#define W4_GO(DH, ASYM) \
+  flash_mfma_phase1<KIND, DH, HOOK, PAGED, ASYM><<<grid, FM_WAVES * 64, 0, s>>>(a, qh0, pl.split_len, part)
+  if (a.D == 128) {
+    if (asym) W4_GO(128, true); else W4_GO(128, false);
+  } else {
+    if (asym) W4_GO(64, true); else W4_GO(64, false);
+  }
+#undef W4_GO
   return hipGetLastError();
 }
 
@@ -373,8 +406,9 @@ static hipError_t go_kind(const FlashArgs& a, int qh0, const FlashPlan& pl, floa
 }
 
 bool flash_mfma_applies(const FlashArgs& a) {
-  if (a.D != FM_D) return false;
-  if (a.kind != KIND_F16 && a.gs % 32) return false;  // one group per lane's 32 K elements
+  if (a.D != 128 && a.D != 64) return false;
+  // one group per lane's K slice (32 elements at D = 128, 16 at D = 64) and per 8-element V block
+  if (a.kind != KIND_F16 && a.gs % (a.D / 4)) return false;
   return ((((uintptr_t)a.k | (uintptr_t)a.v) & 15) == 0) &&
          ((((uintptr_t)a.k_out | (uintptr_t)a.v_out) & 15) == 0);
 }

@@ -462,6 +462,165 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_unrolled_kernel(
   }
 }
 
+// One activation row, long or odd K (K % 32 == 0, K <= 16384; e.g. 11008, 14336,
+// 8192): the W waves of a workgroup share R = 2 weight rows and split K into
+// runs of whole 32-k slices (W is chosen so that the lanes are nearly all busy:
+// 6 waves for K = 11008, 7 for 14336); each wave is the unrolled kernel on its run
+// (activations straight from L2, everything requested before it is consumed,
+// lanes past the end of the quarter clamped to k = 0 with zeroed activations),
+// and the partial sums meet in LDS in wave order.
+template <int MX, int R, int W, int STEPS, bool ASYM, bool GS32, bool HOOK>
+__global__ __launch_bounds__(W * 64) void simt_ksplit_kernel(
+    const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int gs_shift,
+    w4_half* __restrict__ w_out) {
+  __shared__ float red[W][R];
+  constexpr int NS = (MX || GS32) ? 1 : 4;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n0 = blockIdx.x * R;
+  const int wpr = p.K >> 3;
+  const int wg = MX ? 0 : words(p.G);
+  const int slices = p.K >> 5;                              // 32-k slices in a row
+  const int per = (slices + W - 1) / W;                     // ... per wave
+  const int s_lo = wave * per, s_hi = min(slices, s_lo + per);
+
+  int k0[STEPS];
+  bool on[STEPS];
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    const int sl = s_lo + s * 64 + lane;
+    on[s] = sl < s_hi;
+    k0[s] = on[s] ? sl * 32 : 0;
+  }
+  u4 xv[STEPS][4];
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xv[s][j] = *(const u4*)(x + k0[s] + 8 * j);
+  uint32_t sc[STEPS][R][NS], zw[STEPS][R][NS], zsh[STEPS][NS];
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    int g[4];
+    if (NS == 1) g[0] = MX ? (k0[s] >> 5) : gs_shift >= 0 ? (k0[s] >> gs_shift) : k0[s] / p.gs;
+    else groups_of_slice(k0[s], p.gs, gs_shift, g);
+#pragma unroll
+    for (int e = 0; e < NS; ++e) {
+      zsh[s][e] = 4u * (uint32_t)(g[e] & 7);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const size_t n = (size_t)(n0 + r);
+        sc[s][r][e] = MX ? (uint32_t)((const uint8_t*)p.scales)[n * p.B + g[e]]
+                         : (uint32_t)((const uint16_t*)p.scales)[n * p.G + g[e]];
+        zw[s][r][e] = ASYM ? p.zeros[n * wg + (g[e] >> 3)] : 0u;
+      }
+    }
+  }
+  u4 qw[STEPS][R];
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s)
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      qw[s][r] = __builtin_nontemporal_load((const u4*)(p.q + (size_t)(n0 + r) * wpr + (k0[s] >> 3)));
+
+  float acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    u4 xr[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      xr[j] = MX ? xv[s][j] : pair_strided(xv[s][j]);
+      if (!on[s]) xr[j] = u4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float mxs = mx_scale(sc[s][r][0]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int e = NS == 1 ? 0 : j;
+        h2 d[4];
+        if (MX)
+          dq_mx(qw[s][r][j], mxs, d);
+        else
+          dq_w4(qw[s][r][j],
+                w4_group((uint16_t)sc[s][r][e], ASYM ? (int)((zw[s][r][e] >> zsh[s][e]) & 0xFu) : 8), d);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) acc[r] = dot2(d[t], as_h2(xr[j][t]), acc[r]);
+        if (HOOK && on[s]) {
+          h2 nat[4];
+          if (MX) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) nat[t] = d[t];
+          } else {
+            to_natural(d, nat);
+          }
+          *(u4*)(w_out + (size_t)(n0 + r) * p.K + k0[s] + 8 * j) =
+              u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) acc[r] = wave_sum_to_lane63(acc[r]);
+  if (lane == 63) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) red[wave][r] = acc[r];
+  }
+  __syncthreads();
+  if (threadIdx.x < R) {
+    const int r = threadIdx.x;
+    float sum = red[0][r];
+#pragma unroll
+    for (int w = 1; w < W; ++w) sum += red[w][r];
+    const _Float16 h = (_Float16)sum;
+    c[n0 + r] = __builtin_bit_cast(uint16_t, h);
+  }
+}
+
+template <int MX, int W, int STEPS>
+static hipError_t launch_ksplit(const WView& v, const w4_half* x, w4_half* c, hipStream_t s,
+                                w4_half* w_out) {
+  const bool gs32 = MX || v.gs % 32 == 0;
+  const bool pow2 = !MX && (v.gs & (v.gs - 1)) == 0;
+  const int sh = pow2 ? __builtin_ctz((unsigned)v.gs) : -1;
+  const unsigned grid = (unsigned)(v.N / SIMT_R);
+#define W4_GO(ASYM, GS32)                                                                 \
+  do {                                                                                    \
+    if (w_out)                                                                            \
+      simt_ksplit_kernel<MX, SIMT_R, W, STEPS, ASYM, GS32, true>                          \
+          <<<grid, W * 64, 0, s>>>(v, x, c, sh, w_out);                                   \
+    else                                                                                  \
+      simt_ksplit_kernel<MX, SIMT_R, W, STEPS, ASYM, GS32, false>                         \
+          <<<grid, W * 64, 0, s>>>(v, x, c, sh, w_out);                                   \
+  } while (0)
+  if (!MX && !v.symmetric) {
+    if (gs32) W4_GO(true, true); else W4_GO(true, false);
+  } else {
+    if (gs32) W4_GO(false, true); else W4_GO(false, false);
+  }
+#undef W4_GO
+  return hipGetLastError();
+}
+
+template <int MX>
+static bool try_ksplit(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
+                       w4_half* w_out, hipError_t* err) {
+  if (M != 1 || v.K % 32 || v.K > 16384 || v.K < 2048 || v.N % SIMT_R) return false;
+  // shapes of the unrolled kernel stay with it (and, hooked, with the kernel that sums like it)
+  const int blocks = v.K / 2048;
+  if (v.K % 2048 == 0 && (blocks == 1 || blocks == 2 || blocks == 4) && v.N % (SIMT_WAVES * SIMT_R) == 0)
+    return false;
+  if ((((uintptr_t)v.q | (uintptr_t)x | (uintptr_t)w_out) & 15)) return false;
+  const int slices = v.K >> 5;  // 64 ... 512
+  // fewest waves (at least 4) that cover the row in one step of 64 slices each; two steps past 512
+  if (slices <= 256) *err = launch_ksplit<MX, 4, 1>(v, x, c, s, w_out);
+  else if (slices <= 320) *err = launch_ksplit<MX, 5, 1>(v, x, c, s, w_out);
+  else if (slices <= 384) *err = launch_ksplit<MX, 6, 1>(v, x, c, s, w_out);
+  else if (slices <= 448) *err = launch_ksplit<MX, 7, 1>(v, x, c, s, w_out);
+  else *err = launch_ksplit<MX, 8, 1>(v, x, c, s, w_out);
+  return true;
+}
+
 template <int MX, int MT, int STEPS>
 static hipError_t launch_unrolled(const WView& v, const w4_half* x, w4_half* c, int M,
                                   hipStream_t s) {
@@ -505,6 +664,7 @@ static hipError_t launch_mt(const WView& v, const w4_half* x, w4_half* c, int M,
   constexpr int R = SIMT_R;
   hipError_t uerr = hipSuccess;
   if (try_unrolled<MX, MT>(v, x, c, M, s, w_out, &uerr)) return uerr;
+  if (MT == 1 && try_ksplit<MX>(v, x, c, M, s, w_out, &uerr)) return uerr;
   const bool fast = (v.K % 32 == 0) && (((uintptr_t)v.q & 15) == 0) &&
                     (w_out == nullptr || ((uintptr_t)w_out & 15) == 0);
   const bool x_vec = (v.K % 8 == 0) && (((uintptr_t)x & 15) == 0);

@@ -34,7 +34,8 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         # K % 8 == 0 but K % 32 != 0: whole words, rows of packed words not 16-byte aligned
         (9, 64, 4104, 8), (40, 48, 1032, 24), (3, 32, 520, 8), (100, 40, 264, 16),
         # one activation row, long or odd K: the vector kernel that splits K over the waves
-        (1, 64, 11008, 128), (1, 32, 2080, 32), (1, 16, 14336, 64), (1, 24, 5120, 48), (1, 8, 16384, 8)]
+        (1, 64, 11008, 128), (1, 32, 2080, 32), (1, 16, 14336, 64), (1, 24, 5120, 48), (1, 8, 16384, 8),
+        (2, 16, 11008, 128), (4, 8, 5120, 32), (3, 24, 14336, 64), (4, 16, 8192, 128)]
 TOL, CROSS = 1e-3, 2e-3  # rel L2 vs the FP64 oracle; between two gated paths
 
 

@@ -462,26 +462,28 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_unrolled_kernel(
   }
 }
 
-// One activation row, long or odd K (K % 32 == 0, K <= 16384; e.g. 11008, 14336,
-// 8192): the W waves of a workgroup share R = 2 weight rows and split K into
+// One or two activation rows, long or odd K (K % 32 == 0, K <= 16384; e.g. 11008,
+// 14336, 6144): the W waves of a workgroup share R = 2 weight rows and split K into
 // runs of whole 32-k slices (W is chosen so that the lanes are nearly all busy:
 // 6 waves for K = 11008, 7 for 14336); each wave is the unrolled kernel on its run
 // (activations straight from L2, everything requested before it is consumed,
 // lanes past the end of the quarter clamped to k = 0 with zeroed activations),
 // and the partial sums meet in LDS in wave order.
-template <int MX, int R, int W, int STEPS, bool ASYM, bool GS32, bool HOOK>
+template <int MX, int MT, int R, int W, int STEPS, bool ASYM, bool GS32, bool HOOK>
 __global__ __launch_bounds__(W * 64) void simt_ksplit_kernel(
-    const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int gs_shift,
-    w4_half* __restrict__ w_out) {
-  __shared__ float red[W][R];
+    const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
+    const int gs_shift, w4_half* __restrict__ w_out) {
+  __shared__ float red[W][R][MT];
   constexpr int NS = (MX || GS32) ? 1 : 4;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n0 = blockIdx.x * R;
+  const int m0 = blockIdx.y * MT;
   const int wpr = p.K >> 3;
   const int wg = MX ? 0 : words(p.G);
   const int slices = p.K >> 5;                              // 32-k slices in a row
   const int per = (slices + W - 1) / W;                     // ... per wave
   const int s_lo = wave * per, s_hi = min(slices, s_lo + per);
+  const bool hook = HOOK && blockIdx.y == 0;
 
   int k0[STEPS];
   bool on[STEPS];
@@ -491,11 +493,14 @@ __global__ __launch_bounds__(W * 64) void simt_ksplit_kernel(
     on[s] = sl < s_hi;
     k0[s] = on[s] ? sl * 32 : 0;
   }
-  u4 xv[STEPS][4];
+  u4 xv[STEPS][MT][4];
 #pragma unroll
   for (int s = 0; s < STEPS; ++s)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) xv[s][j] = *(const u4*)(x + k0[s] + 8 * j);
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)  // rows past M repeat the last row and are never stored
+        xv[s][m][j] = *(const u4*)(x + (size_t)min(m0 + m, M - 1) * p.K + k0[s] + 8 * j);
   uint32_t sc[STEPS][R][NS], zw[STEPS][R][NS], zsh[STEPS][NS];
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
@@ -521,17 +526,21 @@ __global__ __launch_bounds__(W * 64) void simt_ksplit_kernel(
     for (int r = 0; r < R; ++r)
       qw[s][r] = __builtin_nontemporal_load((const u4*)(p.q + (size_t)(n0 + r) * wpr + (k0[s] >> 3)));
 
-  float acc[R];
+  float acc[R][MT];
 #pragma unroll
-  for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[r][m] = 0.0f;
 #pragma unroll
   for (int s = 0; s < STEPS; ++s) {
-    u4 xr[4];
+    u4 xr[MT][4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      xr[j] = MX ? xv[s][j] : pair_strided(xv[s][j]);
-      if (!on[s]) xr[j] = u4{0u, 0u, 0u, 0u};
-    }
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        xr[m][j] = MX ? xv[s][m][j] : pair_strided(xv[s][m][j]);
+        if (!on[s]) xr[m][j] = u4{0u, 0u, 0u, 0u};
+      }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const float mxs = mx_scale(sc[s][r][0]);
@@ -545,8 +554,10 @@ __global__ __launch_bounds__(W * 64) void simt_ksplit_kernel(
           dq_w4(qw[s][r][j],
                 w4_group((uint16_t)sc[s][r][e], ASYM ? (int)((zw[s][r][e] >> zsh[s][e]) & 0xFu) : 8), d);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) acc[r] = dot2(d[t], as_h2(xr[j][t]), acc[r]);
-        if (HOOK && on[s]) {
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+          for (int t = 0; t < 4; ++t) acc[r][m] = dot2(d[t], as_h2(xr[m][j][t]), acc[r][m]);
+        if (hook && on[s]) {
           h2 nat[4];
           if (MX) {
 #pragma unroll
@@ -561,37 +572,43 @@ __global__ __launch_bounds__(W * 64) void simt_ksplit_kernel(
     }
   }
 #pragma unroll
-  for (int r = 0; r < R; ++r) acc[r] = wave_sum_to_lane63(acc[r]);
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[r][m] = wave_sum_to_lane63(acc[r][m]);
   if (lane == 63) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) red[wave][r] = acc[r];
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int m = 0; m < MT; ++m) red[wave][r][m] = acc[r][m];
   }
   __syncthreads();
-  if (threadIdx.x < R) {
-    const int r = threadIdx.x;
-    float sum = red[0][r];
+  if (threadIdx.x < R * MT) {
+    const int r = threadIdx.x / MT, m = threadIdx.x % MT;
+    float sum = red[0][r][m];
 #pragma unroll
-    for (int w = 1; w < W; ++w) sum += red[w][r];
-    const _Float16 h = (_Float16)sum;
-    c[n0 + r] = __builtin_bit_cast(uint16_t, h);
+    for (int w = 1; w < W; ++w) sum += red[w][r][m];
+    if (m0 + m < M) {
+      const _Float16 h = (_Float16)sum;
+      c[(size_t)(m0 + m) * p.N + n0 + r] = __builtin_bit_cast(uint16_t, h);
+    }
   }
 }
 
-template <int MX, int W, int STEPS>
-static hipError_t launch_ksplit(const WView& v, const w4_half* x, w4_half* c, hipStream_t s,
+template <int MX, int MT, int W, int STEPS>
+static hipError_t launch_ksplit(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                                 w4_half* w_out) {
   const bool gs32 = MX || v.gs % 32 == 0;
   const bool pow2 = !MX && (v.gs & (v.gs - 1)) == 0;
   const int sh = pow2 ? __builtin_ctz((unsigned)v.gs) : -1;
-  const unsigned grid = (unsigned)(v.N / SIMT_R);
+  const dim3 grid((unsigned)(v.N / SIMT_R), (unsigned)((M + MT - 1) / MT));
 #define W4_GO(ASYM, GS32)                                                                 \
   do {                                                                                    \
     if (w_out)                                                                            \
-      simt_ksplit_kernel<MX, SIMT_R, W, STEPS, ASYM, GS32, true>                          \
-          <<<grid, W * 64, 0, s>>>(v, x, c, sh, w_out);                                   \
+      simt_ksplit_kernel<MX, MT, SIMT_R, W, STEPS, ASYM, GS32, true>                      \
+          <<<grid, W * 64, 0, s>>>(v, x, c, M, sh, w_out);                                \
     else                                                                                  \
-      simt_ksplit_kernel<MX, SIMT_R, W, STEPS, ASYM, GS32, false>                         \
-          <<<grid, W * 64, 0, s>>>(v, x, c, sh, w_out);                                   \
+      simt_ksplit_kernel<MX, MT, SIMT_R, W, STEPS, ASYM, GS32, false>                     \
+          <<<grid, W * 64, 0, s>>>(v, x, c, M, sh, w_out);                                \
   } while (0)
   if (!MX && !v.symmetric) {
     if (gs32) W4_GO(true, true); else W4_GO(true, false);
@@ -602,22 +619,24 @@ static hipError_t launch_ksplit(const WView& v, const w4_half* x, w4_half* c, hi
   return hipGetLastError();
 }
 
-template <int MX>
+template <int MX, int MT>
 static bool try_ksplit(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                        w4_half* w_out, hipError_t* err) {
-  if (M != 1 || v.K % 32 || v.K > 16384 || v.K < 2048 || v.N % SIMT_R) return false;
+  // four rows fetched per wave cost more than the staged kernel's barrier (20.7 vs 19 us at K = 11008)
+  if (MT > 2 || v.K % 32 || v.K > 16384 || v.K < 2048 || v.N % SIMT_R) return false;
   // shapes of the unrolled kernel stay with it (and, hooked, with the kernel that sums like it)
   const int blocks = v.K / 2048;
-  if (v.K % 2048 == 0 && (blocks == 1 || blocks == 2 || blocks == 4) && v.N % (SIMT_WAVES * SIMT_R) == 0)
+  if (v.K % 2048 == 0 && (blocks == 1 || blocks == 2 || blocks == 4) && blocks * MT <= 8 &&
+      v.N % (SIMT_WAVES * SIMT_R) == 0)
     return false;
   if ((((uintptr_t)v.q | (uintptr_t)x | (uintptr_t)w_out) & 15)) return false;
   const int slices = v.K >> 5;  // 64 ... 512
   // fewest waves (at least 4) that cover the row in one step of 64 slices each; two steps past 512
-  if (slices <= 256) *err = launch_ksplit<MX, 4, 1>(v, x, c, s, w_out);
-  else if (slices <= 320) *err = launch_ksplit<MX, 5, 1>(v, x, c, s, w_out);
-  else if (slices <= 384) *err = launch_ksplit<MX, 6, 1>(v, x, c, s, w_out);
-  else if (slices <= 448) *err = launch_ksplit<MX, 7, 1>(v, x, c, s, w_out);
-  else *err = launch_ksplit<MX, 8, 1>(v, x, c, s, w_out);
+  if (slices <= 256) *err = launch_ksplit<MX, MT <= 2 ? MT : 1, 4, 1>(v, x, c, M, s, w_out);
+  else if (slices <= 320) *err = launch_ksplit<MX, MT <= 2 ? MT : 1, 5, 1>(v, x, c, M, s, w_out);
+  else if (slices <= 384) *err = launch_ksplit<MX, MT <= 2 ? MT : 1, 6, 1>(v, x, c, M, s, w_out);
+  else if (slices <= 448) *err = launch_ksplit<MX, MT <= 2 ? MT : 1, 7, 1>(v, x, c, M, s, w_out);
+  else *err = launch_ksplit<MX, MT <= 2 ? MT : 1, 8, 1>(v, x, c, M, s, w_out);
   return true;
 }
 
@@ -664,7 +683,7 @@ static hipError_t launch_mt(const WView& v, const w4_half* x, w4_half* c, int M,
   constexpr int R = SIMT_R;
   hipError_t uerr = hipSuccess;
   if (try_unrolled<MX, MT>(v, x, c, M, s, w_out, &uerr)) return uerr;
-  if (MT == 1 && try_ksplit<MX>(v, x, c, M, s, w_out, &uerr)) return uerr;
+  if (try_ksplit<MX, MT>(v, x, c, M, s, w_out, &uerr)) return uerr;
   const bool fast = (v.K % 32 == 0) && (((uintptr_t)v.q & 15) == 0) &&
                     (w_out == nullptr || ((uintptr_t)w_out & 15) == 0);
   const bool x_vec = (v.K % 8 == 0) && (((uintptr_t)x & 15) == 0);

@@ -357,6 +357,62 @@ def extras_attention(b, full):
     return {"c5_flash_decode": res}
 
 
+def extras_quantize(b, full):
+    """Device-side quantizers (memory-bound streams): bytes read + written per call over the
+    call's duration.  Sources: FP64 weights (as the host quantizers take them), FP16 K/V rows."""
+    capi, torch = b.capi, b.torch
+    st = b.stream
+    steps = max(5, b.steps // 20)
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    res = {}
+    N = K = 4096
+    gs, G = 128, 32
+    w = torch.randn(N * K, device="cuda", dtype=torch.float64)
+    q = torch.empty(N * K // 8, dtype=torch.int32, device="cuda")
+    sc = torch.empty(N * G, dtype=torch.int16, device="cuda")
+    z = torch.empty(N * G // 8, dtype=torch.int32, device="cuda")
+    for sym in (True, False):
+        view = capi.packed_view(N, K, gs, G, sym, q.data_ptr(), sc.data_ptr(), 0 if sym else z.data_ptr())
+        ms = _median_events_ms(torch, lambda i: capi.quantize(view, w.data_ptr(), status.data_ptr(), st),
+                               steps, 2)
+        nb = N * K * 8 + w4_bytes(N, K, gs, sym, 0)
+        res["w4_%s_f64_4096x4096" % ("sym" if sym else "asym")] = {"ms": ms, "bytes": nb, "GBs": nb / ms * 1e-6}
+    B = K // 32
+    sb = torch.empty(N * B, dtype=torch.uint8, device="cuda")
+    view = capi.packed_mx_view(N, K, B, q.data_ptr(), sb.data_ptr())
+    ms = _median_events_ms(torch, lambda i: capi.quantize_mx(view, w.data_ptr(), status.data_ptr(), st),
+                           steps, 2)
+    nb = N * K * 8 + mx_bytes(N, K, 0)
+    res["mx_f64_4096x4096"] = {"ms": ms, "bytes": nb, "GBs": nb / ms * 1e-6}
+    del w
+    # KV rows from FP16: a whole prefill (64 slabs x 4096 rows) and one appended row per slab
+    D, gs, G = 128, 32, 4
+    for H, S in ((64, 4096), (64, 1)):
+        rows = H * S
+        k16 = torch.randn(rows * D, device="cuda", dtype=torch.float16)
+        v16 = torch.randn(rows * D, device="cuda", dtype=torch.float16)
+        qk = torch.empty(rows * D // 8, dtype=torch.int32, device="cuda")
+        qv = torch.empty_like(qk)
+        sk = torch.empty(rows * G, dtype=torch.int16, device="cuda")
+        sv = torch.empty_like(sk)
+        view = capi.kv_view(H, S, D, gs, G, True, qk.data_ptr(), sk.data_ptr(), 0, qv.data_ptr(),
+                            sv.data_ptr(), 0)
+        ms = _median_events_ms(torch, lambda i: capi.quantize_cache(
+            view, k16.data_ptr(), v16.data_ptr(), status.data_ptr(), True, st), steps, 2)
+        nb = 2 * rows * (D * 2 + D // 2 + G * 2)
+        res["kv_w4_f16_%dx%d" % (H, S)] = {"ms": ms, "bytes": nb, "GBs": nb / ms * 1e-6}
+        bk = torch.empty(rows * D, dtype=torch.uint8, device="cuda")
+        bv = torch.empty_like(bk)
+        view8 = capi.kv_f8_view(H, S, D, gs, G, bk.data_ptr(), sk.data_ptr(), bv.data_ptr(), sv.data_ptr())
+        ms = _median_events_ms(torch, lambda i: capi.quantize_cache_f8(
+            view8, k16.data_ptr(), v16.data_ptr(), status.data_ptr(), True, st), steps, 2)
+        nb = 2 * rows * (D * 2 + D + G * 2)
+        res["kv_f8_f16_%dx%d" % (H, S)] = {"ms": ms, "bytes": nb, "GBs": nb / ms * 1e-6}
+    torch.cuda.synchronize()
+    assert int(status.item()) == 0
+    return {"quantize": res}
+
+
 def probe(b, which):
     """Short fixed workloads for counter runs under a profiler (no headline, no yardsticks)."""
     capi, torch = b.capi, b.torch
@@ -416,6 +472,7 @@ def main():
     if args.extras != "none":
         extra.update(extras_gemm(b, args.extras == "full"))
         extra.update(extras_attention(b, args.extras == "full"))
+        extra.update(extras_quantize(b, args.extras == "full"))
     cpu = h["cpu"]
     line = {
         "metric": "M=1 W4 GEMM us + achieved HBM GB/s (% of peak); M=2048 MFMA TFLOP/s",

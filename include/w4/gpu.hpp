@@ -269,4 +269,85 @@ inline void attention_w4_flash_paged_batched(const DeviceKVW4& p, const int* bt,
                                                     detail::h(q), detail::h(out), stream));
 }
 
+// ---- device-side quantizers ---------------------------------------------------
+// The host quantizers as kernels: the views' arrays receive the bytes
+// w4::quantize / quantize_mx / quantize_cache / quantize_cache_f8 would
+// produce for the same values.  `status` is one device int the caller owns.
+// The *_async forms only enqueue; the caller reads the status word later (bit 0
+// non-finite input, bit 1 scale out of range).  The plain forms wait for the
+// stream and throw what the host quantizer throws.
+namespace detail {
+inline void raise_status(const int* status, hipStream_t stream, const char* nonfinite,
+                         const char* range) {
+  int st = 0;
+  hip_check(hipMemcpyAsync(&st, status, sizeof st, hipMemcpyDeviceToHost, stream), "status copy");
+  hip_check(hipStreamSynchronize(stream), "status sync");
+  if (st & 1) throw std::invalid_argument(nonfinite);
+  if (st & 2) throw std::invalid_argument(range);
+}
+}  // namespace detail
+
+// pack.hpp:64-130
+inline void quantize_async(const DevicePackedW& out, const double* w, int* status,
+                           hipStream_t stream = 0) {
+  const auto v = detail::abi(out);
+  detail::raise(w4_quantize(&v, w, status, stream));
+}
+inline void quantize(const DevicePackedW& out, const double* w, int* status,
+                     hipStream_t stream = 0) {
+  quantize_async(out, w, status, stream);
+  detail::raise_status(status, stream, "quantize: non-finite input",
+                       "quantize: group scale outside FP16 range");
+}
+
+// mx.hpp:71-119
+inline void quantize_mx_async(const DevicePackedWm& out, const double* w, int* status,
+                              hipStream_t stream = 0) {
+  const auto v = detail::abi(out);
+  detail::raise(w4_quantize_mx(&v, w, status, stream));
+}
+inline void quantize_mx(const DevicePackedWm& out, const double* w, int* status,
+                        hipStream_t stream = 0) {
+  quantize_mx_async(out, w, status, stream);
+  detail::raise_status(status, stream, "quantize_mx: non-finite input",
+                       "quantize_mx: block scale outside E8M0 range");
+}
+
+// kvcache.hpp:60-108.  k, v: H*S*D doubles, or halves with the _f16 forms (the
+// append step of a decode loop, whose new rows are FP16 already).
+inline void quantize_cache_async(const DeviceKVW4& out, const double* k, const double* v,
+                                 int* status, hipStream_t stream = 0) {
+  const auto vw = detail::abi(out);
+  detail::raise(w4_quantize_cache(&vw, k, v, 0, status, stream));
+}
+inline void quantize_cache_f16_async(const DeviceKVW4& out, const __half* k, const __half* v,
+                                     int* status, hipStream_t stream = 0) {
+  const auto vw = detail::abi(out);
+  detail::raise(w4_quantize_cache(&vw, k, v, 1, status, stream));
+}
+inline void quantize_cache(const DeviceKVW4& out, const double* k, const double* v, int* status,
+                           hipStream_t stream = 0) {
+  quantize_cache_async(out, k, v, status, stream);
+  detail::raise_status(status, stream, "quantize: non-finite input",
+                       "quantize: group scale outside FP16 range");
+}
+
+// kvfp8.hpp:70-128
+inline void quantize_cache_f8_async(const DeviceKVF8& out, const double* k, const double* v,
+                                    int* status, hipStream_t stream = 0) {
+  const auto vw = detail::abi(out);
+  detail::raise(w4_quantize_cache_f8(&vw, k, v, 0, status, stream));
+}
+inline void quantize_cache_f8_f16_async(const DeviceKVF8& out, const __half* k, const __half* v,
+                                        int* status, hipStream_t stream = 0) {
+  const auto vw = detail::abi(out);
+  detail::raise(w4_quantize_cache_f8(&vw, k, v, 1, status, stream));
+}
+inline void quantize_cache_f8(const DeviceKVF8& out, const double* k, const double* v,
+                              int* status, hipStream_t stream = 0) {
+  quantize_cache_f8_async(out, k, v, status, stream);
+  detail::raise_status(status, stream, "quantize_cache_f8: non-finite input",
+                       "quantize_cache_f8: group scale outside FP16 range");
+}
+
 }  // namespace w4::gpu

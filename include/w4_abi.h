@@ -146,6 +146,28 @@ int w4_attention_w4_flash_paged_batched(const w4_kv_view* p, const int* bt,
                                         const w4_half* q, w4_half* out,
                                         w4_stream stream);
 
+/* ---- device-side quantizers: the host quantizers as kernels, same bytes -----
+ * The view's arrays are the OUTPUTS (device memory of the sizes the view
+ * implies; no need to clear them).  Sources are row-major FP64, as the host
+ * quantizers take them; the cache forms also take FP16 sources (src_f16 != 0),
+ * which quantize as the same values widened to FP64.  What the host reports by
+ * throwing after looking at the data lands in *status (a device int, cleared
+ * by the call): bit 0 non-finite input, bit 1 a group scale outside the FP16
+ * (E8M0 for MXFP4) range (non-finite input may set both; the host reports it
+ * first).  Outputs are unspecified when it ends non-zero. */
+/* include/w4/pack.hpp:64-130 */
+int w4_quantize(const w4_packed_view* out, const double* w, int* status,
+                w4_stream stream);
+/* include/w4/mx.hpp:71-119 */
+int w4_quantize_mx(const w4_packed_mx_view* out, const double* w, int* status,
+                   w4_stream stream);
+/* include/w4/kvcache.hpp:60-108; k, v: H*S*D elements, head- then row-major */
+int w4_quantize_cache(const w4_kv_view* out, const void* k, const void* v,
+                      int src_f16, int* status, w4_stream stream);
+/* include/w4/kvfp8.hpp:70-128 */
+int w4_quantize_cache_f8(const w4_kv_f8_view* out, const void* k, const void* v,
+                         int src_f16, int* status, w4_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

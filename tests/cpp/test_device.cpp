@@ -270,6 +270,87 @@ void attention_gates(Checks& t) {
   }
 }
 
+// The device quantizers against the host ones of the same headers
+// (pack.hpp:64-130, mx.hpp:71-119, kvcache.hpp:60-108, kvfp8.hpp:70-128): same
+// bytes, same exceptions.
+template <class F>
+bool throws_invalid(F&& f, const char* text) {
+  try {
+    f();
+  } catch (const std::invalid_argument& e) {
+    return std::strstr(e.what(), text) != nullptr;
+  } catch (...) {
+  }
+  return false;
+}
+
+void quantizer_gates(Checks& t) {
+  Dev<int> status(1);
+  const Shape shapes[] = {{0, 5, 200, 64}, {0, 3, 1001, 128}, {0, 7, 100, 24}, {0, 64, 4096, 128}};
+  for (const Shape& c : shapes)
+    for (const bool sym : {true, false}) {
+      auto w = normal_weights(c.N * c.K, 0x51u + (unsigned)c.K);
+      for (size_t i = 0; i < w.size(); i += 3) w[i] *= 9.0;  // heavier tails
+      const PackedW ref = quantize(w, c.N, c.K, c.gs, sym);
+      Dev<double> wd(w);
+      Dev<uint32_t> q(ref.q.size()), z(ref.zeros.size());
+      Dev<__half> s(ref.scales.size());
+      const DevicePackedW out{c.N, c.K, c.gs, ref.G, sym ? 1 : 0, q.p, s.p, sym ? nullptr : z.p};
+      gpu::quantize(out, wd.p, status.p);
+      t.expect(same(q.get(), ref.q) && same(s.get(), ref.scales), "device quantize: codes, scales");
+      if (!sym) t.expect(same(z.get(), ref.zeros), "device quantize: zero-points");
+    }
+  {
+    const int N = 6, K = 1000;
+    auto w = normal_weights(N * K, 77);
+    const mx::PackedWm ref = mx::quantize_mx(w, N, K);
+    Dev<double> wd(w);
+    Dev<uint32_t> q(ref.q.size());
+    Dev<uint8_t> s(ref.scales.size());
+    const DevicePackedWm out{N, K, ref.B, q.p, s.p};
+    gpu::quantize_mx(out, wd.p, status.p);
+    t.expect(same(q.get(), ref.q) && same(s.get(), ref.scales), "device quantize_mx");
+    w[123] = std::nan("");
+    Dev<double> bad(w);
+    t.expect(throws_invalid([&] { gpu::quantize_mx(out, bad.p, status.p); },
+                            "quantize_mx: non-finite input"),
+             "device quantize_mx throws on NaN");
+  }
+  {
+    const int H = 3, S = 65, D = 128, gs = 32;
+    const auto k = normal_weights(H * S * D, 5), v = normal_weights(H * S * D, 6);
+    Dev<double> kd(k), vd(v);
+    for (const bool sym : {true, false}) {
+      const kv::KVCacheW4 ref = kv::quantize_cache(k, v, H, S, D, gs, sym);
+      Dev<uint32_t> qk(ref.q_k.size()), qv(ref.q_v.size()), zk(ref.z_k.size()), zv(ref.z_v.size());
+      Dev<__half> sk(ref.s_k.size()), sv(ref.s_v.size());
+      const DeviceKVW4 out{H, S, D, gs, ref.G, sym ? 1 : 0, qk.p, sk.p, sym ? nullptr : zk.p,
+                           qv.p, sv.p, sym ? nullptr : zv.p};
+      gpu::quantize_cache(out, kd.p, vd.p, status.p);
+      t.expect(same(qk.get(), ref.q_k) && same(qv.get(), ref.q_v) && same(sk.get(), ref.s_k) &&
+                   same(sv.get(), ref.s_v),
+               "device quantize_cache: codes, scales");
+      if (!sym)
+        t.expect(same(zk.get(), ref.z_k) && same(zv.get(), ref.z_v),
+                 "device quantize_cache: zero-points");
+    }
+    const kv8::KVCacheF8 ref8 = kv8::quantize_cache_f8(k, v, H, S, D, gs);
+    Dev<uint8_t> qk(ref8.q_k.size()), qv(ref8.q_v.size());
+    Dev<__half> sk(ref8.s_k.size()), sv(ref8.s_v.size());
+    const DeviceKVF8 out8{H, S, D, gs, ref8.G, qk.p, sk.p, qv.p, sv.p};
+    gpu::quantize_cache_f8(out8, kd.p, vd.p, status.p);
+    t.expect(same(qk.get(), ref8.q_k) && same(qv.get(), ref8.q_v) && same(sk.get(), ref8.s_k) &&
+                 same(sv.get(), ref8.s_v),
+             "device quantize_cache_f8");
+    auto big = v;
+    big[7] = 1e9;
+    Dev<double> bigd(big);
+    t.expect(throws_invalid([&] { gpu::quantize_cache_f8(out8, kd.p, bigd.p, status.p); },
+                            "group scale outside FP16 range"),
+             "device quantize_cache_f8 throws on a scale beyond FP16");
+  }
+}
+
 }  // namespace
 
 int main() {
@@ -281,6 +362,7 @@ int main() {
   Checks t;
   gemm_gates(t);
   attention_gates(t);
+  quantizer_gates(t);
   std::printf("worst rel L2 vs the FP64 references = %.3e\n", g_worst);
   return t.finish("device");
 }

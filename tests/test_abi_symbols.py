@@ -4,6 +4,8 @@ import ctypes
 import os
 import re
 
+import pytest
+
 import w4amd
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -35,3 +37,32 @@ def test_validation_runs_without_a_device():
     else:
         raise AssertionError("a malformed view was accepted")
     assert capi.load().w4_dispatch_mma_min_m() >= 1
+
+
+def test_quantize_contracts():
+    """Malformed calls are rejected before the device is touched (pack.hpp:64-72,
+    mx.hpp:71-76, kvcache.hpp:60-68, kvfp8.hpp:70-79)."""
+    c = w4amd.capi()
+    one = 8  # any non-null address: nothing is dereferenced
+    for view, text in [(c.packed_view(0, 32, 8, 4, 1, one, one), "bad dims"),
+                       (c.packed_view(2, 32, 12, 3, 1, one, one), "multiple of 8"),
+                       (c.packed_view(2, 32, 8, 5, 1, one, one), "G inconsistent"),
+                       (c.packed_view(2, 32, 8, 4, 0, one, one, 0), "asymmetric without zeros"),
+                       (c.packed_view(2, 32, 8, 4, 1, one, one, one), "symmetric carries no zeros"),
+                       (c.packed_view(2, 32, 8, 4, 1, 0, one), "null pointer")]:
+        with pytest.raises(ValueError, match=text):
+            c.quantize(view, one, one)
+    with pytest.raises(ValueError, match="null pointer"):
+        c.quantize(c.packed_view(2, 32, 8, 4, 1, one, one), one, 0)
+    with pytest.raises(ValueError, match="B inconsistent"):
+        c.quantize_mx(c.packed_mx_view(2, 64, 3, one, one), one, one)
+    with pytest.raises(ValueError, match="bad dims"):
+        c.quantize_mx(c.packed_mx_view(2, 0, 0, one, one), one, one)
+    with pytest.raises(ValueError, match="multiple of 8"):
+        c.quantize_cache(c.kv_view(1, 1, 64, 20, 4, 1, one, one, 0, one, one, 0), one, one, one)
+    with pytest.raises(ValueError, match="asymmetric without zeros"):
+        c.quantize_cache(c.kv_view(1, 1, 64, 16, 4, 0, one, one, 0, one, one, 0), one, one, one)
+    with pytest.raises(ValueError, match="null pointer"):
+        c.quantize_cache_f8(c.kv_f8_view(1, 1, 64, 16, 4, one, one, one, one), 0, one, one)
+    with pytest.raises(ValueError, match="G inconsistent"):
+        c.quantize_cache_f8(c.kv_f8_view(1, 1, 64, 16, 3, one, one, one, one), one, one, one)

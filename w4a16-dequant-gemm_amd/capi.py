@@ -57,6 +57,10 @@ SIGNATURES = {
     "w4_attention_f8_flash_gqa": ([C.POINTER(KVF8View), C.c_int, C.c_int, vp, vp, vp, vp, vp], C.c_int),
     "w4_attention_w4_flash_paged_batched": ([C.POINTER(KVView), vp, C.c_int, C.c_int, C.c_int, C.c_int,
                                              C.c_int, vp, vp, vp], C.c_int),
+    "w4_quantize": ([C.POINTER(PackedView), vp, vp, vp], C.c_int),
+    "w4_quantize_mx": ([C.POINTER(PackedMxView), vp, vp, vp], C.c_int),
+    "w4_quantize_cache": ([C.POINTER(KVView), vp, vp, C.c_int, vp, vp], C.c_int),
+    "w4_quantize_cache_f8": ([C.POINTER(KVF8View), vp, vp, C.c_int, vp, vp], C.c_int),
 }
 
 _lib = None
@@ -170,3 +174,23 @@ def attention_w4_flash_paged_batched(view, bt, nseq, bt_stride, page, npages, gr
 
 def dequant_f8(q, s, w, S, D, gs, stream=0):
     check(load().w4_dequant_f8(_n(q), _n(s), _n(w), S, D, gs, _n(stream)))
+
+
+# Device-side quantizers: the view's arrays are outputs; `status` is a device int
+# (bit 0 non-finite input, bit 1 scale out of range), cleared by the call.
+def quantize(view, w, status, stream=0):
+    check(load().w4_quantize(C.byref(view), _n(w), _n(status), _n(stream)))
+
+
+def quantize_mx(view, w, status, stream=0):
+    check(load().w4_quantize_mx(C.byref(view), _n(w), _n(status), _n(stream)))
+
+
+def quantize_cache(view, k, v, status, src_f16=False, stream=0):
+    check(load().w4_quantize_cache(C.byref(view), _n(k), _n(v), int(src_f16), _n(status),
+                                   _n(stream)))
+
+
+def quantize_cache_f8(view, k, v, status, src_f16=False, stream=0):
+    check(load().w4_quantize_cache_f8(C.byref(view), _n(k), _n(v), int(src_f16), _n(status),
+                                      _n(stream)))

@@ -341,6 +341,82 @@ int w4_dequant_f8(const uint8_t* q, const w4_half* s, w4_half* w, int S, int D, 
   return done("dequant_f8", w4k::launch_dequant_f8(q, s, w, S, D, gs, (hipStream_t)stream));
 }
 
+// ---- device-side quantizers -------------------------------------------------------
+// Contracts of the host quantizers (pack.hpp:64-72, mx.hpp:71-76,
+// kvcache.hpp:60-68, kvfp8.hpp:70-79); what they find in the data (non-finite
+// input, scale out of range) lands in *status instead of a throw.
+
+static int start_status(int* status, w4_stream stream, const char* what) {
+  return done(what, w4k::launch_fill_words((uint32_t*)status, 1, 0u, (hipStream_t)stream));
+}
+
+int w4_quantize(const w4_packed_view* out, const double* w, int* status, w4_stream stream) {
+  if (int rc = check_packed(out, "quantize")) return rc;
+  REQUIRE(w && status, "quantize: null pointer");
+  if (int rc = start_status(status, stream, "quantize")) return rc;
+  return done("quantize", w4k::launch_quantize_rows(
+                              out->symmetric ? 0 : 1, w, 0, out->N, out->K, out->gs,
+                              (uint32_t*)out->q, nullptr, (w4_half*)out->scales,
+                              (uint32_t*)out->zeros, status, (hipStream_t)stream));
+}
+
+int w4_quantize_mx(const w4_packed_mx_view* out, const double* w, int* status,
+                   w4_stream stream) {
+  REQUIRE(out != nullptr, "quantize_mx: null view");
+  REQUIRE(out->N >= 1 && out->K >= 1, "quantize_mx: bad dims");
+  REQUIRE(out->B == (out->K + 31) / 32, "quantize_mx: B inconsistent with K");
+  REQUIRE(out->q && out->scales && w && status, "quantize_mx: null pointer");
+  if (int rc = start_status(status, stream, "quantize_mx")) return rc;
+  return done("quantize_mx",
+              w4k::launch_quantize_mx(w, 0, out->N, out->K, (uint32_t*)out->q,
+                                      (uint8_t*)out->scales, status, (hipStream_t)stream));
+}
+
+int w4_quantize_cache(const w4_kv_view* out, const void* k, const void* v, int src_f16,
+                      int* status, w4_stream stream) {
+  REQUIRE(out != nullptr, "quantize_cache: null view");
+  REQUIRE(out->H >= 1 && out->S >= 1 && out->D >= 1, "quantize_cache: bad dims");
+  REQUIRE(out->gs >= 8 && out->gs % 8 == 0, "quantize_cache: gs must be a multiple of 8");
+  REQUIRE(out->G == (out->D + out->gs - 1) / out->gs, "quantize_cache: G inconsistent with D, gs");
+  REQUIRE(out->q_k && out->s_k && out->q_v && out->s_v && k && v && status,
+          "quantize_cache: null pointer");
+  REQUIRE(out->symmetric || (out->z_k && out->z_v), "quantize_cache: asymmetric without zeros");
+  REQUIRE(!out->symmetric || (!out->z_k && !out->z_v),
+          "quantize_cache: symmetric carries no zeros");
+  if (int rc = start_status(status, stream, "quantize_cache")) return rc;
+  const long long rows = (long long)out->H * out->S;
+  const int mode = out->symmetric ? 0 : 1;
+  hipError_t e = w4k::launch_quantize_rows(mode, k, src_f16, rows, out->D, out->gs,
+                                           (uint32_t*)out->q_k, nullptr, (w4_half*)out->s_k,
+                                           (uint32_t*)out->z_k, status, (hipStream_t)stream);
+  if (e == hipSuccess)
+    e = w4k::launch_quantize_rows(mode, v, src_f16, rows, out->D, out->gs, (uint32_t*)out->q_v,
+                                  nullptr, (w4_half*)out->s_v, (uint32_t*)out->z_v, status,
+                                  (hipStream_t)stream);
+  return done("quantize_cache", e);
+}
+
+int w4_quantize_cache_f8(const w4_kv_f8_view* out, const void* k, const void* v, int src_f16,
+                         int* status, w4_stream stream) {
+  REQUIRE(out != nullptr, "quantize_cache_f8: null view");
+  REQUIRE(out->H >= 1 && out->S >= 1 && out->D >= 1, "quantize_cache_f8: bad dims");
+  REQUIRE(out->gs >= 8 && out->gs % 8 == 0, "quantize_cache_f8: gs must be a multiple of 8");
+  REQUIRE(out->G == (out->D + out->gs - 1) / out->gs,
+          "quantize_cache_f8: G inconsistent with D, gs");
+  REQUIRE(out->q_k && out->s_k && out->q_v && out->s_v && k && v && status,
+          "quantize_cache_f8: null pointer");
+  if (int rc = start_status(status, stream, "quantize_cache_f8")) return rc;
+  const long long rows = (long long)out->H * out->S;
+  hipError_t e = w4k::launch_quantize_rows(2, k, src_f16, rows, out->D, out->gs, nullptr,
+                                           (uint8_t*)out->q_k, (w4_half*)out->s_k, nullptr,
+                                           status, (hipStream_t)stream);
+  if (e == hipSuccess)
+    e = w4k::launch_quantize_rows(2, v, src_f16, rows, out->D, out->gs, nullptr,
+                                  (uint8_t*)out->q_v, (w4_half*)out->s_v, nullptr, status,
+                                  (hipStream_t)stream);
+  return done("quantize_cache_f8", e);
+}
+
 }  // extern "C"
 
 // ---- two-pass baseline -------------------------------------------------------------

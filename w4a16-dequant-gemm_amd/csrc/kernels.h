@@ -80,4 +80,15 @@ bool try_flash_mfma(const FlashArgs& a, const FlashPlan& pl, float* part, hipStr
 size_t flash_scratch_floats(const FlashArgs& a);
 hipError_t launch_flash(const FlashArgs& a, float* scratch, hipStream_t s);
 
+// quantize.hip -- the host quantizers as kernels.  mode: 0 W4 symmetric, 1 W4 with
+// zero-points, 2 E4M3 bytes; src is FP64 or (src_f16) FP16; `rows` rows of K
+// elements, groups of gs along K.  status: bit 0 non-finite input, bit 1 scale
+// out of range (OR-ed in by the kernels).
+hipError_t launch_quantize_rows(int mode, const void* src, int src_f16, long long rows, int K,
+                                int gs, uint32_t* q32, uint8_t* q8, w4_half* scales,
+                                uint32_t* zeros, int* status, hipStream_t s);
+hipError_t launch_quantize_mx(const void* src, int src_f16, long long rows, int K, uint32_t* q,
+                              uint8_t* scales, int* status, hipStream_t s);
+hipError_t launch_fill_words(uint32_t* p, long long n, uint32_t value, hipStream_t s);
+
 }  // namespace w4k

@@ -161,12 +161,25 @@ int w4_quantize(const w4_packed_view* out, const double* w, int* status,
 /* include/w4/mx.hpp:71-119 */
 int w4_quantize_mx(const w4_packed_mx_view* out, const double* w, int* status,
                    w4_stream stream);
+/* the same quantizer over FP16 sources (activations): out->N rows of out->K */
+int w4_quantize_mx_f16(const w4_packed_mx_view* out, const w4_half* x,
+                       int* status, w4_stream stream);
 /* include/w4/kvcache.hpp:60-108; k, v: H*S*D elements, head- then row-major */
 int w4_quantize_cache(const w4_kv_view* out, const void* k, const void* v,
                       int src_f16, int* status, w4_stream stream);
 /* include/w4/kvfp8.hpp:70-128 */
 int w4_quantize_cache_f8(const w4_kv_f8_view* out, const void* k, const void* v,
                          int src_f16, int* status, w4_stream stream);
+
+/* ---- W4A4 on the scaled matrix cores (no counterpart in the reference, whose
+ * MXFP4 kernels keep FP16 activations: include/w4/mxfused.cuh:166-198,291-307).
+ * c[M,N] = X[M,K] * W[N,K]^T with both operands packed MXFP4 (x->N = M rows,
+ * x->K == w->K).  E2M1 products and E8M0 scales are exact; accumulation is
+ * FP32, the output FP16.  Its gate is separate from the W4A16 one: rel L2
+ * <= 1e-3 against the FP64 product of the two dequantized operands.  Codes
+ * past K in a row's last word are ignored. */
+int w4_gemm_mx_w4a4(const w4_packed_mx_view* w, const w4_packed_mx_view* x,
+                    w4_half* c, w4_stream stream);
 
 #ifdef __cplusplus
 }

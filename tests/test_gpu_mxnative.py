@@ -1,0 +1,134 @@
+"""GPU gates for the W4A4 path: both operands packed MXFP4, scaled matrix cores.
+
+Separate from the W4A16 gates (the activations are quantized too, so the result is
+a different number): the activation quantizer must write the host quantize_mx bytes
+(mx.hpp:71-119) for the FP16 activations widened to FP64, and the GEMM must be within
+rel L2 1e-3 of the FP64 product of the two dequantized operands (dequant_all_mx,
+mx.hpp:131-140, and gemm_oracle, pack.hpp:150-170).  Where every partial sum is
+exactly representable the result must match bit for bit.
+"""
+import numpy as np
+import pytest
+import torch
+
+import orc
+import w4amd
+from devutil import DEV, DevPackedMx, bits, halves, ptr, to_dev
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+SHAPES = [(1, 64, 512), (16, 256, 4096), (5, 100, 1000), (3, 48, 100), (33, 80, 640),
+          (64, 128, 1024), (100, 64, 512), (17, 1024, 2048), (2, 33, 31), (48, 16, 96),
+          (1, 16, 8), (200, 200, 200)]
+
+
+def _quantize_x_on_device(x16, M, K):
+    c = w4amd.capi()
+    B = (K + 31) // 32
+    q = torch.full((M * orc.words(K),), 0x5A5A5A5A, dtype=torch.int32, device=DEV)
+    s = torch.full((M * B,), 0x5A, dtype=torch.uint8, device=DEV)
+    st = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+    xd = to_dev(x16)
+    view = c.packed_mx_view(M, K, B, ptr(q), ptr(s))
+    c.quantize_mx_f16(view, ptr(xd), ptr(st))
+    torch.cuda.synchronize()
+    assert int(st.item()) == 0
+    return view, q, s
+
+
+@pytest.mark.parametrize("i", range(len(SHAPES)))
+def test_w4a4_matches_fp64_product(i):
+    M, N, K = SHAPES[i]
+    c = w4amd.capi()
+    w = orc.normal_weights(N * K, 0x4A4 + i)
+    x16 = orc.normal_activations(M * K, 0x4A5 + i)  # FP16 bit patterns
+    xf = x16.view(np.float16).astype(np.float64)
+    wq, xq = orc.quantize_mx(w, N, K), orc.quantize_mx(xf, M, K)
+    ref = orc.gemm_oracle(orc.dequant_all_mx(xq), M, K, orc.dequant_all_mx(wq), N)
+    # activations quantized on the device: the host's bytes
+    xview, xq_d, xs_d = _quantize_x_on_device(x16, M, K)
+    assert np.array_equal(xq_d.cpu().numpy().view(np.uint32), xq.q)
+    assert np.array_equal(xs_d.cpu().numpy(), xq.scales)
+    dw = DevPackedMx(wq)
+    out = halves(M * N, 0x7E00)
+    c.gemm_mx_w4a4(dw.view, xview, ptr(out))
+    got = bits(out).view(np.float16).astype(np.float64).reshape(M, N)
+    assert orc.rel_l2(got, ref) <= TOL
+    # codes past K in the last word of a row are ignored
+    if K % 8:
+        junk = np.uint32(0xFFFFFFFF) << np.uint32(4 * (K % 8))
+        wq.q.reshape(N, -1)[:, -1] |= junk
+        xq.q.reshape(M, -1)[:, -1] |= junk
+        dw2, dx2 = DevPackedMx(wq), DevPackedMx(xq)
+        out2 = halves(M * N, 0x7E00)
+        c.gemm_mx_w4a4(dw2.view, dx2.view, ptr(out2))
+        assert np.array_equal(bits(out2), bits(out))
+
+
+E2M1 = np.array([0, .5, 1, 1.5, 2, 3, 4, 6, -0., -.5, -1, -1.5, -2, -3, -4, -6])
+
+
+def _decode(p, rows):
+    """E2M1 table times 2^(byte - 127), in FP64 (no FP16 rounding of the operands)."""
+    K = p.K
+    codes = (p.q.reshape(rows, -1)[:, :, None] >> (4 * np.arange(8, dtype=np.uint32))) & 0xF
+    vals = E2M1[codes.reshape(rows, -1)[:, :K]]
+    scale = np.ldexp(1.0, p.scales.reshape(rows, -1).astype(np.int64) - 127)
+    return vals * np.repeat(scale, 32, axis=1)[:, :K]
+
+
+@pytest.mark.parametrize("M,N,K", [(16, 64, 512), (7, 40, 1536), (20, 24, 200)])
+def test_w4a4_exact_when_sums_are_representable(M, N, K):
+    """Codes in {0, +-0.5, +-1} with unit scales: every partial sum is a multiple of 0.25
+    below 2048, exact in FP32 and FP16, so the output bits are determined."""
+    c = w4amd.capi()
+    rng = np.random.default_rng(K)
+    pick = np.array([0, 1, 2, 9, 10], np.uint32)
+    def pack(rows):
+        codes = pick[rng.integers(0, 5, (rows, orc.words(K) * 8))]
+        codes[:, K:] = 0
+        q = (codes.reshape(rows, -1, 8) << (4 * np.arange(8, dtype=np.uint32))).sum(axis=2)
+        return orc.PackedWm(rows, K, q.astype(np.uint32).ravel(),
+                            np.full(rows * ((K + 31) // 32), 127, np.uint8))
+    wq, xq = pack(N), pack(M)
+    ref = _decode(xq, M) @ _decode(wq, N).T
+    assert np.abs(ref).max() < 2048
+    dw, dx = DevPackedMx(wq), DevPackedMx(xq)
+    out = halves(M * N, 0x7E00)
+    c.gemm_mx_w4a4(dw.view, dx.view, ptr(out))
+    assert np.array_equal(bits(out).view(np.float16).reshape(M, N), ref.astype(np.float16))
+
+
+def test_w4a4_block_scales_far_from_fp16():
+    """Weight scales around 2^+20 against activation scales around 2^-20: neither operand
+    is representable in FP16, the products are; the instruction applies the scales exactly."""
+    M, N, K = 12, 48, 1024
+    c = w4amd.capi()
+    rng = np.random.default_rng(3)
+    wq = orc.quantize_mx(orc.normal_weights(N * K, 11), N, K)
+    xq = orc.quantize_mx(orc.normal_weights(M * K, 12), M, K)
+    wq.scales = (wq.scales.astype(np.int64) + rng.integers(15, 25, wq.scales.shape)).astype(np.uint8)
+    xq.scales = (xq.scales.astype(np.int64) - rng.integers(15, 25, xq.scales.shape)).astype(np.uint8)
+    ref = _decode(xq, M) @ _decode(wq, N).T
+    dw, dx = DevPackedMx(wq), DevPackedMx(xq)
+    out = halves(M * N, 0x7E00)
+    c.gemm_mx_w4a4(dw.view, dx.view, ptr(out))
+    got = bits(out).view(np.float16).astype(np.float64).reshape(M, N)
+    assert np.isfinite(got).all()
+    assert orc.rel_l2(got, ref) <= TOL
+
+
+def test_w4a4_decode_shapes_of_the_benchmarks():
+    c = w4amd.capi()
+    for (M, N, K) in [(1, 4096, 4096), (16, 14336, 4096), (64, 4096, 4096)]:
+        w = orc.normal_weights(N * K, N + M)
+        x16 = orc.normal_activations(M * K, K + M)
+        wq = orc.quantize_mx(w, N, K)
+        xq = orc.quantize_mx(x16.view(np.float16).astype(np.float64), M, K)
+        ref = orc.gemm_oracle(orc.dequant_all_mx(xq), M, K, orc.dequant_all_mx(wq), N)
+        dw, dx = DevPackedMx(wq), DevPackedMx(xq)
+        out = halves(M * N, 0x7E00)
+        c.gemm_mx_w4a4(dw.view, dx.view, ptr(out))
+        got = bits(out).view(np.float16).astype(np.float64).reshape(M, N)
+        assert orc.rel_l2(got, ref) <= TOL, (M, N, K)

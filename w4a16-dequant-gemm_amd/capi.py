@@ -59,6 +59,8 @@ SIGNATURES = {
                                              C.c_int, vp, vp, vp], C.c_int),
     "w4_quantize": ([C.POINTER(PackedView), vp, vp, vp], C.c_int),
     "w4_quantize_mx": ([C.POINTER(PackedMxView), vp, vp, vp], C.c_int),
+    "w4_quantize_mx_f16": ([C.POINTER(PackedMxView), vp, vp, vp], C.c_int),
+    "w4_gemm_mx_w4a4": ([C.POINTER(PackedMxView), C.POINTER(PackedMxView), vp, vp], C.c_int),
     "w4_quantize_cache": ([C.POINTER(KVView), vp, vp, C.c_int, vp, vp], C.c_int),
     "w4_quantize_cache_f8": ([C.POINTER(KVF8View), vp, vp, C.c_int, vp, vp], C.c_int),
 }
@@ -194,3 +196,12 @@ def quantize_cache(view, k, v, status, src_f16=False, stream=0):
 def quantize_cache_f8(view, k, v, status, src_f16=False, stream=0):
     check(load().w4_quantize_cache_f8(C.byref(view), _n(k), _n(v), int(src_f16), _n(status),
                                       _n(stream)))
+
+
+def quantize_mx_f16(view, x, status, stream=0):
+    check(load().w4_quantize_mx_f16(C.byref(view), _n(x), _n(status), _n(stream)))
+
+
+def gemm_mx_w4a4(w_view, x_view, c, stream=0):
+    """Both operands packed MXFP4 (x_view.N = M); scaled matrix cores."""
+    check(load().w4_gemm_mx_w4a4(C.byref(w_view), C.byref(x_view), _n(c), _n(stream)))

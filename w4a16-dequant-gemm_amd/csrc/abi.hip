@@ -372,6 +372,30 @@ int w4_quantize_mx(const w4_packed_mx_view* out, const double* w, int* status,
                                       (uint8_t*)out->scales, status, (hipStream_t)stream));
 }
 
+int w4_quantize_mx_f16(const w4_packed_mx_view* out, const w4_half* x, int* status,
+                       w4_stream stream) {
+  REQUIRE(out != nullptr, "quantize_mx: null view");
+  REQUIRE(out->N >= 1 && out->K >= 1, "quantize_mx: bad dims");
+  REQUIRE(out->B == (out->K + 31) / 32, "quantize_mx: B inconsistent with K");
+  REQUIRE(out->q && out->scales && x && status, "quantize_mx: null pointer");
+  if (int rc = start_status(status, stream, "quantize_mx")) return rc;
+  return done("quantize_mx",
+              w4k::launch_quantize_mx(x, 1, out->N, out->K, (uint32_t*)out->q,
+                                      (uint8_t*)out->scales, status, (hipStream_t)stream));
+}
+
+// ---- W4A4 on the scaled matrix cores ---------------------------------------------
+
+int w4_gemm_mx_w4a4(const w4_packed_mx_view* w, const w4_packed_mx_view* x, w4_half* c,
+                    w4_stream stream) {
+  if (int rc = check_mx(w)) return rc;
+  if (int rc = check_mx(x)) return rc;
+  REQUIRE(w->K == x->K, "mx w4a4: operands disagree on K");
+  REQUIRE(c != nullptr, "mx w4a4: null pointer");
+  REQUIRE(x->N <= 65535LL * 64, "mx w4a4: launch grid out of range");
+  return done("gemm_mx_w4a4", w4k::launch_gemm_mx_w4a4(*w, *x, c, (hipStream_t)stream));
+}
+
 int w4_quantize_cache(const w4_kv_view* out, const void* k, const void* v, int src_f16,
                       int* status, w4_stream stream) {
   REQUIRE(out != nullptr, "quantize_cache: null view");

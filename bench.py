@@ -74,6 +74,33 @@ class Bench:
         self.yard.w4bench_gemm_loop.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p,
                                                 C.c_int, C.c_int, C.c_void_p]
 
+    def w4a4_us(self, views, M, N, K, reps=5):
+        """us per w4_gemm_mx_w4a4 call over rotating weight copies (C loop, HIP events)."""
+        torch = self.torch
+        xv = self.rand_mx(M, K, 1)[0]
+        c = torch.empty(M * N, dtype=torch.float16, device="cuda")
+        fn = C.cast(self.capi.load().w4_gemm_mx_w4a4, C.c_void_p)
+        arr = (C.c_void_p * len(views))(*[C.addressof(v[0]) for v in views])
+        self.yard.w4bench_w4a4_loop.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p,
+                                                C.c_int, C.c_void_p]
+
+        def run(n):
+            rc = self.yard.w4bench_w4a4_loop(fn, arr, len(views), C.addressof(xv[0]), c.data_ptr(), n,
+                                             self.stream)
+            if rc:
+                raise RuntimeError("w4a4 loop failed: %d" % rc)
+        run(self.warmup)
+        torch.cuda.synchronize()
+        out = []
+        for _ in range(reps):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            run(self.steps)
+            b.record()
+            torch.cuda.synchronize()
+            out.append(a.elapsed_time(b) / self.steps * 1e3)
+        return sorted(out)[len(out) // 2]
+
     def loop_ms(self, entry, views, x_ptr, c_ptr, M, steps, warmup, reps=5):
         """Mean ms per call over `steps` launches issued by a C loop (no
         interpreter between launches), HIP events on the launch stream; median of reps."""
@@ -357,6 +384,22 @@ def extras_attention(b, full):
     return {"c5_flash_decode": res}
 
 
+def extras_w4a4(b, full):
+    """Both operands MXFP4 on the scaled matrix cores (separately gated W4A4 entry)."""
+    torch = b.torch
+    rows = []
+    for (N, K) in ((4096, 4096), (14336, 4096)):
+        views = b.rand_mx(N, K, max(2, int(400e6 // mx_bytes(N, K, 1)) + 1))
+        for M in ((1, 16, 64, 256) if not full else (1, 8, 16, 32, 64, 128, 256)):
+            nb = mx_bytes(N, K, 0) + M * (K // 2 + K // 32) + 2 * M * N
+            us = b.w4a4_us(views, M, N, K)
+            rows.append({"N": N, "K": K, "M": M, "bytes": nb, "us": us, "GBs": nb / us * 1e-3,
+                         "TFLOPs": 2.0 * M * N * K / us * 1e-6})
+        del views
+        torch.cuda.empty_cache()
+    return {"w4a4_mxfp4": rows}
+
+
 def extras_quantize(b, full):
     """Device-side quantizers (memory-bound streams): bytes read + written per call over the
     call's duration.  Sources: FP64 weights (as the host quantizers take them), FP16 K/V rows."""
@@ -473,6 +516,7 @@ def main():
         extra.update(extras_gemm(b, args.extras == "full"))
         extra.update(extras_attention(b, args.extras == "full"))
         extra.update(extras_quantize(b, args.extras == "full"))
+        extra.update(extras_w4a4(b, args.extras == "full"))
     cpu = h["cpu"]
     line = {
         "metric": "M=1 W4 GEMM us + achieved HBM GB/s (% of peak); M=2048 MFMA TFLOP/s",

@@ -54,3 +54,14 @@ extern "C" int w4bench_gemm_loop(w4bench_gemm_fn fn, const void* const* views, i
   }
   return 0;
 }
+
+// The same loop for the two-view W4A4 entry point.
+typedef int (*w4bench_w4a4_fn)(const void* w_view, const void* x_view, void* c, void* stream);
+extern "C" int w4bench_w4a4_loop(w4bench_w4a4_fn fn, const void* const* views, int nviews,
+                                 const void* x_view, void* c, int steps, void* stream) {
+  for (int i = 0; i < steps; ++i) {
+    const int rc = fn(views[i % nviews], x_view, c, stream);
+    if (rc) return rc;
+  }
+  return 0;
+}

@@ -30,34 +30,38 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 constexpr int NV_WAVES = 8;   // waves of a decode workgroup (they split K)
 constexpr int FMT_FP4 = 4;    // operand format code of the instruction
 
-// One MFMA over the 32-blocks picked by SEL: byte SEL of each lane's scale word.
-template <int SEL>
+// One MFMA over 128 k: every lane brings 32 codes and, in byte 0 of its scale
+// register, the E8M0 byte of that 32-block.
 __device__ __forceinline__ f4 mfma_fp4(u4 a, uint32_t sa, u4 b, uint32_t sb, f4 c) {
   const v4i a4 = __builtin_bit_cast(v4i, a), b4 = __builtin_bit_cast(v4i, b);
   // FP4 operands occupy the low four of the eight operand registers
   const v8i va = __builtin_shufflevector(a4, a4, 0, 1, 2, 3, -1, -1, -1, -1);
   const v8i vb = __builtin_shufflevector(b4, b4, 0, 1, 2, 3, -1, -1, -1, -1);
-  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(va, vb, c, FMT_FP4, FMT_FP4, SEL,
-                                                          (int)sa, SEL, (int)sb);
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(va, vb, c, FMT_FP4, FMT_FP4, 0,
+                                                          (int)sa, 0, (int)sb);
 }
 
-// The four consecutive 32-blocks b0..b0+3 of one packed row (64 bytes of codes)
-// and their four scale bytes as one word.  FULL: every block exists and rows
-// are 16-byte aligned.  Otherwise words past the row read as zero codes, codes
-// past K are masked off, and missing blocks take the neutral scale byte 127.
+// A lane's share of one 512-k super-step of a packed row: block 4j + g of the
+// super-step for j = 0..3 (g = lane / 16), so that load j of the four lane
+// groups covers one contiguous 64-byte piece of every row, and MFMA j contracts
+// 128 consecutive k.  sc[j] carries the block's scale in byte 0.  FULL: every
+// block exists and rows are 16-byte aligned.  Otherwise words past the row read
+// as zero codes, codes past K are masked off, and missing blocks take the
+// neutral scale byte 127.
 template <bool FULL>
 __device__ __forceinline__ void load_blocks(const uint32_t* __restrict__ qrow,
-                                            const uint8_t* __restrict__ srow, int b0, int B,
-                                            int wk, int K, u4 q[4], uint32_t& sc) {
+                                            const uint8_t* __restrict__ srow, int ss, int g,
+                                            int B, int wk, int K, u4 q[4], uint32_t sc[4]) {
   if (FULL) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) q[j] = *(const u4*)(qrow + (size_t)(b0 + j) * 4);
-    sc = *(const uint32_t*)(srow + b0);
+    for (int j = 0; j < 4; ++j) q[j] = *(const u4*)(qrow + (size_t)(ss * 16 + 4 * j + g) * 4);
+    const u4 s16 = *(const u4*)(srow + ss * 16);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sc[j] = s16[j] >> (8 * g);
   } else {
-    sc = 0;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int b = b0 + j;
+      const int b = ss * 16 + 4 * j + g;
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         const int wi = b * 4 + t;
@@ -65,30 +69,34 @@ __device__ __forceinline__ void load_blocks(const uint32_t* __restrict__ qrow,
         if (wi == wk - 1 && (K & 7)) word &= (1u << (4 * (K & 7))) - 1u;
         q[j][t] = word;
       }
-      sc |= (uint32_t)(b < B ? srow[b] : (uint8_t)127) << (8 * j);
+      sc[j] = b < B ? srow[b] : 127u;
     }
   }
 }
 
-// Skinny M: a workgroup owns 16 rows of W and 16*MT rows of X (grid.y walks
-// further X rows); its 8 waves take 512-k super-steps round-robin.  Inside a
-// super-step lane group g = l/16 holds blocks 4g..4g+3 of its row, and MFMA j
-// contracts block 4g+j of every group: the k order inside a super-step is
-// permuted identically for both operands.  Partial sums meet in LDS and are
-// added in wave order.
-template <int MT, bool FULL>
+// Skinny M: a workgroup owns 16*NT rows of W and 16*MT rows of X (grid.y walks
+// further X rows); its 8 waves take 512-k super-steps round-robin.  A wave
+// loads the X pieces of its super-step once and reuses them for the NT row
+// tiles, so X crosses L2 -> CU once per workgroup.  Partial sums meet in LDS
+// and are added in wave order.
+template <int MT, int NT, bool FULL>
 __global__ __launch_bounds__(NV_WAVES * 64) void mxn_decode_kernel(
     const uint32_t* __restrict__ wq, const uint8_t* __restrict__ ws,
     const uint32_t* __restrict__ xq, const uint8_t* __restrict__ xs, w4_half* __restrict__ c,
     int N, int K, int B, int M) {
-  __shared__ f4 red[NV_WAVES][MT][64];
+  __shared__ f4 red[NV_WAVES][NT * MT][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int wk = words(K);
-  const int n0 = blockIdx.x * 16, m0 = blockIdx.y * (16 * MT);
-  const int n = n0 + r < N ? n0 + r : N - 1;
-  const uint32_t* wrow = wq + (size_t)n * wk;
-  const uint8_t* wsrow = ws + (size_t)n * B;
+  const int n0 = blockIdx.x * (16 * NT), m0 = blockIdx.y * (16 * MT);
+  const uint32_t* wrow[NT];
+  const uint8_t* wsrow[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int n = n0 + nt * 16 + r < N ? n0 + nt * 16 + r : N - 1;
+    wrow[nt] = wq + (size_t)n * wk;
+    wsrow[nt] = ws + (size_t)n * B;
+  }
   const uint32_t* xrow[MT];
   const uint8_t* xsrow[MT];
 #pragma unroll
@@ -97,37 +105,45 @@ __global__ __launch_bounds__(NV_WAVES * 64) void mxn_decode_kernel(
     xrow[mt] = xq + (size_t)m * wk;
     xsrow[mt] = xs + (size_t)m * B;
   }
-  f4 acc[MT];
+  f4 acc[NT][MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = f4{0.f, 0.f, 0.f, 0.f};
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = f4{0.f, 0.f, 0.f, 0.f};
 
   const int supers = (B + 15) >> 4;
   for (int ss = wave; ss < supers; ss += NV_WAVES) {
-    const int b0 = ss * 16 + g * 4;
-    u4 a[4];
-    uint32_t sa;
-    load_blocks<FULL>(wrow, wsrow, b0, B, wk, K, a, sa);
+    u4 b[MT][4], a[NT][4];
+    uint32_t sb[MT][4], sa[NT][4];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      u4 b[4];
-      uint32_t sb;
-      load_blocks<FULL>(xrow[mt], xsrow[mt], b0, B, wk, K, b, sb);
-      acc[mt] = mfma_fp4<0>(a[0], sa, b[0], sb, acc[mt]);
-      acc[mt] = mfma_fp4<1>(a[1], sa, b[1], sb, acc[mt]);
-      acc[mt] = mfma_fp4<2>(a[2], sa, b[2], sb, acc[mt]);
-      acc[mt] = mfma_fp4<3>(a[3], sa, b[3], sb, acc[mt]);
-    }
+    for (int nt = 0; nt < NT; ++nt)
+      load_blocks<FULL>(wrow[nt], wsrow[nt], ss, g, B, wk, K, a[nt], sa[nt]);
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      load_blocks<FULL>(xrow[mt], xsrow[mt], ss, g, B, wk, K, b[mt], sb[mt]);
+    // every load of the super-step is in flight before the first product waits
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[nt][mt] = mfma_fp4(a[nt][j], sa[nt][j], b[mt][j], sb[mt][j], acc[nt][mt]);
   }
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) red[wave][mt][lane] = acc[mt];
-  __syncthreads();
-  // MT * 64 lane slots of four n each
-  for (int o = threadIdx.x; o < MT * 64; o += NV_WAVES * 64) {
-    const int mt = o >> 6, l = o & 63;
-    f4 sum = red[0][mt][l];
+  for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-    for (int w = 1; w < NV_WAVES; ++w) sum += red[w][mt][l];
-    const int m = m0 + mt * 16 + (l & 15), nn = n0 + 4 * (l >> 4);
+    for (int mt = 0; mt < MT; ++mt) red[wave][nt * MT + mt][lane] = acc[nt][mt];
+  __syncthreads();
+  // NT * MT * 64 lane slots of four n each
+  for (int o = threadIdx.x; o < NT * MT * 64; o += NV_WAVES * 64) {
+    const int t = o >> 6, l = o & 63;
+    const int nt = t / MT, mt = t - nt * MT;
+    f4 sum = red[0][t][l];
+#pragma unroll
+    for (int w = 1; w < NV_WAVES; ++w) sum += red[w][t][l];
+    const int m = m0 + mt * 16 + (l & 15), nn = n0 + nt * 16 + 4 * (l >> 4);
     if (m >= M) continue;
     w4_half* dst = c + (size_t)m * N + nn;
     if (nn + 3 < N && ((uintptr_t)dst & 7) == 0) {
@@ -145,21 +161,37 @@ __global__ __launch_bounds__(NV_WAVES * 64) void mxn_decode_kernel(
   }
 }
 
+template <int MT, int NT>
+hipError_t launch_decode_nt(const w4_packed_mx_view& w, const w4_packed_mx_view& x, w4_half* c,
+                            hipStream_t s) {
+  const int N = w.N, K = w.K, M = x.N;
+  const bool full = K % 512 == 0 && ((uintptr_t)w.q & 15) == 0 && ((uintptr_t)x.q & 15) == 0 &&
+                    ((uintptr_t)w.scales & 15) == 0 && ((uintptr_t)x.scales & 15) == 0;
+  const dim3 grid((unsigned)((N + 16 * NT - 1) / (16 * NT)),
+                  (unsigned)((M + 16 * MT - 1) / (16 * MT)));
+  const dim3 block(NV_WAVES * 64);
+  if (full)
+    mxn_decode_kernel<MT, NT, true><<<grid, block, 0, s>>>(w.q, w.scales, x.q, x.scales, c, N,
+                                                          K, w.B, M);
+  else
+    mxn_decode_kernel<MT, NT, false><<<grid, block, 0, s>>>(w.q, w.scales, x.q, x.scales, c, N,
+                                                           K, w.B, M);
+  return hipGetLastError();
+}
+
+// Row tiles per workgroup: as many as keep at least one workgroup per CU.
 template <int MT>
 hipError_t launch_decode(const w4_packed_mx_view& w, const w4_packed_mx_view& x, w4_half* c,
                          hipStream_t s) {
-  const int N = w.N, K = w.K, M = x.N;
-  const bool full = K % 512 == 0 && ((uintptr_t)w.q & 15) == 0 && ((uintptr_t)x.q & 15) == 0 &&
-                    ((uintptr_t)w.scales & 3) == 0 && ((uintptr_t)x.scales & 3) == 0;
-  const dim3 grid((unsigned)((N + 15) / 16), (unsigned)((M + 16 * MT - 1) / (16 * MT)));
-  const dim3 block(NV_WAVES * 64);
-  if (full)
-    mxn_decode_kernel<MT, true><<<grid, block, 0, s>>>(w.q, w.scales, x.q, x.scales, c, N, K,
-                                                      w.B, M);
-  else
-    mxn_decode_kernel<MT, false><<<grid, block, 0, s>>>(w.q, w.scales, x.q, x.scales, c, N, K,
-                                                       w.B, M);
-  return hipGetLastError();
+  const int tiles = (w.N + 15) / 16;
+  const int mblocks = (x.N + 16 * MT - 1) / (16 * MT);
+  // more row tiles per workgroup cut the X traffic, but only pay while several
+  // workgroups per CU remain (a second, partly filled round of fat workgroups
+  // costs more than it saves)
+  const int nt = MT >= 3 ? tiles * mblocks / 512 : 1;
+  if (nt >= 3) return launch_decode_nt<MT, 3>(w, x, c, s);
+  if (nt >= 2) return launch_decode_nt<MT, 2>(w, x, c, s);
+  return launch_decode_nt<MT, 1>(w, x, c, s);
 }
 
 }  // namespace

@@ -20,7 +20,12 @@ TOL = 1e-3
 
 SHAPES = [(1, 64, 512), (16, 256, 4096), (5, 100, 1000), (3, 48, 100), (33, 80, 640),
           (64, 128, 1024), (100, 64, 512), (17, 1024, 2048), (2, 33, 31), (48, 16, 96),
-          (1, 16, 8), (200, 200, 200)]
+          (1, 16, 8), (200, 200, 200),
+          # a few hundred rows on the skinny kernel's grid.y walk
+          (128, 256, 512), (96, 64, 128), (200, 300, 1024), (300, 520, 384), (129, 257, 256),
+          # K % 256 == 0 and M >= 384: the LDS-tiled kernel (ragged tiles on both sides, step
+          # counts that are and are not multiples of the unrolled loop body)
+          (384, 256, 512), (500, 300, 1024), (385, 520, 256), (700, 257, 768), (400, 64, 1280)]
 
 
 def _quantize_x_on_device(x16, M, K):
@@ -132,3 +137,22 @@ def test_w4a4_decode_shapes_of_the_benchmarks():
         c.gemm_mx_w4a4(dw.view, dx.view, ptr(out))
         got = bits(out).view(np.float16).astype(np.float64).reshape(M, N)
         assert orc.rel_l2(got, ref) <= TOL, (M, N, K)
+
+
+def test_w4a4_prefill_shape_sampled_rows():
+    """M = 2048, N = K = 4096: every output element of 96 sampled activation rows against
+    the FP64 product (the full FP64 product is 3.4e10 multiply-adds)."""
+    M, N, K = 2048, 4096, 4096
+    c = w4amd.capi()
+    wq = orc.quantize_mx(orc.normal_weights(N * K, 21), N, K)
+    x16 = orc.normal_activations(M * K, 22)
+    xq = orc.quantize_mx(x16.view(np.float16).astype(np.float64), M, K)
+    dw, dx = DevPackedMx(wq), DevPackedMx(xq)
+    out = halves(M * N, 0x7E00)
+    c.gemm_mx_w4a4(dw.view, dx.view, ptr(out))
+    got = bits(out).view(np.float16).astype(np.float64).reshape(M, N)
+    rows = np.unique(np.concatenate([np.arange(0, 16), np.arange(M - 16, M),
+                                     np.random.default_rng(5).integers(0, M, 64)]))
+    ref = _decode(xq, M)[rows] @ _decode(wq, N).T
+    assert orc.rel_l2(got[rows], ref) <= TOL
+    assert np.isfinite(got).all()

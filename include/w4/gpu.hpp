@@ -350,4 +350,22 @@ inline void quantize_cache_f8(const DeviceKVF8& out, const double* k, const doub
                        "quantize_cache_f8: group scale outside FP16 range");
 }
 
+// ---- W4A4 on the scaled matrix cores (additive; the reference's MXFP4 kernels
+// keep FP16 activations, mxfused.cuh:166-198,291-307) --------------------------
+// Activations are quantized to MXFP4 like weights (same bytes as mx::quantize_mx
+// of the FP16 values widened to FP64), then c[M,N] = X * W^T runs on packed
+// operands: exact products, FP32 accumulation, FP16 output.  x.N is M.  Its
+// gate is its own: rel L2 <= 1e-3 against gemm_oracle over the two dequantized
+// operands.
+inline void quantize_mx_f16_async(const DevicePackedWm& out, const __half* x, int* status,
+                                  hipStream_t stream = 0) {
+  const auto v = detail::abi(out);
+  detail::raise(w4_quantize_mx_f16(&v, detail::h(x), status, stream));
+}
+inline void gemm_mx_w4a4(const DevicePackedWm& w, const DevicePackedWm& x, __half* c,
+                         hipStream_t stream = 0) {
+  const auto vw = detail::abi(w), vx = detail::abi(x);
+  detail::raise(w4_gemm_mx_w4a4(&vw, &vx, detail::h(c), stream));
+}
+
 }  // namespace w4::gpu

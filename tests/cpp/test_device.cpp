@@ -351,6 +351,31 @@ void quantizer_gates(Checks& t) {
   }
 }
 
+// W4A4: activations quantized on the device equal the host quantizer's bytes, and
+// the product of the two packed operands is within 1e-3 of the FP64 product of
+// their dequantized values (mx.hpp:131-140, pack.hpp:150-170).
+void w4a4_gates(Checks& t) {
+  Dev<int> status(1);
+  const Shape shapes[] = {{5, 100, 1000, 0}, {64, 128, 1024, 0}, {400, 300, 512, 0}};
+  for (const Shape& c : shapes) {
+    const mx::PackedWm w = mx::quantize_mx(normal_weights(c.N * c.K, 31), c.N, c.K);
+    const auto x16 = normal_activations(c.M * c.K, 32);
+    std::vector<double> xd(x16.size());
+    for (size_t i = 0; i < xd.size(); ++i) xd[i] = (double)__half2float(x16[i]);
+    const mx::PackedWm xq = mx::quantize_mx(xd, c.M, c.K);
+    const auto ref = gemm_oracle(mx::dequant_all_mx(xq), c.M, c.K, mx::dequant_all_mx(w), c.N);
+    Dev<uint32_t> wq(w.q), xqd(xq.q.size());
+    Dev<uint8_t> wsc(w.scales), xsd(xq.scales.size());
+    Dev<__half> x(x16), out((size_t)c.M * c.N);
+    const DevicePackedWm dw{c.N, c.K, w.B, wq.p, wsc.p}, dx{c.M, c.K, xq.B, xqd.p, xsd.p};
+    quantize_mx_f16_async(dx, x.p, status.p);
+    t.expect(same(xqd.get(), xq.q) && same(xsd.get(), xq.scales) && status.get()[0] == 0,
+             "activations quantized on the device: host bytes");
+    gemm_mx_w4a4(dw, dx, out.p);
+    oracle_gate(t, out.get(), ref, "W4A4 product vs FP64 product of the dequantized operands");
+  }
+}
+
 }  // namespace
 
 int main() {
@@ -363,6 +388,7 @@ int main() {
   gemm_gates(t);
   attention_gates(t);
   quantizer_gates(t);
+  w4a4_gates(t);
   std::printf("worst rel L2 vs the FP64 references = %.3e\n", g_worst);
   return t.finish("device");
 }

@@ -66,3 +66,13 @@ def test_quantize_contracts():
         c.quantize_cache_f8(c.kv_f8_view(1, 1, 64, 16, 4, one, one, one, one), 0, one, one)
     with pytest.raises(ValueError, match="G inconsistent"):
         c.quantize_cache_f8(c.kv_f8_view(1, 1, 64, 16, 3, one, one, one, one), one, one, one)
+    # W4A4: both views checked, K must agree
+    w, x = c.packed_mx_view(8, 64, 2, one, one), c.packed_mx_view(2, 32, 1, one, one)
+    with pytest.raises(ValueError, match="disagree on K"):
+        c.gemm_mx_w4a4(w, x, one)
+    with pytest.raises(ValueError, match="null pointer"):
+        c.gemm_mx_w4a4(w, c.packed_mx_view(2, 64, 2, one, one), 0)
+    with pytest.raises(ValueError, match="B inconsistent"):
+        c.gemm_mx_w4a4(w, c.packed_mx_view(2, 64, 3, one, one), one)
+    with pytest.raises(ValueError, match="null pointer"):
+        c.quantize_mx_f16(c.packed_mx_view(2, 64, 2, one, one), 0, one)

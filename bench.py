@@ -390,7 +390,7 @@ def extras_w4a4(b, full):
     rows = []
     for (N, K) in ((4096, 4096), (14336, 4096)):
         views = b.rand_mx(N, K, max(2, int(400e6 // mx_bytes(N, K, 1)) + 1))
-        for M in ((1, 16, 64, 256) if not full else (1, 8, 16, 32, 64, 128, 256)):
+        for M in ((1, 16, 64, 256, 2048) if not full else (1, 8, 16, 32, 64, 128, 256, 512, 2048, 8192)):
             nb = mx_bytes(N, K, 0) + M * (K // 2 + K // 32) + 2 * M * N
             us = b.w4a4_us(views, M, N, K)
             rows.append({"N": N, "K": K, "M": M, "bytes": nb, "us": us, "GBs": nb / us * 1e-3,

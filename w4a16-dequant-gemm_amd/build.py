@@ -19,6 +19,8 @@ FLAGS = [
     # packed-FP32 VALU forms stay off for every kernel in this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
+    # the direct-to-LDS loads name M0 in their clobber list on purpose
+    "-Wno-inline-asm",
 ]
 
 

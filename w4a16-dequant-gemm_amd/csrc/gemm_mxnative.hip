@@ -195,32 +195,11 @@ hipError_t launch_decode(const w4_packed_mx_view& w, const w4_packed_mx_view& x,
 }
 
 // ---- large M: LDS-tiled kernel -----------------------------------------------
-// Uses the 32x32x64 form of the instruction (measured 8.1 PFLOP/s on FP4 against
+// Uses the 32x32x64 form of the instruction (measured 7.9 PFLOP/s on FP4 against
 // 5.8 for 16x16x128; same lane scheme: A lane l = row l%32, k-block l/32; D lane
-// l = column l%32, rows 4*(l/32) + e%4 + 8*(e/4), e = 0..15).
-//
-// A workgroup of 4 waves (2 x 2) owns 256 rows of W x 128 rows of X; a wave 128 x
-// 64 = 4 x 2 MFMA tiles, two MFMAs deep per 128-k step (8 waves of 64 x 64
-// measured the same).  Memory is read 256 k at a
-// time -- 8 threads take the 128 bytes of a row, so every cache line that crosses
-// L2 -> CU is used whole (with 64-byte pieces each line crossed twice and the L2
-// bandwidth, not the matrix pipe, set the pace) -- into a ring of TL_PAIRS register
-// slots, and goes on to LDS still packed, one 128-k half per step (64 bytes a row,
-// rows padded to 80 so that 16 rows x 16 bytes fall on distinct banks); a lane
-// reads each operand with one ds_read_b128.  Scale bytes travel the same way, one
-// dword (4 blocks) per row and step; a lane shifts its block's byte down.
-// Software pipeline, one barrier per step: while the MFMAs of step k run from
-// registers, the operands of step k+1 are read from one LDS buffer and step k+2
-// is written into the other.
+// l = column l%32, rows 4*(l/32) + e%4 + 8*(e/4), e = 0..15).  A workgroup owns
+// 256 rows of W x 128 rows of X.
 constexpr int TL_TN = 256, TL_TM = 128, TL_ROWS = TL_TN + TL_TM;
-constexpr int TL_ROWB = 80;   // LDS bytes per row and step
-constexpr int TL_WN = 2;                       // waves along n (and 2 along m)
-constexpr int TL_THREADS = 64 * TL_WN * 2;
-constexpr int TL_NT = TL_TN / (32 * TL_WN);    // 32-row MFMA tiles of W per wave
-constexpr int TL_RP = TL_THREADS / 4;          // rows one pass of the workgroup fetches
-constexpr int TL_WI = TL_TN / TL_RP, TL_XI = TL_TM / TL_RP;
-constexpr int TL_PAIRS = 2;   // 256-k register slots in flight
-constexpr int TL_STAGE = TL_ROWS * TL_ROWB + TL_ROWS * 4;
 
 typedef float f16v __attribute__((ext_vector_type(16)));
 
@@ -232,161 +211,191 @@ __device__ __forceinline__ f16v mfma_fp4_32(u4 a, uint32_t sa, u4 b, uint32_t sb
                                                          0, (int)sb);
 }
 
-struct TileRegs {  // one thread's share of 256 k on its way to LDS
-  u4 w[2][TL_WI], x[2][TL_XI];  // [128-k half][row t/4 + TL_RP i], 16-byte piece t%4
-  u2 sw, sx;         // the two steps' scale dwords of W row t%256 / X row t%128
-};
-struct TileFrags {  // one lane's MFMA operands of a step: [k half][tile]
-  u4 a[2][TL_NT], b[2][2];
-  uint32_t sa[TL_NT], sb[2];  // the rows' four scale bytes
+// Operands go global -> LDS directly.
+// global_load_lds_dwordx4 writes lane l's 16 bytes to LDS at (wave-uniform base)
+// + 16 l, so a wave instruction fills 1 KB, and which piece of which row a lane
+// fetches is free to choose.  A stage holds 256 k: 128 bytes = one cache line per
+// row, so every line crosses L2 -> CU once, whole.  An instruction takes 8 rows;
+// lane l fetches row l/8, piece (l%8) ^ key(row), key(R) = (R/2) % 8: eight
+// neighbouring lanes still cover one contiguous line (coalesced), and the 16
+// rows x 16 bytes a lane group reads back for one MFMA operand land on 16
+// distinct 16-byte bank groups (conflict-free ds_read_b128 without padding).
+// No staging registers, no ds_write instructions: DM_STAGES stages of 256 k sit
+// in LDS (dynamic LDS, 153 KB); one barrier per stage.  Per stage d: multiply
+// the first 128 k of d while reading the operands of the second; wait for d+1,
+// barrier -- every wave is now done with d's buffer, so request d+3 into it;
+// multiply the second 128 k while reading the first operands of d+1.
+constexpr int DM_STAGES = 3;
+constexpr int DM_W_BYTES = TL_TN * 128, DM_X_BYTES = TL_TM * 128;
+constexpr int DM_TILE_BYTES = DM_W_BYTES + DM_X_BYTES;       // 48 KB, unpadded
+constexpr int DM_STAGE = DM_TILE_BYTES + 2 * TL_ROWS * 4;    // + two scale dwords per row
+constexpr int DM_WN = 4;                                     // waves along n (2 along m)
+constexpr int DM_WAVES = 2 * DM_WN;
+constexpr int DM_THREADS = 64 * DM_WAVES;
+constexpr int DM_NT = TL_TN / (32 * DM_WN);                  // 32-row tiles of W per wave
+constexpr int DM_WI = 32 / DM_WAVES, DM_XI = 16 / DM_WAVES;  // 8-row blocks a wave fetches
+constexpr int DM_LOADS = DM_WI + DM_XI + 2;                  // wave instructions per stage
+
+struct DmFrags {  // one lane's MFMA operands of a 128-k half: [k half][tile]
+  u4 a[2][DM_NT], b[2][2];
+  uint32_t sa[DM_NT], sb[2];
 };
 
-template <int PAIRS>
-__global__ __launch_bounds__(TL_THREADS) void mxn_tile_kernel(
+typedef __attribute__((address_space(3))) void* lds_ptr;
+
+// s_waitcnt vmcnt(N) alone (gfx9 encoding: vmcnt in [3:0] and [15:14])
+constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
+
+extern __shared__ __attribute__((aligned(16))) uint8_t dm_lds[];
+
+__global__ __launch_bounds__(DM_THREADS) void mxn_tile_dma_kernel(
     const uint32_t* __restrict__ wq, const uint8_t* __restrict__ ws,
     const uint32_t* __restrict__ xq, const uint8_t* __restrict__ xs, w4_half* __restrict__ c,
     int N, int K, int B, int M, int tiles_n, int tiles_m) {
-  __shared__ __attribute__((aligned(16))) uint8_t lds[2][TL_STAGE];
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // in an SGPR: LDS addresses go to M0
   const int r = lane & 31, h = lane >> 5;
-  const int wn = wave % TL_WN, wm = wave / TL_WN;  // TL_WN x 2 waves
-  // XCD-aware order: consecutive workgroup ids land on different XCDs, so give
-  // each XCD a contiguous run of the tile order (m fastest: its workgroups share
-  // a few W tiles and walk X)
+  const int wn = wave % DM_WN, wm = wave / DM_WN;  // DM_WN x 2 waves
+  // XCD-aware order: consecutive workgroup ids land on different XCDs (each with
+  // its own L2), so give each XCD a contiguous run of the tile order, m fastest:
+  // its workgroups share a few W tiles and walk X.  (Blocks of 4 x 8 tiles per
+  // XCD measured no better.)
   int L = blockIdx.x;
   const int total = tiles_n * tiles_m;
   if (total % 8 == 0) L = (L & 7) * (total >> 3) + (L >> 3);
   const int n0 = (L / tiles_m) * TL_TN, m0 = (L % tiles_m) * TL_TM;
-  const int wk = K >> 3;  // words per row (K % 256 == 0)
+  const int wk = K >> 3;
 
-  // byte offsets of this thread's rows (32-bit: tile_applies bounds the operands)
-  uint32_t wo[TL_WI], xo[TL_XI];
+  // what this lane fetches: row l/8 of an 8-row block, swizzled 16-byte piece.
+  // Wave w takes blocks w + 4 i; the key only needs the row's position in its
+  // 16-row group: ((block & 1) * 8 + l/8) / 2.
+  const int row8 = lane >> 3;
+  uint32_t wo[DM_WI], xo[DM_XI];  // byte offsets (32-bit: tile_applies bounds the operands)
 #pragma unroll
-  for (int i = 0; i < TL_WI; ++i) {
-    const int n = n0 + (t >> 2) + TL_RP * i;
-    wo[i] = ((uint32_t)(n < N ? n : N - 1) * (uint32_t)wk + (t & 3) * 4) * 4u;
+  for (int i = 0; i < DM_WI; ++i) {
+    const int blk = wave + DM_WAVES * i, R = blk * 8 + row8, n = n0 + R;
+    wo[i] = ((uint32_t)(n < N ? n : N - 1) * (uint32_t)wk) * 4u + (((lane & 7) ^ ((R >> 1) & 7)) * 16);
   }
 #pragma unroll
-  for (int i = 0; i < TL_XI; ++i) {
-    const int m = m0 + (t >> 2) + TL_RP * i;
-    xo[i] = ((uint32_t)(m < M ? m : M - 1) * (uint32_t)wk + (t & 3) * 4) * 4u;
+  for (int i = 0; i < DM_XI; ++i) {
+    const int blk = wave + DM_WAVES * i, R = blk * 8 + row8, m = m0 + R;
+    xo[i] = ((uint32_t)(m < M ? m : M - 1) * (uint32_t)wk) * 4u + (((lane & 7) ^ ((R >> 1) & 7)) * 16);
   }
-  const uint32_t swo = (uint32_t)(n0 + (t & 255) < N ? n0 + (t & 255) : N - 1) * (uint32_t)B;
-  const uint32_t sxo = (uint32_t)(m0 + (t & 127) < M ? m0 + (t & 127) : M - 1) * (uint32_t)B;
+  // scale dwords: waves 0-3 take W rows 64 wave + lane, the others X rows 64 (wave & 1)
+  // + lane (a wave fetches two per stage either way)
+  const bool w_scales = wave < 4;
+  const int srow = w_scales ? n0 + wave * 64 + lane : m0 + (wave & 1) * 64 + lane;
+  const int slim = w_scales ? N : M;
+  const uint32_t sco = (uint32_t)(srow < slim ? srow : slim - 1) * (uint32_t)B;
+  const uint8_t* scb = w_scales ? ws : xs;
+  const uint32_t sc_lds = w_scales ? wave * 256 : TL_TN * 4 + (wave & 1) * 256;
   const char* wqb = (const char*)wq;
   const char* xqb = (const char*)xq;
 
-  const int steps = K >> 7, pairs = K >> 8;
-  // the two 64-byte halves of a row's line are requested back to back
-  auto fetch = [&](TileRegs& q, int p) {
-    const uint32_t pp = (uint32_t)(p < pairs ? p : pairs - 1);  // past the end: valid, never used
-#pragma unroll
-    for (int i = 0; i < TL_WI; ++i) {
-      q.w[0][i] = *(const u4*)(wqb + (wo[i] + pp * 128u));
-      q.w[1][i] = *(const u4*)(wqb + (wo[i] + pp * 128u + 64u));
-    }
-#pragma unroll
-    for (int i = 0; i < TL_XI; ++i) {
-      q.x[0][i] = *(const u4*)(xqb + (xo[i] + pp * 128u));
-      q.x[1][i] = *(const u4*)(xqb + (xo[i] + pp * 128u + 64u));
-    }
-    q.sw = *(const u2*)(ws + (swo + pp * 8u));
-    q.sx = *(const u2*)(xs + (sxo + pp * 8u));
+  const int stages = K >> 8;
+  // The loads are written as asm so that the compiler neither tracks them (it would
+  // wait for all of them before any LDS read) nor moves LDS reads across them; the
+  // vmcnt waits below are by hand.  M0 carries the wave-uniform LDS address.
+  auto dma16 = [](const void* gbase, uint32_t goff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(goff), "s"(gbase), "s"(lds_addr)
+                 : "memory", "m0");
   };
-  // One 128-k half of a slot goes to LDS.  `keep` is 0 for a step past the end of
-  // K: its codes go in as zeros, so the loop needs no branch for a ragged last
-  // group of steps.
-  auto stage = [&](const TileRegs& q, int buf, int half, uint32_t keep) {
-    uint8_t* base = lds[buf];
-#pragma unroll
-    for (int i = 0; i < TL_WI; ++i)
-      *(u4*)(base + ((t >> 2) + TL_RP * i) * TL_ROWB + (t & 3) * 16) = q.w[half][i] & keep;
-#pragma unroll
-    for (int i = 0; i < TL_XI; ++i)
-      *(u4*)(base + (TL_TN + (t >> 2) + TL_RP * i) * TL_ROWB + (t & 3) * 16) = q.x[half][i] & keep;
-    uint32_t* sc = (uint32_t*)(base + TL_ROWS * TL_ROWB);
-    // several threads hold (and write) the same row's scale dword
-    sc[t & 255] = q.sw[half] & keep;
-    sc[TL_TN + (t & 127)] = q.sx[half] & keep;
+  auto dma4 = [](const void* gbase, uint32_t goff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1"
+                 :
+                 : "v"(goff), "s"(gbase), "s"(lds_addr)
+                 : "memory", "m0");
   };
-  auto read_frags = [&](TileFrags& f, int buf) {
-    const uint8_t* base = lds[buf];
-    const uint32_t* sc = (const uint32_t*)(base + TL_ROWS * TL_ROWB);
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr)dm_lds;
+  auto request = [&](int d) {
+    const uint32_t dd = (uint32_t)(d < stages ? d : stages - 1);  // past the end: valid, never used
+    const uint32_t st = lds0 + (uint32_t)(d % DM_STAGES) * DM_STAGE;
+#pragma unroll
+    for (int i = 0; i < DM_WI; ++i)
+      dma16(wqb, wo[i] + dd * 128u, st + (wave + DM_WAVES * i) * 1024);
+#pragma unroll
+    for (int i = 0; i < DM_XI; ++i)
+      dma16(xqb, xo[i] + dd * 128u, st + DM_W_BYTES + (wave + DM_WAVES * i) * 1024);
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2)  // the two 128-k halves' scale dwords
+      dma4(scb, sco + dd * 8u + s2 * 4u, st + DM_TILE_BYTES + s2 * (TL_ROWS * 4) + sc_lds);
+  };
+  // row R of an operand tile, 16-byte piece p (0..7) of the 256 k -> byte offset
+  auto at = [](int R, int p) { return (R >> 3) * 1024 + ((R & 7) * 8 + (p ^ ((R >> 1) & 7))) * 16; };
+  // operands of the 128-k half s2 of stage d
+  auto read_frags = [&](DmFrags& f, int d, int s2) {
+    const uint8_t* base = dm_lds + (d % DM_STAGES) * DM_STAGE;
+    const uint32_t* sc = (const uint32_t*)(base + DM_TILE_BYTES) + s2 * TL_ROWS;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int row = TL_TN + wm * 64 + j * 32 + r;
-      f.b[0][j] = *(const u4*)(base + row * TL_ROWB + h * 16);
-      f.b[1][j] = *(const u4*)(base + row * TL_ROWB + (2 + h) * 16);
-      f.sb[j] = sc[row];
+      const int row = wm * 64 + j * 32 + r;
+      f.b[0][j] = *(const u4*)(base + DM_W_BYTES + at(row, 4 * s2 + h));
+      f.b[1][j] = *(const u4*)(base + DM_W_BYTES + at(row, 4 * s2 + 2 + h));
+      f.sb[j] = sc[TL_TN + row];
     }
 #pragma unroll
-    for (int i = 0; i < TL_NT; ++i) {
-      const int row = wn * (32 * TL_NT) + i * 32 + r;
-      f.a[0][i] = *(const u4*)(base + row * TL_ROWB + h * 16);
-      f.a[1][i] = *(const u4*)(base + row * TL_ROWB + (2 + h) * 16);
+    for (int i = 0; i < DM_NT; ++i) {
+      const int row = wn * (32 * DM_NT) + i * 32 + r;
+      f.a[0][i] = *(const u4*)(base + at(row, 4 * s2 + h));
+      f.a[1][i] = *(const u4*)(base + at(row, 4 * s2 + 2 + h));
       f.sa[i] = sc[row];
     }
   };
 
-  f16v acc[TL_NT][2];
+  f16v acc[DM_NT][2];
 #pragma unroll
-  for (int i = 0; i < TL_NT; ++i)
+  for (int i = 0; i < DM_NT; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-
-  auto multiply = [&](const TileFrags& f) {
+  auto multiply = [&](const DmFrags& f) {
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh) {
-      const int sh = 16 * kh + 8 * h;  // this lane's block of the step: 2 kh + h
+      const int sh = 16 * kh + 8 * h;
 #pragma unroll
-      for (int i = 0; i < TL_NT; ++i)
+      for (int i = 0; i < DM_NT; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
           acc[i][j] = mfma_fp4_32(f.a[kh][i], f.sa[i] >> sh, f.b[kh][j], f.sb[j] >> sh, acc[i][j]);
     }
   };
 
-  TileRegs ring[PAIRS];
-  TileFrags frags[2];
-  // steps 2p and 2p+1 travel in ring slot p % PAIRS
-#pragma unroll
-  for (int d = 0; d < PAIRS; ++d) fetch(ring[d], d);
-  stage(ring[0], 0, 0, ~0u);
-  stage(ring[0], 1, 1, ~0u);
-  fetch(ring[0], PAIRS);
+  DmFrags fa, fb;
+  request(0);
+  request(1);
+  request(2);
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * DM_LOADS));  // stage 0 has landed (this wave's part)
   __syncthreads();
-  read_frags(frags[0], 0);
-  __syncthreads();  // buffer 0 is rewritten in the first iteration
-
-  // The unrolled body spans PAIRS slots = 2 * PAIRS steps: slot, half and buffer
-  // parity are constants, and there is no branch (every wait counts exactly the
-  // loads it needs).
+  read_frags(fa, 0, 0);
 #pragma unroll 1
-  for (int kb = 0; kb < steps; kb += 2 * PAIRS) {
-#pragma unroll
-    for (int u = 0; u < 2 * PAIRS; ++u) {
-      const int k = kb + u;
-      const int slot = ((u + 2) >> 1) % PAIRS;  // of step k + 2
-      read_frags(frags[(u + 1) & 1], (u + 1) & 1);
-      stage(ring[slot], u & 1, u & 1, k + 2 < steps ? ~0u : 0u);
-      if (u & 1) fetch(ring[slot], ((k + 2) >> 1) + PAIRS);
-      multiply(frags[u & 1]);
-      __syncthreads();
-    }
+  for (int d = 0; d < stages; ++d) {
+    read_frags(fb, d, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(fa);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(DM_LOADS));  // stage d + 1 has landed
+    __syncthreads();
+    // every wave has read both halves of stage d: its buffer takes stage d + 3
+    request(d + 3);
+    read_frags(fa, d + 1, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(fb);
+    __builtin_amdgcn_sched_barrier(0);
   }
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // nothing may still be writing LDS at exit
 
-  // lane: m = .. + r; e = 4 q + p holds n = .. + 8 q + 4 h + p
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int m = m0 + wm * 64 + j * 32 + r;
     if (m >= M) continue;
 #pragma unroll
-    for (int i = 0; i < TL_NT; ++i)
+    for (int i = 0; i < DM_NT; ++i)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int nn = n0 + wn * (32 * TL_NT) + i * 32 + 8 * q + 4 * h;
+        const int nn = n0 + wn * (32 * DM_NT) + i * 32 + 8 * q + 4 * h;
         w4_half* dst = c + (size_t)m * N + nn;
         if (nn + 3 < N && ((uintptr_t)dst & 7) == 0) {
           h4 out;
@@ -416,8 +425,13 @@ hipError_t launch_tile(const w4_packed_mx_view& w, const w4_packed_mx_view& x, w
                        hipStream_t s) {
   const int tiles_n = (w.N + TL_TN - 1) / TL_TN, tiles_m = (x.N + TL_TM - 1) / TL_TM;
   if ((long long)tiles_n * tiles_m > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
-  mxn_tile_kernel<TL_PAIRS><<<dim3((unsigned)(tiles_n * tiles_m)), dim3(TL_THREADS), 0, s>>>(
-      w.q, w.scales, x.q, x.scales, c, w.N, w.K, w.B, x.N, tiles_n, tiles_m);
+  static const hipError_t attr =
+      hipFuncSetAttribute((const void*)mxn_tile_dma_kernel,
+                          hipFuncAttributeMaxDynamicSharedMemorySize, DM_STAGES * DM_STAGE);
+  if (attr != hipSuccess) return attr;
+  mxn_tile_dma_kernel<<<dim3((unsigned)(tiles_n * tiles_m)), dim3(DM_THREADS),
+                        DM_STAGES * DM_STAGE, s>>>(w.q, w.scales, x.q, x.scales, c, w.N, w.K, w.B,
+                                                   x.N, tiles_n, tiles_m);
   return hipGetLastError();
 }
 

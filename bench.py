@@ -27,12 +27,12 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 PREWARM_LAUNCHES = 2000
 # HBM bytes one launch of the headline kernel moves, from rocprofv3 --pmc runs of
-# `python3 bench.py --extras none --steps 50 --warmup 5`: FETCH_SIZE 4287.5 and
+# `python3 bench.py --extras none --steps 50 --warmup 5`: FETCH_SIZE 4281.0 and
 # WRITE_SIZE 16.0 per dispatch, scaled by what the same counters read for the
 # 1 GiB stream_copy kernel of this file's yardstick (FETCH_SIZE 524298 and
 # WRITE_SIZE 1048591 for 1048576 KiB each way, i.e. factors 2.0 and 1.0):
-# 8575 KiB fetched + 16 KiB written, against 8 667 136 algorithmic bytes.
-HEADLINE_TRAFFIC_BYTES = int((4287.5 * 2.0 + 16.0 * 1.0) * 1024)
+# 8562 KiB fetched + 16 KiB written, against 8 667 136 algorithmic bytes.
+HEADLINE_TRAFFIC_BYTES = int((4281.0 * 2.0 + 16.0 * 1.0) * 1024)
 
 
 def _pkg():
@@ -465,6 +465,15 @@ def probe(b, which):
         views = b.rand_w4(N, K, 128, True, 18)
         for M, fn in ((1, "w4_gemm_fused"), (8, "w4_gemm_mma"), (16, "w4_gemm_mma")):
             out["%s_M%d_us" % (fn, M)] = b.gemm_us(fn, views, M, N, K)
+    elif which == "quantize":  # the device-side quantizers, 20 calls of each workload
+        b.steps, b.warmup = 200, 2
+        out.update(extras_quantize(b, False))
+    elif which == "w4a4":  # both operands MXFP4: skinny kernel at M=1/16/64, tile kernel at M=2048
+        N = K = 4096
+        views = b.rand_mx(N, K, 46)
+        for M in (1, 16, 64, 2048):
+            b.steps, b.warmup = (20, 3) if M > 64 else (100, 10)
+            out["w4a4_M%d_us" % M] = b.w4a4_us(views, M, N, K, reps=1)
     else:  # prefill: the fused tile kernel and the plain FP16 library GEMM, 20 calls each
         N = K = 4096
         M = 2048
@@ -486,7 +495,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--extras", choices=["none", "quick", "full"], default="quick")
-    ap.add_argument("--probe", choices=["decode", "prefill"], default=None,
+    ap.add_argument("--probe", choices=["decode", "prefill", "quantize", "w4a4"], default=None,
                     help="run only a short fixed workload (for counter collection) and exit")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -23,9 +23,11 @@ SHAPES = [(1, 64, 512), (16, 256, 4096), (5, 100, 1000), (3, 48, 100), (33, 80, 
           (1, 16, 8), (200, 200, 200),
           # a few hundred rows on the skinny kernel's grid.y walk
           (128, 256, 512), (96, 64, 128), (200, 300, 1024), (300, 520, 384), (129, 257, 256),
-          # K % 256 == 0 and M >= 384: the LDS-tiled kernel (ragged tiles on both sides, step
-          # counts that are and are not multiples of the unrolled loop body)
-          (384, 256, 512), (500, 300, 1024), (385, 520, 256), (700, 257, 768), (400, 64, 1280)]
+          # many rows of X on the skinny kernel's grid.y walk (too few tiles for the tiled kernel)
+          (384, 256, 512), (500, 300, 1024), (385, 520, 256),
+          # K % 256 == 0 and at least 64 tiles of 256 x 128: the LDS-tiled kernel, ragged on both
+          # sides, 2 to 5 stages of 256 k
+          (900, 2100, 512), (1030, 2050, 768), (1024, 2048, 1280)]
 
 
 def _quantize_x_on_device(x16, M, K):

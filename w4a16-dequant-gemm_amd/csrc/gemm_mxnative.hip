@@ -414,11 +414,15 @@ __global__ __launch_bounds__(DM_THREADS) void mxn_tile_dma_kernel(
 }
 
 bool tile_applies(const w4_packed_mx_view& w, const w4_packed_mx_view& x) {
-  // below a few hundred rows of X the skinny kernel's grid.y walk is faster (measured:
-  // M = 256 at N = 4096 takes 21 us there, 37 us here on 32 workgroups)
-  return x.N >= 384 && w.K % 256 == 0 && (long long)w.N * w.K < (1LL << 32) &&
-         (long long)x.N * x.K < (1LL << 32) && ((uintptr_t)w.q & 15) == 0 && ((uintptr_t)x.q & 15) == 0 &&
-         ((uintptr_t)w.scales & 7) == 0 && ((uintptr_t)x.scales & 7) == 0;
+  // Worth it once the tile grid covers a good part of the chip; below that the
+  // skinny kernel's grid.y walk is faster (measured at K = 4096: N = 4096, M = 256
+  // -> 32 tiles 37 us here, 23 us there; M = 512 -> 64 tiles 31 us here; N = 14336,
+  // M = 256 -> 112 tiles 34 us here, 54 us there).
+  const long long tiles = (long long)((w.N + TL_TN - 1) / TL_TN) * ((x.N + TL_TM - 1) / TL_TM);
+  return x.N >= 128 && tiles >= 64 && w.K % 256 == 0 && (long long)w.N * w.K < (1LL << 32) &&
+         (long long)x.N * x.K < (1LL << 32) && ((uintptr_t)w.q & 15) == 0 &&
+         ((uintptr_t)x.q & 15) == 0 && ((uintptr_t)w.scales & 7) == 0 &&
+         ((uintptr_t)x.scales & 7) == 0;
 }
 
 hipError_t launch_tile(const w4_packed_mx_view& w, const w4_packed_mx_view& x, w4_half* c,

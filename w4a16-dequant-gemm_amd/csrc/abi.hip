@@ -354,10 +354,10 @@ int w4_quantize(const w4_packed_view* out, const double* w, int* status, w4_stre
   if (int rc = check_packed(out, "quantize")) return rc;
   REQUIRE(w && status, "quantize: null pointer");
   if (int rc = start_status(status, stream, "quantize")) return rc;
-  return done("quantize", w4k::launch_quantize_rows(
-                              out->symmetric ? 0 : 1, w, 0, out->N, out->K, out->gs,
-                              (uint32_t*)out->q, nullptr, (w4_half*)out->scales,
-                              (uint32_t*)out->zeros, status, (hipStream_t)stream));
+  const w4k::QuantSide side{w, (uint32_t*)out->q, nullptr, (w4_half*)out->scales,
+                            (uint32_t*)out->zeros};
+  return done("quantize", w4k::launch_quantize_rows(out->symmetric ? 0 : 1, &side, 1, 0, out->N,
+                                                    out->K, out->gs, status, (hipStream_t)stream));
 }
 
 int w4_quantize_mx(const w4_packed_mx_view* out, const double* w, int* status,
@@ -408,16 +408,13 @@ int w4_quantize_cache(const w4_kv_view* out, const void* k, const void* v, int s
   REQUIRE(!out->symmetric || (!out->z_k && !out->z_v),
           "quantize_cache: symmetric carries no zeros");
   if (int rc = start_status(status, stream, "quantize_cache")) return rc;
-  const long long rows = (long long)out->H * out->S;
-  const int mode = out->symmetric ? 0 : 1;
-  hipError_t e = w4k::launch_quantize_rows(mode, k, src_f16, rows, out->D, out->gs,
-                                           (uint32_t*)out->q_k, nullptr, (w4_half*)out->s_k,
-                                           (uint32_t*)out->z_k, status, (hipStream_t)stream);
-  if (e == hipSuccess)
-    e = w4k::launch_quantize_rows(mode, v, src_f16, rows, out->D, out->gs, (uint32_t*)out->q_v,
-                                  nullptr, (w4_half*)out->s_v, (uint32_t*)out->z_v, status,
-                                  (hipStream_t)stream);
-  return done("quantize_cache", e);
+  const w4k::QuantSide sides[2] = {
+      {k, (uint32_t*)out->q_k, nullptr, (w4_half*)out->s_k, (uint32_t*)out->z_k},
+      {v, (uint32_t*)out->q_v, nullptr, (w4_half*)out->s_v, (uint32_t*)out->z_v}};
+  return done("quantize_cache",
+              w4k::launch_quantize_rows(out->symmetric ? 0 : 1, sides, 2, src_f16,
+                                        (long long)out->H * out->S, out->D, out->gs, status,
+                                        (hipStream_t)stream));
 }
 
 int w4_quantize_cache_f8(const w4_kv_f8_view* out, const void* k, const void* v, int src_f16,
@@ -430,15 +427,11 @@ int w4_quantize_cache_f8(const w4_kv_f8_view* out, const void* k, const void* v,
   REQUIRE(out->q_k && out->s_k && out->q_v && out->s_v && k && v && status,
           "quantize_cache_f8: null pointer");
   if (int rc = start_status(status, stream, "quantize_cache_f8")) return rc;
-  const long long rows = (long long)out->H * out->S;
-  hipError_t e = w4k::launch_quantize_rows(2, k, src_f16, rows, out->D, out->gs, nullptr,
-                                           (uint8_t*)out->q_k, (w4_half*)out->s_k, nullptr,
-                                           status, (hipStream_t)stream);
-  if (e == hipSuccess)
-    e = w4k::launch_quantize_rows(2, v, src_f16, rows, out->D, out->gs, nullptr,
-                                  (uint8_t*)out->q_v, (w4_half*)out->s_v, nullptr, status,
-                                  (hipStream_t)stream);
-  return done("quantize_cache_f8", e);
+  const w4k::QuantSide sides[2] = {{k, nullptr, (uint8_t*)out->q_k, (w4_half*)out->s_k, nullptr},
+                                   {v, nullptr, (uint8_t*)out->q_v, (w4_half*)out->s_v, nullptr}};
+  return done("quantize_cache_f8",
+              w4k::launch_quantize_rows(2, sides, 2, src_f16, (long long)out->H * out->S, out->D,
+                                        out->gs, status, (hipStream_t)stream));
 }
 
 }  // extern "C"

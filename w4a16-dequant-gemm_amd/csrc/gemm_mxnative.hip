@@ -429,10 +429,17 @@ hipError_t launch_tile(const w4_packed_mx_view& w, const w4_packed_mx_view& x, w
                        hipStream_t s) {
   const int tiles_n = (w.N + TL_TN - 1) / TL_TN, tiles_m = (x.N + TL_TM - 1) / TL_TM;
   if ((long long)tiles_n * tiles_m > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
-  static const hipError_t attr =
-      hipFuncSetAttribute((const void*)mxn_tile_dma_kernel,
-                          hipFuncAttributeMaxDynamicSharedMemorySize, DM_STAGES * DM_STAGE);
-  if (attr != hipSuccess) return attr;
+  // more than 64 KB of LDS has to be granted per device, once
+  static bool granted[64] = {};
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+  if (dev < 0 || dev >= 64 || !granted[dev]) {
+    const hipError_t e =
+        hipFuncSetAttribute((const void*)mxn_tile_dma_kernel,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, DM_STAGES * DM_STAGE);
+    if (e != hipSuccess) return e;
+    if (dev >= 0 && dev < 64) granted[dev] = true;
+  }
   mxn_tile_dma_kernel<<<dim3((unsigned)(tiles_n * tiles_m)), dim3(DM_THREADS),
                         DM_STAGES * DM_STAGE, s>>>(w.q, w.scales, x.q, x.scales, c, w.N, w.K, w.B,
                                                    x.N, tiles_n, tiles_m);

@@ -84,9 +84,16 @@ hipError_t launch_flash(const FlashArgs& a, float* scratch, hipStream_t s);
 // zero-points, 2 E4M3 bytes; src is FP64 or (src_f16) FP16; `rows` rows of K
 // elements, groups of gs along K.  status: bit 0 non-finite input, bit 1 scale
 // out of range (OR-ed in by the kernels).
-hipError_t launch_quantize_rows(int mode, const void* src, int src_f16, long long rows, int K,
-                                int gs, uint32_t* q32, uint8_t* q8, w4_half* scales,
-                                uint32_t* zeros, int* status, hipStream_t s);
+struct QuantSide {  // one source and its outputs (q32: W4 words, q8: E4M3 bytes)
+  const void* src;
+  uint32_t* q32;
+  uint8_t* q8;
+  w4_half* scales;
+  uint32_t* zeros;
+};
+// nsides (1 or 2) jobs of the same shape in one launch: the K and V sides of a cache
+hipError_t launch_quantize_rows(int mode, const QuantSide* sides, int nsides, int src_f16,
+                                long long rows, int K, int gs, int* status, hipStream_t s);
 hipError_t launch_quantize_mx(const void* src, int src_f16, long long rows, int K, uint32_t* q,
                               uint8_t* scales, int* status, hipStream_t s);
 // gemm_mxnative.hip -- both operands packed MXFP4 (x.N = M rows of K), scaled MFMA

@@ -36,6 +36,17 @@ __global__ void fill_words_kernel(uint32_t* p, long long n, uint32_t value) {
 
 enum { QM_SYM = 0, QM_ASYM = 1, QM_F8 = 2 };
 
+// Up to two independent jobs of the same shape in one launch (the K and the V
+// side of a cache): blockIdx.y picks the side.
+template <typename T>
+struct Sides {
+  const T* src[2];
+  uint32_t* q32[2];
+  uint8_t* q8[2];
+  uint16_t* scales[2];
+  uint32_t* zeros[2];
+};
+
 // lround() for |v| far below 2^52: the fraction v - trunc(v) is exact.
 __device__ __forceinline__ long round_half_away(double v) {
   double t = trunc(v);
@@ -77,9 +88,12 @@ __device__ __forceinline__ int pow2_at_least(int n) {
 // source element type (double or _Float16).
 template <typename T, int MODE>
 __global__ __launch_bounds__(QT) void quantize_rows_kernel(
-    const T* __restrict__ src, long long rows, int K, int gs, int G, uint32_t* __restrict__ q32,
-    uint8_t* __restrict__ q8, uint16_t* __restrict__ scales, uint32_t* __restrict__ zeros,
-    int* __restrict__ status) {
+    const Sides<T> sd, long long rows, int K, int gs, int G, int* __restrict__ status) {
+  const T* __restrict__ src = sd.src[blockIdx.y];
+  uint32_t* __restrict__ q32 = sd.q32[blockIdx.y];
+  uint8_t* __restrict__ q8 = sd.q8[blockIdx.y];
+  uint16_t* __restrict__ scales = sd.scales[blockIdx.y];
+  uint32_t* __restrict__ zeros = sd.zeros[blockIdx.y];
   __shared__ double s_lo[QT], s_hi[QT];
   __shared__ float s_scale[QT];
   __shared__ int s_zero[QT];
@@ -246,9 +260,12 @@ __device__ __forceinline__ void load8(const _Float16* p, float v[8]) {
 // workgroup both multiples of 8); otherwise nibbles are OR-ed in atomically.
 template <typename T, int MODE, bool ZPACK>
 __global__ __launch_bounds__(QT) void quantize_rows_fast_kernel(
-    const T* __restrict__ src, long long nwords, int wpg, int wpg_shift, int G,
-    uint32_t* __restrict__ q32, uint8_t* __restrict__ q8, uint16_t* __restrict__ scales,
-    uint32_t* __restrict__ zeros, int* __restrict__ status) {
+    const Sides<T> sd, long long nwords, int wpg, int wpg_shift, int G, int* __restrict__ status) {
+  const T* __restrict__ src = sd.src[blockIdx.y];
+  uint32_t* __restrict__ q32 = sd.q32[blockIdx.y];
+  uint8_t* __restrict__ q8 = sd.q8[blockIdx.y];
+  uint16_t* __restrict__ scales = sd.scales[blockIdx.y];
+  uint32_t* __restrict__ zeros = sd.zeros[blockIdx.y];
   typedef typename Quot<T>::type A;
   __shared__ int s_zero[QT];
   const int t = threadIdx.x;
@@ -430,52 +447,58 @@ __global__ __launch_bounds__(QT) void quantize_mx_kernel(const T* __restrict__ s
 }
 
 template <typename T, int MODE>
-hipError_t launch_rows_t(const T* src, long long rows, int K, int gs, uint32_t* q32, uint8_t* q8,
-                         w4_half* scales, uint32_t* zeros, int* status, hipStream_t s) {
+hipError_t launch_rows_t(const Sides<T>& sd, int nsides, long long rows, int K, int gs,
+                         int* status, hipStream_t s) {
   const int G = (K + gs - 1) / gs;
   const int wpg = gs >> 3, tpg = wpg < QT ? wpg : QT, gpb = QT / tpg;
   const bool pow2 = (wpg & (wpg - 1)) == 0;
-  const bool out8 = MODE != QM_F8 || ((uintptr_t)q8 & 7) == 0;
-  if (pow2 && wpg <= 64 && K % gs == 0 && ((uintptr_t)src & 15) == 0 && out8) {
+  bool aligned = true;
+  for (int i = 0; i < nsides; ++i)
+    aligned = aligned && ((uintptr_t)sd.src[i] & 15) == 0 &&
+              (MODE != QM_F8 || ((uintptr_t)sd.q8[i] & 7) == 0);
+  const bool fast = pow2 && wpg <= 64 && K % gs == 0 && aligned;
+  const bool zpack = fast && MODE == QM_ASYM && G % 8 == 0 && (QT / wpg) % 8 == 0;
+  if (MODE == QM_ASYM && !zpack) {
+    // zero-points are OR-ed in nibble by nibble
+    const long long nz = rows * words(G);
+    for (int i = 0; i < nsides; ++i)
+      fill_words_kernel<<<dim3((unsigned)((nz + 255) / 256)), dim3(256), 0, s>>>(sd.zeros[i], nz, 0u);
+  }
+  if (fast) {
     const long long nwords = rows * (K >> 3);
     const long long nb = (nwords + QT - 1) / QT;
     if (nb > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
     const int shift = __builtin_ctz(wpg);
-    const bool zpack = MODE == QM_ASYM && G % 8 == 0 && (QT / wpg) % 8 == 0;
+    const dim3 grid((unsigned)nb, (unsigned)nsides);
     if (zpack)
-      quantize_rows_fast_kernel<T, MODE, true><<<dim3((unsigned)nb), dim3(QT), 0, s>>>(
-          src, nwords, wpg, shift, G, q32, q8, scales, zeros, status);
-    else {
-      if (MODE == QM_ASYM) {
-        const long long nz = rows * words(G);
-        fill_words_kernel<<<dim3((unsigned)((nz + 255) / 256)), dim3(256), 0, s>>>(zeros, nz, 0u);
-      }
-      quantize_rows_fast_kernel<T, MODE, false><<<dim3((unsigned)nb), dim3(QT), 0, s>>>(
-          src, nwords, wpg, shift, G, q32, q8, scales, zeros, status);
-    }
+      quantize_rows_fast_kernel<T, MODE, true><<<grid, dim3(QT), 0, s>>>(sd, nwords, wpg, shift, G,
+                                                                        status);
+    else
+      quantize_rows_fast_kernel<T, MODE, false><<<grid, dim3(QT), 0, s>>>(sd, nwords, wpg, shift,
+                                                                         G, status);
     return hipGetLastError();
   }
   const long long blocks = (rows * G + gpb - 1) / gpb;
   if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
-  if (MODE == QM_ASYM) {
-    // zero-points are OR-ed in nibble by nibble
-    const long long nz = rows * words(G);
-    fill_words_kernel<<<dim3((unsigned)((nz + 255) / 256)), dim3(256), 0, s>>>(zeros, nz, 0u);
-  }
-  quantize_rows_kernel<T, MODE><<<dim3((unsigned)blocks), dim3(QT), 0, s>>>(
-      src, rows, K, gs, G, q32, q8, scales, zeros, status);
+  quantize_rows_kernel<T, MODE><<<dim3((unsigned)blocks, (unsigned)nsides), dim3(QT), 0, s>>>(
+      sd, rows, K, gs, G, status);
   return hipGetLastError();
 }
 
 template <typename T>
-hipError_t launch_rows(int mode, const T* src, long long rows, int K, int gs, uint32_t* q32,
-                       uint8_t* q8, w4_half* scales, uint32_t* zeros, int* status,
-                       hipStream_t s) {
-  if (mode == QM_SYM)
-    return launch_rows_t<T, QM_SYM>(src, rows, K, gs, q32, q8, scales, zeros, status, s);
-  if (mode == QM_ASYM)
-    return launch_rows_t<T, QM_ASYM>(src, rows, K, gs, q32, q8, scales, zeros, status, s);
-  return launch_rows_t<T, QM_F8>(src, rows, K, gs, q32, q8, scales, zeros, status, s);
+hipError_t launch_rows(int mode, const QuantSide* sides, int nsides, long long rows, int K, int gs,
+                       int* status, hipStream_t s) {
+  Sides<T> sd{};
+  for (int i = 0; i < nsides; ++i) {
+    sd.src[i] = (const T*)sides[i].src;
+    sd.q32[i] = sides[i].q32;
+    sd.q8[i] = sides[i].q8;
+    sd.scales[i] = sides[i].scales;
+    sd.zeros[i] = sides[i].zeros;
+  }
+  if (mode == QM_SYM) return launch_rows_t<T, QM_SYM>(sd, nsides, rows, K, gs, status, s);
+  if (mode == QM_ASYM) return launch_rows_t<T, QM_ASYM>(sd, nsides, rows, K, gs, status, s);
+  return launch_rows_t<T, QM_F8>(sd, nsides, rows, K, gs, status, s);
 }
 
 }  // namespace
@@ -485,13 +508,10 @@ hipError_t launch_fill_words(uint32_t* p, long long n, uint32_t value, hipStream
   return hipGetLastError();
 }
 
-hipError_t launch_quantize_rows(int mode, const void* src, int src_f16, long long rows, int K,
-                                int gs, uint32_t* q32, uint8_t* q8, w4_half* scales,
-                                uint32_t* zeros, int* status, hipStream_t s) {
-  return src_f16 ? launch_rows(mode, (const _Float16*)src, rows, K, gs, q32, q8, scales, zeros,
-                               status, s)
-                 : launch_rows(mode, (const double*)src, rows, K, gs, q32, q8, scales, zeros,
-                               status, s);
+hipError_t launch_quantize_rows(int mode, const QuantSide* sides, int nsides, int src_f16,
+                                long long rows, int K, int gs, int* status, hipStream_t s) {
+  return src_f16 ? launch_rows<_Float16>(mode, sides, nsides, rows, K, gs, status, s)
+                 : launch_rows<double>(mode, sides, nsides, rows, K, gs, status, s);
 }
 
 hipError_t launch_quantize_mx(const void* src, int src_f16, long long rows, int K, uint32_t* q,

@@ -74,12 +74,19 @@ class Bench:
         self.yard.w4bench_gemm_loop.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p,
                                                 C.c_int, C.c_int, C.c_void_p]
 
-    def w4a4_us(self, views, M, N, K, reps=5):
-        """us per w4_gemm_mx_w4a4 call over rotating weight copies (C loop, HIP events)."""
+    def w4a4_us(self, views, M, N, K, reps=5, a8=False):
+        """us per w4_gemm_mx_w4a4 (a8: w4_gemm_mx_w4a8) call over rotating weight copies (C
+        loop, HIP events)."""
         torch = self.torch
-        xv = self.rand_mx(M, K, 1)[0]
+        if a8:
+            xq = torch.randint(0, 0x78, (M * K,), dtype=torch.uint8, device="cuda")
+            xs = torch.randint(118, 123, (M * (K // 32),), dtype=torch.uint8, device="cuda")
+            xv = (self.capi.act_mx8_view(M, K, K // 32, xq.data_ptr(), xs.data_ptr()), (xq, xs))
+        else:
+            xv = self.rand_mx(M, K, 1)[0]
         c = torch.empty(M * N, dtype=torch.float16, device="cuda")
-        fn = C.cast(self.capi.load().w4_gemm_mx_w4a4, C.c_void_p)
+        fn = C.cast(self.capi.load().w4_gemm_mx_w4a8 if a8 else self.capi.load().w4_gemm_mx_w4a4,
+                    C.c_void_p)
         arr = (C.c_void_p * len(views))(*[C.addressof(v[0]) for v in views])
         self.yard.w4bench_w4a4_loop.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p,
                                                 C.c_int, C.c_void_p]
@@ -395,6 +402,9 @@ def extras_w4a4(b, full):
             us = b.w4a4_us(views, M, N, K)
             rows.append({"N": N, "K": K, "M": M, "bytes": nb, "us": us, "GBs": nb / us * 1e-3,
                          "TFLOPs": 2.0 * M * N * K / us * 1e-6})
+            if M <= 256:  # E4M3 activations (skinny kernel only)
+                us8 = b.w4a4_us(views, M, N, K, a8=True)
+                rows[-1].update({"a8_us": us8, "a8_TFLOPs": 2.0 * M * N * K / us8 * 1e-6})
         del views
         torch.cuda.empty_cache()
     return {"w4a4_mxfp4": rows}

@@ -23,6 +23,7 @@
 #include "kvfp8.hpp"
 #include "kvpaged.hpp"
 #include "mx.hpp"
+#include "mxact.hpp"
 #include "pack.hpp"
 
 namespace w4::gpu {
@@ -366,6 +367,24 @@ inline void gemm_mx_w4a4(const DevicePackedWm& w, const DevicePackedWm& x, __hal
                          hipStream_t stream = 0) {
   const auto vw = detail::abi(w), vx = detail::abi(x);
   detail::raise(w4_gemm_mx_w4a4(&vw, &vx, detail::h(c), stream));
+}
+
+// W4A8: MXFP8 activations (include/w4/mxact.hpp), device view and entry points.
+struct DeviceActMx8 {
+  int M, K, B;
+  const uint8_t* q;
+  const uint8_t* scales;
+};
+inline void quantize_mx8_f16_async(const DeviceActMx8& out, const __half* x, int* status,
+                                   hipStream_t stream = 0) {
+  const w4_act_mx8_view v{out.M, out.K, out.B, out.q, out.scales};
+  detail::raise(w4_quantize_mx8_f16(&v, detail::h(x), status, stream));
+}
+inline void gemm_mx_w4a8(const DevicePackedWm& w, const DeviceActMx8& x, __half* c,
+                         hipStream_t stream = 0) {
+  const auto vw = detail::abi(w);
+  const w4_act_mx8_view vx{x.M, x.K, x.B, x.q, x.scales};
+  detail::raise(w4_gemm_mx_w4a8(&vw, &vx, detail::h(c), stream));
 }
 
 }  // namespace w4::gpu

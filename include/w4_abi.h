@@ -66,6 +66,14 @@ typedef struct w4_kv_f8_view {
   const w4_half* s_v;
 } w4_kv_f8_view;
 
+/* MXFP8 activations, device view: E4M3 bytes under one E8M0 scale per 32 along K
+ * (no counterpart in the reference; host side: include/w4/mxact.hpp here). */
+typedef struct w4_act_mx8_view {
+  int M, K, B;           /* B = ceil(K / 32)                               */
+  const uint8_t* q;      /* M * K E4M3 bytes                               */
+  const uint8_t* scales; /* M * B E8M0 bytes                               */
+} w4_act_mx8_view;
+
 const char* w4_last_error(void);
 
 /* M at or above this goes to the matrix-core kernel in w4_gemm / w4_gemm_mx.
@@ -179,6 +187,15 @@ int w4_quantize_cache_f8(const w4_kv_f8_view* out, const void* k, const void* v,
  * <= 1e-3 against the FP64 product of the two dequantized operands.  Codes
  * past K in a row's last word are ignored. */
 int w4_gemm_mx_w4a4(const w4_packed_mx_view* w, const w4_packed_mx_view* x,
+                    w4_half* c, w4_stream stream);
+
+/* W4A8: MXFP4 weights against MXFP8 activations (E4M3 elements, E8M0 block
+ * scales; w4_quantize_mx8_f16 makes them from FP16 with the bytes of the host
+ * mxa::quantize_mx8).  Same exactness and gate as W4A4.  K must be a multiple
+ * of 32 and x->q 16-byte aligned. */
+int w4_quantize_mx8_f16(const w4_act_mx8_view* out, const w4_half* x, int* status,
+                        w4_stream stream);
+int w4_gemm_mx_w4a8(const w4_packed_mx_view* w, const w4_act_mx8_view* x,
                     w4_half* c, w4_stream stream);
 
 #ifdef __cplusplus

@@ -467,6 +467,60 @@ int orc_quantize_mx(const double* w, size_t w_len, int N, int K, uint32_t* q,
   return ORC_OK;
 }
 
+/* MXFP8 activations: see the header.  No reference counterpart. */
+int orc_quantize_mx8(const double* x, size_t x_len, int M, int K, uint8_t* q,
+                     uint8_t* scales) {
+  if (M < 1 || K < 1) return fail("quantize_mx8: bad dims");
+  if (x_len != (size_t)M * (size_t)K) return fail("quantize_mx8: size");
+  if (!all_finite(x, x_len)) return fail("quantize_mx8: non-finite input");
+  const int B = orc_blocks(K);
+  for (int m = 0; m < M; ++m) {
+    const double* row = x + (size_t)m * K;
+    for (int b = 0; b < B; ++b) {
+      const int k0 = b * 32, k1 = (k0 + 32 < K) ? k0 + 32 : K;
+      double amax = 0.0;
+      for (int k = k0; k < k1; ++k)
+        if (fabs(row[k]) > amax) amax = fabs(row[k]);
+      int e = 0;
+      if (amax > 0.0) {
+        e = -127; /* smallest e with amax <= 448 * 2^e, by search */
+        while (e <= 127 && amax > 448.0 * ldexp(1.0, e)) ++e;
+        if (e > 127) return fail("quantize_mx8: block scale outside E8M0 range");
+      }
+      const double s = ldexp(1.0, e);
+      scales[(size_t)m * B + b] = (uint8_t)(e + 127);
+      for (int k = k0; k < k1; ++k)
+        q[(size_t)m * K + k] = orc_f32_to_e4m3_satfinite((float)(row[k] / s));
+    }
+  }
+  return ORC_OK;
+}
+
+int orc_dequant_mx8(int M, int K, const uint8_t* q, const uint8_t* scales,
+                    double* out) {
+  if (M < 1 || K < 1) return fail("mx8: bad dims");
+  const int B = orc_blocks(K);
+  for (int m = 0; m < M; ++m)
+    for (int k = 0; k < K; ++k)
+      out[(size_t)m * K + k] =
+          (double)orc_decode_f8_e4m3(q[(size_t)m * K + k]) *
+          ldexp(1.0, (int)scales[(size_t)m * B + k / 32] - 127);
+  return ORC_OK;
+}
+
+int orc_gemm_f64(const double* x, int M, int K, const double* w, int N, double* c) {
+  if (M < 1 || N < 1 || K < 1) return fail("gemm_f64: bad dims");
+#pragma omp parallel for schedule(static) num_threads(g_threads)
+  for (int n = 0; n < N; ++n)
+    for (int m = 0; m < M; ++m) {
+      const double *xr = x + (size_t)m * K, *wr = w + (size_t)n * K;
+      double acc = 0.0;
+      for (int k = 0; k < K; ++k) acc += xr[k] * wr[k];
+      c[(size_t)m * N + n] = acc;
+    }
+  return ORC_OK;
+}
+
 /* mx.hpp:121-140. */
 int orc_dequant_all_mx(int N, int K, int B, const uint32_t* q, size_t q_len,
                        const uint8_t* scales, size_t s_len, uint16_t* w) {

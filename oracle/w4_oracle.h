@@ -101,6 +101,21 @@ int orc_paged_scatter(const void* src, void* dst, int H, int S, int page,
                       const int* bt, int bt_len, size_t row_elems,
                       size_t elem_size);
 
+/* ---- MXFP8 activations (additive: the reference has no such format) --------
+ * E4M3 elements under one E8M0 scale per 32, defined by analogy with
+ * mx.hpp:71-119: the block exponent is the smallest e with amax <= 448 * 2^e
+ * (clamped to [-127, 127]; larger fails), an element is the RNE / saturating
+ * E4M3 code (kvfp8.hpp:48-53) of float(v / 2^e).  Pinned by closed forms in the
+ * CPU suite (exact round trip of representable values, block maxima on both
+ * sides of 448 * 2^e, agreement with the independent C++ header). */
+int orc_quantize_mx8(const double* x, size_t x_len, int M, int K, uint8_t* q,
+                     uint8_t* scales);
+int orc_dequant_mx8(int M, int K, const uint8_t* q, const uint8_t* scales,
+                    double* out);
+/* c[m][n] = sum_k x[m][k] * w[n][k] over FP64 operands (pack.hpp:150-170
+ * without the FP16 widening). */
+int orc_gemm_f64(const double* x, int M, int K, const double* w, int N, double* c);
+
 /* ---- helpers ------------------------------------------------------------- */
 /* sqrt(sum((half(b)-a)^2)/sum(a^2)): the benches' quantization-error figure. */
 double orc_rel_l2_f16_vs_f64(const double* a, const uint16_t* b, size_t n);

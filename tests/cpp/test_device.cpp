@@ -376,6 +376,30 @@ void w4a4_gates(Checks& t) {
   }
 }
 
+// W4A8: the same gates with MXFP8 activations (include/w4/mxact.hpp).
+void w4a8_gates(Checks& t) {
+  Dev<int> status(1);
+  const Shape shapes[] = {{5, 100, 992, 0}, {64, 128, 1024, 0}, {200, 72, 512, 0}};
+  for (const Shape& c : shapes) {
+    const mx::PackedWm w = mx::quantize_mx(normal_weights(c.N * c.K, 41), c.N, c.K);
+    const auto x16 = normal_activations(c.M * c.K, 42);
+    std::vector<double> xd(x16.size());
+    for (size_t i = 0; i < xd.size(); ++i) xd[i] = (double)__half2float(x16[i]);
+    const mxa::PackedXm8 xq = mxa::quantize_mx8(xd, c.M, c.K);
+    const auto ref = mxa::gemm_reference_w4a8(xq, w);
+    Dev<uint32_t> wq(w.q);
+    Dev<uint8_t> wsc(w.scales), xqd(xq.q.size()), xsd(xq.scales.size());
+    Dev<__half> x(x16), out((size_t)c.M * c.N);
+    const DevicePackedWm dw{c.N, c.K, w.B, wq.p, wsc.p};
+    const DeviceActMx8 dx{c.M, c.K, xq.B, xqd.p, xsd.p};
+    quantize_mx8_f16_async(dx, x.p, status.p);
+    t.expect(same(xqd.get(), xq.q) && same(xsd.get(), xq.scales) && status.get()[0] == 0,
+             "MXFP8 activations quantized on the device: host bytes");
+    gemm_mx_w4a8(dw, dx, out.p);
+    oracle_gate(t, out.get(), ref, "W4A8 product vs FP64 product of the dequantized operands");
+  }
+}
+
 }  // namespace
 
 int main() {
@@ -389,6 +413,7 @@ int main() {
   attention_gates(t);
   quantizer_gates(t);
   w4a4_gates(t);
+  w4a8_gates(t);
   std::printf("worst rel L2 vs the FP64 references = %.3e\n", g_worst);
   return t.finish("device");
 }

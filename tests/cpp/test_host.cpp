@@ -15,6 +15,7 @@
 #include "w4/kvfp8.hpp"
 #include "w4/kvpaged.hpp"
 #include "w4/mx.hpp"
+#include "w4/mxact.hpp"
 #include "w4/pack.hpp"
 
 namespace {
@@ -361,10 +362,60 @@ void paged_gates(Checks& t) {
   t.throws_invalid([&] { w4::kv::validate_paged(badpool); }, "paged q size");
 }
 
+// MXFP8 activations (additive format): the header against the C oracle byte for
+// byte, per-element error bound of a 3-bit mantissa, no block saturates, exact
+// round trip of representable values, contracts.
+void mx8_gates(Checks& t) {
+  const int shapes[][2] = {{4, 64}, {7, 100}, {3, 33}, {16, 256}, {1, 1}};
+  for (size_t i = 0; i < 5; ++i) {
+    const int M = shapes[i][0], K = shapes[i][1];
+    auto x = w4::normal_weights(M * K, 0x8A8AULL ^ (uint64_t)(i * 131));
+    for (size_t j = 0; j < x.size(); j += 5) x[j] *= 50.0;  // spread the block maxima
+    const auto p = w4::mxa::quantize_mx8(x, M, K);
+    std::vector<uint8_t> oq(p.q.size()), os(p.scales.size());
+    t.expect(orc_quantize_mx8(x.data(), x.size(), M, K, oq.data(), os.data()) == 0 && oq == p.q &&
+                 os == p.scales,
+             "mx8: header == oracle bytes");
+    const auto d = w4::mxa::dequant_all_mx8(p);
+    std::vector<double> od(d.size());
+    orc_dequant_mx8(M, K, oq.data(), os.data(), od.data());
+    t.expect(od == d, "mx8: dequant header == oracle");
+    bool bound = true, unsat = true;
+    for (int m = 0; m < M; ++m)
+      for (int k = 0; k < K; ++k) {
+        const double s = std::ldexp(1.0, (int)p.scales[(size_t)m * p.B + k / 32] - 127);
+        const double v = x[(size_t)m * K + k], err = std::fabs(d[(size_t)m * K + k] - v);
+        // half a step of the binade of |v| / s (3 mantissa bits), or of the subnormal row
+        const double step = std::max(std::ldexp(1.0, std::ilogb(std::max(std::fabs(v) / s, 1e-300)) - 3), std::ldexp(1.0, -9));
+        bound &= err <= 0.5 * step * s * (1 + 1e-9);
+        unsat &= std::fabs(v) <= 448.0 * s;
+      }
+    t.expect(bound, "mx8 per-element bound");
+    t.expect(unsat, "mx8 no block saturates");
+    // representable values come back exactly
+    const auto p2 = w4::mxa::quantize_mx8(d, M, K);
+    t.expect(w4::mxa::dequant_all_mx8(p2) == d, "mx8 round trip of representable values");
+  }
+  {  // block maxima on and around 448 * 2^e
+    std::vector<double> x(3 * 32, 0.01);
+    x[0] = 448.0; x[32] = std::nextafter(448.0, 1e9); x[64] = std::nextafter(448.0, 0.0);
+    const auto p = w4::mxa::quantize_mx8(x, 3, 32);
+    t.expect(p.scales[0] == 127 && p.scales[1] == 128 && p.scales[2] == 127, "mx8 scale boundaries");
+    t.expect(p.q[0] == 0x7E && p.q[32] == 0x76 && p.q[64] == 0x7E, "mx8 codes at the boundaries");
+  }
+  t.throws_invalid([] { w4::mxa::quantize_mx8(std::vector<double>(4, 1.0), 0, 4); }, "quantize_mx8: bad dims");
+  t.throws_invalid([] { w4::mxa::quantize_mx8(std::vector<double>(5, 1.0), 1, 4); }, "quantize_mx8: size");
+  t.throws_invalid([] { w4::mxa::quantize_mx8(std::vector<double>(4, std::nan("")), 1, 4); },
+                   "quantize_mx8: non-finite input");
+  t.throws_invalid([] { w4::mxa::quantize_mx8(std::vector<double>(4, 1e300), 1, 4); },
+                   "quantize_mx8: block scale outside E8M0 range");
+}
+
 }  // namespace
 
 int main() {
   Checks t;
+  mx8_gates(t);
   w4_gates(t);
   mx_gates(t);
   kv_gates(t);

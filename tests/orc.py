@@ -166,6 +166,36 @@ def dequant_all_mx(p):
     return out
 
 
+# ---- MXFP8 activations (additive format) -------------------------------------
+class PackedXm8:
+    def __init__(self, M, K, q, scales):
+        self.M, self.K, self.B = M, K, (K + 31) // 32
+        self.q, self.scales = q, scales
+
+
+def quantize_mx8(x, M, K):
+    x = np.ascontiguousarray(x, np.float64).ravel()
+    q = np.zeros(max(1, M) * max(1, K), np.uint8)
+    s = np.zeros(max(1, M) * ((max(1, K) + 31) // 32), np.uint8)
+    _chk(lib().orc_quantize_mx8(_p(x), _sz(x.size), M, K, _p(q), _p(s)))
+    return PackedXm8(M, K, q, s)
+
+
+def dequant_mx8(p):
+    out = np.empty(p.M * p.K, np.float64)
+    _chk(lib().orc_dequant_mx8(p.M, p.K, _p(p.q), _p(p.scales), _p(out)))
+    return out.reshape(p.M, p.K)
+
+
+def gemm_f64(x, M, K, w, N):
+    x = np.ascontiguousarray(x, np.float64).ravel()
+    w = np.ascontiguousarray(w, np.float64).ravel()
+    assert x.size == M * K and w.size == N * K
+    c = np.empty(M * N, np.float64)
+    _chk(lib().orc_gemm_f64(_p(x), M, K, _p(w), N, _p(c)))
+    return c.reshape(M, N)
+
+
 # ---- KV caches -------------------------------------------------------------
 class KVCacheW4:
     pass

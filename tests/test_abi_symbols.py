@@ -76,3 +76,15 @@ def test_quantize_contracts():
         c.gemm_mx_w4a4(w, c.packed_mx_view(2, 64, 3, one, one), one)
     with pytest.raises(ValueError, match="null pointer"):
         c.quantize_mx_f16(c.packed_mx_view(2, 64, 2, one, one), 0, one)
+    # W4A8
+    x8 = c.act_mx8_view(2, 64, 2, 16, one)
+    with pytest.raises(ValueError, match="disagree on K"):
+        c.gemm_mx_w4a8(c.packed_mx_view(8, 32, 1, one, one), x8, one)
+    with pytest.raises(ValueError, match="multiple of 32"):
+        c.gemm_mx_w4a8(c.packed_mx_view(8, 40, 2, one, one), c.act_mx8_view(2, 40, 2, 16, one), one)
+    with pytest.raises(ValueError, match="16-byte aligned"):
+        c.gemm_mx_w4a8(w, c.act_mx8_view(2, 64, 2, 8, one), one)
+    with pytest.raises(ValueError, match="B inconsistent"):
+        c.gemm_mx_w4a8(w, c.act_mx8_view(2, 64, 3, 16, one), one)
+    with pytest.raises(ValueError, match="null pointer"):
+        c.quantize_mx8_f16(x8, 0, one)

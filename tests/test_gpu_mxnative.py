@@ -158,3 +158,105 @@ def test_w4a4_prefill_shape_sampled_rows():
     ref = _decode(xq, M)[rows] @ _decode(wq, N).T
     assert orc.rel_l2(got[rows], ref) <= TOL
     assert np.isfinite(got).all()
+
+
+# ---- W4A8: MXFP4 weights against MXFP8 (E4M3, block-scaled) activations ---------------
+W4A8_SHAPES = [(1, 64, 512), (16, 256, 4096), (5, 100, 992), (33, 80, 640), (64, 128, 1024),
+               (100, 64, 512), (2, 33, 32), (48, 16, 96), (300, 520, 384)]
+
+
+class _DevXm8:
+    def __init__(self, p):
+        c = w4amd.capi()
+        self.q, self.s = to_dev(p.q), to_dev(p.scales)
+        self.view = c.act_mx8_view(p.M, p.K, p.B, ptr(self.q), ptr(self.s))
+
+
+@pytest.mark.parametrize("i", range(len(W4A8_SHAPES)))
+def test_w4a8_matches_fp64_product(i):
+    """Activations quantized on the device carry the host quantizer's bytes
+    (include/w4/mxact.hpp, restated in the oracle); the product is within rel L2 1e-3 of
+    the FP64 product of the two dequantized operands."""
+    M, N, K = W4A8_SHAPES[i]
+    c = w4amd.capi()
+    w = orc.normal_weights(N * K, 0x8A8 + i)
+    x16 = orc.normal_activations(M * K, 0x8A9 + i)
+    xf = x16.view(np.float16).astype(np.float64)
+    xf[::7] *= 37.0  # spread the block maxima (still FP16 values after the cast below)
+    x16 = xf.astype(np.float16)
+    xf = x16.astype(np.float64)
+    wq, xq = orc.quantize_mx(w, N, K), orc.quantize_mx8(xf, M, K)
+    wd = orc.dequant_all_mx(wq).view(np.float16).astype(np.float64)
+    ref = orc.gemm_f64(orc.dequant_mx8(xq), M, K, wd, N)
+    B = (K + 31) // 32
+    q = torch.full((M * K,), 0x5A, dtype=torch.uint8, device=DEV)
+    s = torch.full((M * B,), 0x5A, dtype=torch.uint8, device=DEV)
+    st = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+    xd = to_dev(x16)
+    xview = c.act_mx8_view(M, K, B, ptr(q), ptr(s))
+    c.quantize_mx8_f16(xview, ptr(xd), ptr(st))
+    torch.cuda.synchronize()
+    assert int(st.item()) == 0
+    assert np.array_equal(s.cpu().numpy(), xq.scales)
+    assert np.array_equal(q.cpu().numpy(), xq.q)
+    dw = DevPackedMx(wq)
+    out = halves(M * N, 0x7E00)
+    c.gemm_mx_w4a8(dw.view, xview, ptr(out))
+    got = bits(out).view(np.float16).astype(np.float64).reshape(M, N)
+    assert orc.rel_l2(got, ref) <= TOL
+
+
+def test_w4a8_exact_when_sums_are_representable():
+    """Small integer activations (exact in E4M3) against weight codes in {0, +-0.5, +-1}:
+    every partial sum is a multiple of 0.5 below 2048, so the output bits are determined."""
+    M, N, K = 9, 40, 768
+    c = w4amd.capi()
+    rng = np.random.default_rng(8)
+    pick = np.array([0, 1, 2, 9, 10], np.uint32)
+    codes = pick[rng.integers(0, 5, (N, K))]
+    wq = orc.PackedWm(N, K, (codes.reshape(N, -1, 8) << (4 * np.arange(8, dtype=np.uint32))).sum(axis=2)
+                      .astype(np.uint32).ravel(), np.full(N * (K // 32), 127, np.uint8))
+    xv = rng.integers(-3, 4, (M, K)).astype(np.float64)
+    xq = orc.quantize_mx8(xv, M, K)
+    assert np.array_equal(orc.dequant_mx8(xq), xv)
+    ref = xv @ _decode(wq, N).T
+    assert np.abs(ref).max() < 2048
+    dw, dx = DevPackedMx(wq), _DevXm8(xq)
+    out = halves(M * N, 0x7E00)
+    c.gemm_mx_w4a8(dw.view, dx.view, ptr(out))
+    assert np.array_equal(bits(out).view(np.float16).reshape(M, N), ref.astype(np.float16))
+
+
+def test_w4a8_quantizer_boundaries_and_status():
+    """Block maxima on and beside 448 * 2^e, FP16 subnormals, zeros; non-finite input lands
+    in the status word."""
+    c = w4amd.capi()
+    rows = []
+    for e in range(-22, 8):
+        top = np.float16(448.0 * 2.0 ** e) if e <= 7 else None
+        for amax in (top, np.nextafter(top, np.float16(np.inf)), np.nextafter(top, np.float16(0))):
+            if not np.isfinite(amax):
+                continue
+            row = np.zeros(32, np.float16)
+            row[0], row[1] = amax, -amax
+            row[2:18] = (np.arange(16) / 16.0 * float(amax)).astype(np.float16)
+            row[18] = np.float16(6e-8)
+            row[19] = np.float16(-0.0)
+            rows.append(row)
+    x16 = np.array(rows, np.float16)
+    M, K = x16.shape
+    ref = orc.quantize_mx8(x16.astype(np.float64), M, K)
+    q = torch.zeros(M * K, dtype=torch.uint8, device=DEV)
+    s = torch.zeros(M, dtype=torch.uint8, device=DEV)
+    st = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+    xd = to_dev(x16.ravel())
+    view = c.act_mx8_view(M, K, 1, ptr(q), ptr(s))
+    c.quantize_mx8_f16(view, ptr(xd), ptr(st))
+    torch.cuda.synchronize()
+    assert int(st.item()) == 0
+    assert np.array_equal(s.cpu().numpy(), ref.scales)
+    assert np.array_equal(q.cpu().numpy(), ref.q)
+    x16[3, 5] = np.float16(np.inf)
+    c.quantize_mx8_f16(view, ptr(to_dev(x16.ravel())), ptr(st))
+    torch.cuda.synchronize()
+    assert int(st.item()) & 1

@@ -294,3 +294,33 @@ def test_paged_scatter_resolves_to_contiguous_rows():
     for badbt, pg in (([2, 0, 1], 0), ([0, 1], 16), ([0, 1, 1], 16), ([0, 1, 9], 16)):
         with pytest.raises(orc.OracleInvalid):
             orc.paged_scatter(c.q_k, H, S, pg, np.array(badbt, np.int32), wd)
+
+
+def test_mx8_activation_format_closed_forms():
+    """MXFP8 activations (an additive format, no reference counterpart): the block
+    exponent is the smallest e with amax <= 448 * 2^e, representable values round-trip
+    exactly, the per-element error is at most half an E4M3 step of the scaled value."""
+    rows = []
+    for e in range(-20, 20):
+        top = 448.0 * 2.0 ** e
+        for amax in (top, np.nextafter(top, np.inf), np.nextafter(top, 0.0)):
+            rows.append([amax, -amax] + [amax * t / 30.0 for t in range(30)])
+    x = np.array(rows)
+    M, K = x.shape
+    p = orc.quantize_mx8(x, M, K)
+    amax = np.abs(x).max(axis=1)
+    e = p.scales.astype(np.int64) - 127
+    assert np.all(amax <= 448.0 * 2.0 ** e) and np.all(amax > 448.0 * 2.0 ** (e - 1))
+    d = orc.dequant_mx8(p)
+    step = np.maximum(2.0 ** (np.floor(np.log2(np.maximum(np.abs(x) / 2.0 ** e[:, None], 1e-300))) - 3), 2.0 ** -9)
+    assert np.all(np.abs(d - x) <= 0.5 * step * 2.0 ** e[:, None] * (1 + 1e-9))
+    p2 = orc.quantize_mx8(d, M, K)
+    assert np.array_equal(orc.dequant_mx8(p2), d)
+    assert np.array_equal(orc.quantize_mx8(np.zeros(32), 1, 32).scales, [127])
+    with pytest.raises(ValueError, match="non-finite"):
+        orc.quantize_mx8(np.full(32, np.nan), 1, 32)
+    with pytest.raises(ValueError, match="E8M0 range"):
+        orc.quantize_mx8(np.full(32, 1e300), 1, 32)
+    # gemm_f64 against numpy
+    a, b = orc.normal_weights(5 * 64, 1).reshape(5, 64), orc.normal_weights(7 * 64, 2).reshape(7, 64)
+    assert np.allclose(orc.gemm_f64(a, 5, 64, b, 7), a @ b.T, rtol=1e-13, atol=1e-13)

@@ -23,6 +23,10 @@ class PackedMxView(C.Structure):
     _fields_ = [("N", C.c_int), ("K", C.c_int), ("B", C.c_int), ("q", vp), ("scales", vp)]
 
 
+class ActMx8View(C.Structure):
+    _fields_ = [("M", C.c_int), ("K", C.c_int), ("B", C.c_int), ("q", vp), ("scales", vp)]
+
+
 class KVView(C.Structure):
     _fields_ = [("H", C.c_int), ("S", C.c_int), ("D", C.c_int), ("gs", C.c_int), ("G", C.c_int),
                 ("symmetric", C.c_int), ("q_k", vp), ("s_k", vp), ("z_k", vp), ("q_v", vp),
@@ -61,6 +65,8 @@ SIGNATURES = {
     "w4_quantize_mx": ([C.POINTER(PackedMxView), vp, vp, vp], C.c_int),
     "w4_quantize_mx_f16": ([C.POINTER(PackedMxView), vp, vp, vp], C.c_int),
     "w4_gemm_mx_w4a4": ([C.POINTER(PackedMxView), C.POINTER(PackedMxView), vp, vp], C.c_int),
+    "w4_quantize_mx8_f16": ([C.POINTER(ActMx8View), vp, vp, vp], C.c_int),
+    "w4_gemm_mx_w4a8": ([C.POINTER(PackedMxView), C.POINTER(ActMx8View), vp, vp], C.c_int),
     "w4_quantize_cache": ([C.POINTER(KVView), vp, vp, C.c_int, vp, vp], C.c_int),
     "w4_quantize_cache_f8": ([C.POINTER(KVF8View), vp, vp, C.c_int, vp, vp], C.c_int),
 }
@@ -205,3 +211,16 @@ def quantize_mx_f16(view, x, status, stream=0):
 def gemm_mx_w4a4(w_view, x_view, c, stream=0):
     """Both operands packed MXFP4 (x_view.N = M); scaled matrix cores."""
     check(load().w4_gemm_mx_w4a4(C.byref(w_view), C.byref(x_view), _n(c), _n(stream)))
+
+
+def act_mx8_view(M, K, B, q, scales):
+    return ActMx8View(M, K, B, q or None, scales or None)
+
+
+def quantize_mx8_f16(view, x, status, stream=0):
+    check(load().w4_quantize_mx8_f16(C.byref(view), _n(x), _n(status), _n(stream)))
+
+
+def gemm_mx_w4a8(w_view, x_view, c, stream=0):
+    """MXFP4 weights against MXFP8 activations (x_view.M rows); scaled matrix cores."""
+    check(load().w4_gemm_mx_w4a8(C.byref(w_view), C.byref(x_view), _n(c), _n(stream)))

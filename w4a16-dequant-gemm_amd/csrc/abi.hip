@@ -396,6 +396,36 @@ int w4_gemm_mx_w4a4(const w4_packed_mx_view* w, const w4_packed_mx_view* x, w4_h
   return done("gemm_mx_w4a4", w4k::launch_gemm_mx_w4a4(*w, *x, c, (hipStream_t)stream));
 }
 
+static int check_mx8(const w4_act_mx8_view* p) {
+  REQUIRE(p != nullptr, "mx8: null view");
+  REQUIRE(p->M >= 1 && p->K >= 1, "mx8: bad dims");
+  REQUIRE(p->B == (p->K + 31) / 32, "mx8: B inconsistent with K");
+  REQUIRE(p->q && p->scales, "mx8: null pointer");
+  return W4_OK;
+}
+
+int w4_quantize_mx8_f16(const w4_act_mx8_view* out, const w4_half* x, int* status,
+                        w4_stream stream) {
+  if (int rc = check_mx8(out)) return rc;
+  REQUIRE(x && status, "quantize_mx8: null pointer");
+  if (int rc = start_status(status, stream, "quantize_mx8")) return rc;
+  return done("quantize_mx8",
+              w4k::launch_quantize_mx8(x, 1, out->M, out->K, (uint8_t*)out->q,
+                                       (uint8_t*)out->scales, status, (hipStream_t)stream));
+}
+
+int w4_gemm_mx_w4a8(const w4_packed_mx_view* w, const w4_act_mx8_view* x, w4_half* c,
+                    w4_stream stream) {
+  if (int rc = check_mx(w)) return rc;
+  if (int rc = check_mx8(x)) return rc;
+  REQUIRE(w->K == x->K, "mx w4a8: operands disagree on K");
+  REQUIRE(w->K % 32 == 0, "mx w4a8: K must be a multiple of 32");
+  REQUIRE(((uintptr_t)x->q & 15) == 0, "mx w4a8: x must be 16-byte aligned");
+  REQUIRE(c != nullptr, "mx w4a8: null pointer");
+  REQUIRE(x->M <= 65535LL * 64, "mx w4a8: launch grid out of range");
+  return done("gemm_mx_w4a8", w4k::launch_gemm_mx_w4a8(*w, *x, c, (hipStream_t)stream));
+}
+
 int w4_quantize_cache(const w4_kv_view* out, const void* k, const void* v, int src_f16,
                       int* status, w4_stream stream) {
   REQUIRE(out != nullptr, "quantize_cache: null view");

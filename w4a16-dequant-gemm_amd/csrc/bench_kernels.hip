@@ -55,7 +55,7 @@ extern "C" int w4bench_gemm_loop(w4bench_gemm_fn fn, const void* const* views, i
   return 0;
 }
 
-// The same loop for the two-view W4A4 entry point.
+// The same loop for the two-view W4A4 / W4A8 entry points.
 typedef int (*w4bench_w4a4_fn)(const void* w_view, const void* x_view, void* c, void* stream);
 extern "C" int w4bench_w4a4_loop(w4bench_w4a4_fn fn, const void* const* views, int nviews,
                                  const void* x_view, void* c, int steps, void* stream) {

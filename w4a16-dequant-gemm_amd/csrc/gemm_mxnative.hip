@@ -14,7 +14,8 @@
 //
 // Layout of the instruction (checked on the device against a host product):
 //   A: lane l holds row l%16, k-block l/16 (32 codes, 4 dwords)
-//   B: lane l holds column l%16, k-block l/16
+//   B: lane l holds column l%16, k-block l/16 (4-bit; an 8-bit B differs, see
+//      load_blocks8)
 //   D: lane l holds D[4*(l/16) + i][l%16], i = 0..3
 // W supplies A (rows n), X supplies B (columns m): a lane ends with four
 // consecutive n of one m.
@@ -38,6 +39,17 @@ __device__ __forceinline__ f4 mfma_fp4(u4 a, uint32_t sa, u4 b, uint32_t sb, f4 
   const v8i va = __builtin_shufflevector(a4, a4, 0, 1, 2, 3, -1, -1, -1, -1);
   const v8i vb = __builtin_shufflevector(b4, b4, 0, 1, 2, 3, -1, -1, -1, -1);
   return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(va, vb, c, FMT_FP4, FMT_FP4, 0,
+                                                          (int)sa, 0, (int)sb);
+}
+
+// The same with E4M3 activations: the B operand is 32 bytes (all eight registers).
+constexpr int FMT_FP8 = 0;
+__device__ __forceinline__ f4 mfma_fp4_fp8(u4 a, uint32_t sa, u4 b0, u4 b1, uint32_t sb, f4 c) {
+  const v4i a4 = __builtin_bit_cast(v4i, a);
+  const v8i va = __builtin_shufflevector(a4, a4, 0, 1, 2, 3, -1, -1, -1, -1);
+  const v4i lo = __builtin_bit_cast(v4i, b0), hi = __builtin_bit_cast(v4i, b1);
+  const v8i vb = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(va, vb, c, FMT_FP4, FMT_FP8, 0,
                                                           (int)sa, 0, (int)sb);
 }
 
@@ -74,12 +86,45 @@ __device__ __forceinline__ void load_blocks(const uint32_t* __restrict__ qrow,
   }
 }
 
+// The matching share of a row of E4M3 bytes (K a multiple of 32).  An 8-bit
+// operand is laid out differently from a 4-bit one (checked on the device element
+// by element): of the 128 k of MFMA j, lane group g holds k 16g..16g+15 in its
+// first four registers and k 64+16g..64+16g+15 in the other four, while its scale
+// register still carries the scale of 32-block g of those 128 k.  The four lane
+// groups of either load cover 64 contiguous bytes of every row.
+template <bool FULL>
+__device__ __forceinline__ void load_blocks8(const uint8_t* __restrict__ qrow,
+                                             const uint8_t* __restrict__ srow, int ss, int g,
+                                             int B, int K, u4 q[4][2], uint32_t sc[4]) {
+  if (FULL) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint8_t* p = qrow + (size_t)ss * 512 + 128 * j + 16 * g;
+      q[j][0] = *(const u4*)p;
+      q[j][1] = *(const u4*)(p + 64);
+    }
+    const u4 s16 = *(const u4*)(srow + ss * 16);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sc[j] = s16[j] >> (8 * g);
+  } else {
+    const u4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int k = ss * 512 + 128 * j + 16 * g, b = ss * 16 + 4 * j + g;
+      q[j][0] = k < K ? *(const u4*)(qrow + k) : zero;
+      q[j][1] = k + 64 < K ? *(const u4*)(qrow + k + 64) : zero;
+      sc[j] = b < B ? srow[b] : 127u;
+    }
+  }
+}
+
 // Skinny M: a workgroup owns 16*NT rows of W and 16*MT rows of X (grid.y walks
 // further X rows); its 8 waves take 512-k super-steps round-robin.  A wave
 // loads the X pieces of its super-step once and reuses them for the NT row
 // tiles, so X crosses L2 -> CU once per workgroup.  Partial sums meet in LDS
 // and are added in wave order.
-template <int MT, int NT, bool FULL>
+// XF8: X holds E4M3 bytes (K per row) instead of packed E2M1 codes.
+template <int MT, int NT, bool FULL, bool XF8>
 __global__ __launch_bounds__(NV_WAVES * 64) void mxn_decode_kernel(
     const uint32_t* __restrict__ wq, const uint8_t* __restrict__ ws,
     const uint32_t* __restrict__ xq, const uint8_t* __restrict__ xs, w4_half* __restrict__ c,
@@ -102,7 +147,7 @@ __global__ __launch_bounds__(NV_WAVES * 64) void mxn_decode_kernel(
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = m0 + mt * 16 + r < M ? m0 + mt * 16 + r : M - 1;
-    xrow[mt] = xq + (size_t)m * wk;
+    xrow[mt] = xq + (size_t)m * (XF8 ? K >> 2 : wk);  // K bytes or words(K) words a row
     xsrow[mt] = xs + (size_t)m * B;
   }
   f4 acc[NT][MT];
@@ -113,14 +158,22 @@ __global__ __launch_bounds__(NV_WAVES * 64) void mxn_decode_kernel(
 
   const int supers = (B + 15) >> 4;
   for (int ss = wave; ss < supers; ss += NV_WAVES) {
-    u4 b[MT][4], a[NT][4];
+    u4 b[MT][4][XF8 ? 2 : 1], a[NT][4];
     uint32_t sb[MT][4], sa[NT][4];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
       load_blocks<FULL>(wrow[nt], wsrow[nt], ss, g, B, wk, K, a[nt], sa[nt]);
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-      load_blocks<FULL>(xrow[mt], xsrow[mt], ss, g, B, wk, K, b[mt], sb[mt]);
+    for (int mt = 0; mt < MT; ++mt) {
+      if constexpr (XF8) {
+        load_blocks8<FULL>((const uint8_t*)xrow[mt], xsrow[mt], ss, g, B, K, b[mt], sb[mt]);
+      } else {
+        u4 q[4];
+        load_blocks<FULL>(xrow[mt], xsrow[mt], ss, g, B, wk, K, q, sb[mt]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b[mt][j][0] = q[j];
+      }
+    }
     // every load of the super-step is in flight before the first product waits
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -128,8 +181,13 @@ __global__ __launch_bounds__(NV_WAVES * 64) void mxn_decode_kernel(
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[nt][mt] = mfma_fp4(a[nt][j], sa[nt][j], b[mt][j], sb[mt][j], acc[nt][mt]);
+        for (int j = 0; j < 4; ++j) {
+          if constexpr (XF8)
+            acc[nt][mt] = mfma_fp4_fp8(a[nt][j], sa[nt][j], b[mt][j][0], b[mt][j][1], sb[mt][j],
+                                       acc[nt][mt]);
+          else
+            acc[nt][mt] = mfma_fp4(a[nt][j], sa[nt][j], b[mt][j][0], sb[mt][j], acc[nt][mt]);
+        }
   }
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
@@ -161,37 +219,46 @@ __global__ __launch_bounds__(NV_WAVES * 64) void mxn_decode_kernel(
   }
 }
 
-template <int MT, int NT>
-hipError_t launch_decode_nt(const w4_packed_mx_view& w, const w4_packed_mx_view& x, w4_half* c,
-                            hipStream_t s) {
-  const int N = w.N, K = w.K, M = x.N;
-  const bool full = K % 512 == 0 && ((uintptr_t)w.q & 15) == 0 && ((uintptr_t)x.q & 15) == 0 &&
-                    ((uintptr_t)w.scales & 15) == 0 && ((uintptr_t)x.scales & 15) == 0;
+template <int MT, int NT, bool XF8>
+hipError_t launch_decode_nt(const w4_packed_mx_view& w, const void* xq, const uint8_t* xs, int M,
+                            w4_half* c, hipStream_t s) {
+  const int N = w.N, K = w.K;
+  const bool full = K % 512 == 0 && ((uintptr_t)w.q & 15) == 0 && ((uintptr_t)xq & 15) == 0 &&
+                    ((uintptr_t)w.scales & 15) == 0 && ((uintptr_t)xs & 15) == 0;
   const dim3 grid((unsigned)((N + 16 * NT - 1) / (16 * NT)),
                   (unsigned)((M + 16 * MT - 1) / (16 * MT)));
   const dim3 block(NV_WAVES * 64);
   if (full)
-    mxn_decode_kernel<MT, NT, true><<<grid, block, 0, s>>>(w.q, w.scales, x.q, x.scales, c, N,
-                                                          K, w.B, M);
+    mxn_decode_kernel<MT, NT, true, XF8><<<grid, block, 0, s>>>(
+        w.q, w.scales, (const uint32_t*)xq, xs, c, N, K, w.B, M);
   else
-    mxn_decode_kernel<MT, NT, false><<<grid, block, 0, s>>>(w.q, w.scales, x.q, x.scales, c, N,
-                                                           K, w.B, M);
+    mxn_decode_kernel<MT, NT, false, XF8><<<grid, block, 0, s>>>(
+        w.q, w.scales, (const uint32_t*)xq, xs, c, N, K, w.B, M);
   return hipGetLastError();
 }
 
 // Row tiles per workgroup: as many as keep at least one workgroup per CU.
-template <int MT>
-hipError_t launch_decode(const w4_packed_mx_view& w, const w4_packed_mx_view& x, w4_half* c,
-                         hipStream_t s) {
+template <int MT, bool XF8>
+hipError_t launch_decode(const w4_packed_mx_view& w, const void* xq, const uint8_t* xs, int M,
+                         w4_half* c, hipStream_t s) {
   const int tiles = (w.N + 15) / 16;
-  const int mblocks = (x.N + 16 * MT - 1) / (16 * MT);
+  const int mblocks = (M + 16 * MT - 1) / (16 * MT);
   // more row tiles per workgroup cut the X traffic (every workgroup reads all of
   // its X rows through L2): worth it from three X tiles on, while a workgroup per
   // CU remains (N = 14336, M = 64: 21.8 us with three row tiles, 29.5 us with one)
   const int nt = MT >= 3 ? tiles * mblocks / 256 : 1;
-  if (nt >= 3) return launch_decode_nt<MT, 3>(w, x, c, s);
-  if (nt >= 2) return launch_decode_nt<MT, 2>(w, x, c, s);
-  return launch_decode_nt<MT, 1>(w, x, c, s);
+  if (nt >= 3) return launch_decode_nt<MT, 3, XF8>(w, xq, xs, M, c, s);
+  if (nt >= 2) return launch_decode_nt<MT, 2, XF8>(w, xq, xs, M, c, s);
+  return launch_decode_nt<MT, 1, XF8>(w, xq, xs, M, c, s);
+}
+
+template <bool XF8>
+hipError_t launch_skinny(const w4_packed_mx_view& w, const void* xq, const uint8_t* xs, int M,
+                         w4_half* c, hipStream_t s) {
+  if (M <= 16) return launch_decode<1, XF8>(w, xq, xs, M, c, s);
+  if (M <= 32) return launch_decode<2, XF8>(w, xq, xs, M, c, s);
+  if (M <= 48) return launch_decode<3, XF8>(w, xq, xs, M, c, s);
+  return launch_decode<4, XF8>(w, xq, xs, M, c, s);
 }
 
 // ---- large M: LDS-tiled kernel -----------------------------------------------
@@ -450,12 +517,15 @@ hipError_t launch_tile(const w4_packed_mx_view& w, const w4_packed_mx_view& x, w
 
 hipError_t launch_gemm_mx_w4a4(const w4_packed_mx_view& w, const w4_packed_mx_view& x,
                                w4_half* c, hipStream_t s) {
-  const int M = x.N;
   if (tile_applies(w, x)) return launch_tile(w, x, c, s);
-  if (M <= 16) return launch_decode<1>(w, x, c, s);
-  if (M <= 32) return launch_decode<2>(w, x, c, s);
-  if (M <= 48) return launch_decode<3>(w, x, c, s);
-  return launch_decode<4>(w, x, c, s);
+  return launch_skinny<false>(w, x.q, x.scales, x.N, c, s);
+}
+
+// E4M3 activations (K a multiple of 32, rows 16-byte aligned): the skinny kernel
+// for every M (grid.y walks the rows of X).
+hipError_t launch_gemm_mx_w4a8(const w4_packed_mx_view& w, const w4_act_mx8_view& x, w4_half* c,
+                               hipStream_t s) {
+  return launch_skinny<true>(w, x.q, x.scales, x.M, c, s);
 }
 
 }  // namespace w4k

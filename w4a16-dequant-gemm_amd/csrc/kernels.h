@@ -99,6 +99,10 @@ hipError_t launch_quantize_mx(const void* src, int src_f16, long long rows, int 
 // gemm_mxnative.hip -- both operands packed MXFP4 (x.N = M rows of K), scaled MFMA
 hipError_t launch_gemm_mx_w4a4(const w4_packed_mx_view& w, const w4_packed_mx_view& x,
                                w4_half* c, hipStream_t s);
+hipError_t launch_gemm_mx_w4a8(const w4_packed_mx_view& w, const w4_act_mx8_view& x, w4_half* c,
+                               hipStream_t s);
+hipError_t launch_quantize_mx8(const void* src, int src_f16, long long rows, int K, uint8_t* q,
+                               uint8_t* scales, int* status, hipStream_t s);
 hipError_t launch_fill_words(uint32_t* p, long long n, uint32_t value, hipStream_t s);
 
 }  // namespace w4k

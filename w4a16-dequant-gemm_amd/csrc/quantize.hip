@@ -360,13 +360,17 @@ __global__ __launch_bounds__(QT) void quantize_rows_fast_kernel(
   }
 }
 
-// mx.hpp:91-101 in closed form: the smallest e with amax <= 6 * 2^e.
+// mx.hpp:91-101 in closed form: the smallest e with amax <= TOP * 2^e, TOP the
+// largest magnitude of the element type (6 for E2M1, 448 for E4M3).  With amax in
+// [2^p, 2^(p+1)) the answer lies within two steps of p - ilogb(TOP).
+template <int TOP>
 __device__ __forceinline__ int mx_exponent(double amax, bool* out_of_range) {
   if (!(amax > 0.0)) return 0;
-  if (amax <= 6.0 * 0x1p-127) return -127;
+  if (amax <= (double)TOP * 0x1p-127) return -127;
   const int p = (int)((__builtin_bit_cast(uint64_t, amax) >> 52) & 0x7FFu) - 1023;
-  int e = p - 2;  // 6 * 2^(p-3) < 2^p <= amax, and amax < 2^(p+1) < 6 * 2^(p-1)
-  if (amax > 6.0 * ldexp(1.0, e)) ++e;
+  int e = p - (TOP == 6 ? 2 : 9);  // TOP * 2^(e - 1) < 2^p <= amax
+  if (amax > (double)TOP * ldexp(1.0, e)) ++e;
+  if (amax > (double)TOP * ldexp(1.0, e)) ++e;
   if (e > 127) {
     *out_of_range = true;
     e = 127;
@@ -390,11 +394,14 @@ __device__ __forceinline__ int nearest_e2m1(double a) {
   return best;
 }
 
-// Four threads per 32-element block, one packed word each.
-template <typename T, bool FULL>
+// Four threads per 32-element block, eight elements each: one packed word of
+// E2M1 codes, or (F8: the MXFP8 activation format, no host counterpart in the
+// reference; same block rule with 448 in place of 6) eight E4M3 bytes.
+template <typename T, bool FULL, bool F8>
 __global__ __launch_bounds__(QT) void quantize_mx_kernel(const T* __restrict__ src,
                                                          long long rows, int K, int B,
                                                          uint32_t* __restrict__ q,
+                                                         uint8_t* __restrict__ q8,
                                                          uint8_t* __restrict__ scales,
                                                          int* __restrict__ status) {
   const long long id = (long long)blockIdx.x * QT + threadIdx.x;
@@ -430,19 +437,36 @@ __global__ __launch_bounds__(QT) void quantize_mx_kernel(const T* __restrict__ s
   amax = fmax(amax, __shfl_xor(amax, 1));
   amax = fmax(amax, __shfl_xor(amax, 2));
   bool range = false;
-  const int e = mx_exponent(amax, &range);
+  const int e = mx_exponent<F8 ? 448 : 6>(amax, &range);
   if (range && j4 == 0) atomicOr(status, 2);
   if (n == 0) return;
   const double scale = ldexp(1.0, e);
-  uint32_t word = 0;
+  if (F8) {
+    uint8_t* dst = q8 + row * (long long)K + k0;
+    uint32_t c[8];
 #pragma unroll
-  for (int j = 0; j < 8; ++j)
-    if (j < n) {
-      const double u = v[j] / scale;
-      const uint32_t code = (__builtin_signbit(u) ? 8u : 0u) | (uint32_t)nearest_e2m1(fabs(u));
-      word |= code << (4 * j);
+    for (int j = 0; j < 8; ++j) c[j] = encode_e4m3((float)(v[j] / scale));
+    if (n == 8 && ((uintptr_t)dst & 7) == 0) {
+      u2 out;
+      out[0] = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+      out[1] = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
+      *(u2*)dst = out;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (j < n) dst[j] = (uint8_t)c[j];
     }
-  q[row * (long long)words(K) + b * 4 + j4] = word;
+  } else {
+    uint32_t word = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (j < n) {
+        const double u = v[j] / scale;
+        const uint32_t code = (__builtin_signbit(u) ? 8u : 0u) | (uint32_t)nearest_e2m1(fabs(u));
+        word |= code << (4 * j);
+      }
+    q[row * (long long)words(K) + b * 4 + j4] = word;
+  }
   if (j4 == 0) scales[blk] = (uint8_t)(e + 127);
 }
 
@@ -519,15 +543,31 @@ hipError_t launch_quantize_mx(const void* src, int src_f16, long long rows, int 
   const int B = (K + 31) / 32;
   const long long blocks = (rows * B * 4 + QT - 1) / QT;
   if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
+  const dim3 grid((unsigned)blocks), block(QT);
   if (src_f16)
-    quantize_mx_kernel<_Float16, false><<<dim3((unsigned)blocks), dim3(QT), 0, s>>>(
-        (const _Float16*)src, rows, K, B, q, scales, status);
+    quantize_mx_kernel<_Float16, false, false><<<grid, block, 0, s>>>((const _Float16*)src, rows, K,
+                                                                     B, q, nullptr, scales, status);
   else if (K % 8 == 0 && ((uintptr_t)src & 15) == 0)
-    quantize_mx_kernel<double, true><<<dim3((unsigned)blocks), dim3(QT), 0, s>>>(
-        (const double*)src, rows, K, B, q, scales, status);
+    quantize_mx_kernel<double, true, false><<<grid, block, 0, s>>>((const double*)src, rows, K, B,
+                                                                  q, nullptr, scales, status);
   else
-    quantize_mx_kernel<double, false><<<dim3((unsigned)blocks), dim3(QT), 0, s>>>(
-        (const double*)src, rows, K, B, q, scales, status);
+    quantize_mx_kernel<double, false, false><<<grid, block, 0, s>>>((const double*)src, rows, K, B,
+                                                                   q, nullptr, scales, status);
+  return hipGetLastError();
+}
+
+hipError_t launch_quantize_mx8(const void* src, int src_f16, long long rows, int K, uint8_t* q,
+                               uint8_t* scales, int* status, hipStream_t s) {
+  const int B = (K + 31) / 32;
+  const long long blocks = (rows * B * 4 + QT - 1) / QT;
+  if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
+  const dim3 grid((unsigned)blocks), block(QT);
+  if (src_f16)
+    quantize_mx_kernel<_Float16, false, true><<<grid, block, 0, s>>>((const _Float16*)src, rows, K,
+                                                                    B, nullptr, q, scales, status);
+  else
+    quantize_mx_kernel<double, false, true><<<grid, block, 0, s>>>((const double*)src, rows, K, B,
+                                                                  nullptr, q, scales, status);
   return hipGetLastError();
 }
 

@@ -402,7 +402,7 @@ def extras_w4a4(b, full):
             us = b.w4a4_us(views, M, N, K)
             rows.append({"N": N, "K": K, "M": M, "bytes": nb, "us": us, "GBs": nb / us * 1e-3,
                          "TFLOPs": 2.0 * M * N * K / us * 1e-6})
-            if M <= 256:  # E4M3 activations (skinny kernel only)
+            if M <= 256 or M == 2048:  # E4M3 activations
                 us8 = b.w4a4_us(views, M, N, K, a8=True)
                 rows[-1].update({"a8_us": us8, "a8_TFLOPs": 2.0 * M * N * K / us8 * 1e-6})
         del views

@@ -162,7 +162,9 @@ def test_w4a4_prefill_shape_sampled_rows():
 
 # ---- W4A8: MXFP4 weights against MXFP8 (E4M3, block-scaled) activations ---------------
 W4A8_SHAPES = [(1, 64, 512), (16, 256, 4096), (5, 100, 992), (33, 80, 640), (64, 128, 1024),
-               (100, 64, 512), (2, 33, 32), (48, 16, 96), (300, 520, 384)]
+               (100, 64, 512), (2, 33, 32), (48, 16, 96), (300, 520, 384),
+               # at least 64 tiles and K % 256 == 0: the LDS-tiled kernel with 8-bit X
+               (900, 2100, 512), (1030, 2050, 768), (1024, 2048, 1280)]
 
 
 class _DevXm8:
@@ -260,3 +262,20 @@ def test_w4a8_quantizer_boundaries_and_status():
     c.quantize_mx8_f16(view, ptr(to_dev(x16.ravel())), ptr(st))
     torch.cuda.synchronize()
     assert int(st.item()) & 1
+
+
+def test_w4a8_prefill_shape_sampled_rows():
+    M, N, K = 2048, 4096, 4096
+    c = w4amd.capi()
+    wq = orc.quantize_mx(orc.normal_weights(N * K, 23), N, K)
+    x16 = orc.normal_activations(M * K, 24)
+    xq = orc.quantize_mx8(x16.view(np.float16).astype(np.float64), M, K)
+    dw, dx = DevPackedMx(wq), _DevXm8(xq)
+    out = halves(M * N, 0x7E00)
+    c.gemm_mx_w4a8(dw.view, dx.view, ptr(out))
+    got = bits(out).view(np.float16).astype(np.float64).reshape(M, N)
+    rows = np.unique(np.concatenate([np.arange(0, 16), np.arange(M - 16, M),
+                                     np.random.default_rng(6).integers(0, M, 64)]))
+    ref = orc.dequant_mx8(xq)[rows] @ _decode(wq, N).T
+    assert orc.rel_l2(got[rows], ref) <= TOL
+    assert np.isfinite(got).all()

@@ -287,26 +287,46 @@ __device__ __forceinline__ f16v mfma_fp4_32(u4 a, uint32_t sa, u4 b, uint32_t sb
 // neighbouring lanes still cover one contiguous line (coalesced), and the 16
 // rows x 16 bytes a lane group reads back for one MFMA operand land on 16
 // distinct 16-byte bank groups (conflict-free ds_read_b128 without padding).
-// No staging registers, no ds_write instructions: DM_STAGES stages of 256 k sit
-// in LDS (dynamic LDS, 153 KB); one barrier per stage.  Per stage d: multiply
+// No staging registers, no ds_write instructions: three stages of 256 k sit in
+// LDS (dynamic LDS, 153 KB; two stages, 134 KB, with 8-bit X); one barrier per stage.  Per stage d: multiply
 // the first 128 k of d while reading the operands of the second; wait for d+1,
 // barrier -- every wave is now done with d's buffer, so request d+3 into it;
 // multiply the second 128 k while reading the first operands of d+1.
-constexpr int DM_STAGES = 3;
-constexpr int DM_W_BYTES = TL_TN * 128, DM_X_BYTES = TL_TM * 128;
-constexpr int DM_TILE_BYTES = DM_W_BYTES + DM_X_BYTES;       // 48 KB, unpadded
-constexpr int DM_STAGE = DM_TILE_BYTES + 2 * TL_ROWS * 4;    // + two scale dwords per row
+// XF8: X holds E4M3 bytes -- rows of 256 bytes per stage, four rows per load
+// instruction, piece key = row % 16, and room for two stages instead of three.
+constexpr int DM_W_BYTES = TL_TN * 128;
 constexpr int DM_WN = 4;                                     // waves along n (2 along m)
 constexpr int DM_WAVES = 2 * DM_WN;
 constexpr int DM_THREADS = 64 * DM_WAVES;
 constexpr int DM_NT = TL_TN / (32 * DM_WN);                  // 32-row tiles of W per wave
-constexpr int DM_WI = 32 / DM_WAVES, DM_XI = 16 / DM_WAVES;  // 8-row blocks a wave fetches
-constexpr int DM_LOADS = DM_WI + DM_XI + 2;                  // wave instructions per stage
+constexpr int DM_WI = 32 / DM_WAVES;                         // 8-row blocks of W a wave fetches
+template <bool XF8>
+struct Dm {
+  static constexpr int STAGES = XF8 ? 2 : 3;
+  static constexpr int X_ROWB = XF8 ? 256 : 128;             // bytes of an X row per stage
+  static constexpr int X_BYTES = TL_TM * X_ROWB;
+  static constexpr int TILE_BYTES = DM_W_BYTES + X_BYTES;    // 48 / 64 KB, unpadded
+  static constexpr int STAGE = TILE_BYTES + 2 * TL_ROWS * 4; // + two scale dwords per row
+  static constexpr int XI = X_BYTES / 1024 / DM_WAVES;       // 1 KB blocks of X a wave fetches
+  static constexpr int LOADS = DM_WI + XI + 2;               // wave instructions per stage
+  static constexpr int NB = XF8 ? 2 : 1;                     // register quads of a B operand
+};
 
+template <bool XF8>
 struct DmFrags {  // one lane's MFMA operands of a 128-k half: [k half][tile]
-  u4 a[2][DM_NT], b[2][2];
+  u4 a[2][DM_NT], b[2][2][Dm<XF8>::NB];
   uint32_t sa[DM_NT], sb[2];
 };
+
+__device__ __forceinline__ f16v mfma_fp4_fp8_32(u4 a, uint32_t sa, u4 b0, u4 b1, uint32_t sb,
+                                                f16v c) {
+  const v4i a4 = __builtin_bit_cast(v4i, a);
+  const v8i va = __builtin_shufflevector(a4, a4, 0, 1, 2, 3, -1, -1, -1, -1);
+  const v4i lo = __builtin_bit_cast(v4i, b0), hi = __builtin_bit_cast(v4i, b1);
+  const v8i vb = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va, vb, c, FMT_FP4, FMT_FP8, 0, (int)sa,
+                                                         0, (int)sb);
+}
 
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
@@ -315,6 +335,7 @@ constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; 
 
 extern __shared__ __attribute__((aligned(16))) uint8_t dm_lds[];
 
+template <bool XF8>
 __global__ __launch_bounds__(DM_THREADS) void mxn_tile_dma_kernel(
     const uint32_t* __restrict__ wq, const uint8_t* __restrict__ ws,
     const uint32_t* __restrict__ xq, const uint8_t* __restrict__ xs, w4_half* __restrict__ c,
@@ -336,17 +357,25 @@ __global__ __launch_bounds__(DM_THREADS) void mxn_tile_dma_kernel(
   // what this lane fetches: row l/8 of an 8-row block, swizzled 16-byte piece.
   // Wave w takes blocks w + 4 i; the key only needs the row's position in its
   // 16-row group: ((block & 1) * 8 + l/8) / 2.
+  typedef Dm<XF8> C;
   const int row8 = lane >> 3;
-  uint32_t wo[DM_WI], xo[DM_XI];  // byte offsets (32-bit: tile_applies bounds the operands)
+  uint32_t wo[DM_WI], xo[C::XI];  // byte offsets (32-bit: tile_applies bounds the operands)
 #pragma unroll
   for (int i = 0; i < DM_WI; ++i) {
     const int blk = wave + DM_WAVES * i, R = blk * 8 + row8, n = n0 + R;
     wo[i] = ((uint32_t)(n < N ? n : N - 1) * (uint32_t)wk) * 4u + (((lane & 7) ^ ((R >> 1) & 7)) * 16);
   }
 #pragma unroll
-  for (int i = 0; i < DM_XI; ++i) {
-    const int blk = wave + DM_WAVES * i, R = blk * 8 + row8, m = m0 + R;
-    xo[i] = ((uint32_t)(m < M ? m : M - 1) * (uint32_t)wk) * 4u + (((lane & 7) ^ ((R >> 1) & 7)) * 16);
+  for (int i = 0; i < C::XI; ++i) {
+    const int blk = wave + DM_WAVES * i;
+    if (XF8) {  // 4 rows of 256 bytes per instruction, piece key R % 16, K bytes a row
+      const int R = blk * 4 + (lane >> 4), m = m0 + R;
+      xo[i] = (uint32_t)(m < M ? m : M - 1) * (uint32_t)K + (((lane & 15) ^ (R & 15)) * 16);
+    } else {
+      const int R = blk * 8 + row8, m = m0 + R;
+      xo[i] = ((uint32_t)(m < M ? m : M - 1) * (uint32_t)wk) * 4u +
+              (((lane & 7) ^ ((R >> 1) & 7)) * 16);
+    }
   }
   // scale dwords: waves 0-3 take W rows 64 wave + lane, the others X rows 64 (wave & 1)
   // + lane (a wave fetches two per stage either way)
@@ -378,28 +407,38 @@ __global__ __launch_bounds__(DM_THREADS) void mxn_tile_dma_kernel(
   const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr)dm_lds;
   auto request = [&](int d) {
     const uint32_t dd = (uint32_t)(d < stages ? d : stages - 1);  // past the end: valid, never used
-    const uint32_t st = lds0 + (uint32_t)(d % DM_STAGES) * DM_STAGE;
+    const uint32_t st = lds0 + (uint32_t)(d % C::STAGES) * C::STAGE;
 #pragma unroll
     for (int i = 0; i < DM_WI; ++i)
       dma16(wqb, wo[i] + dd * 128u, st + (wave + DM_WAVES * i) * 1024);
 #pragma unroll
-    for (int i = 0; i < DM_XI; ++i)
-      dma16(xqb, xo[i] + dd * 128u, st + DM_W_BYTES + (wave + DM_WAVES * i) * 1024);
+    for (int i = 0; i < C::XI; ++i)
+      dma16(xqb, xo[i] + dd * (uint32_t)C::X_ROWB, st + DM_W_BYTES + (wave + DM_WAVES * i) * 1024);
 #pragma unroll
     for (int s2 = 0; s2 < 2; ++s2)  // the two 128-k halves' scale dwords
-      dma4(scb, sco + dd * 8u + s2 * 4u, st + DM_TILE_BYTES + s2 * (TL_ROWS * 4) + sc_lds);
+      dma4(scb, sco + dd * 8u + s2 * 4u, st + C::TILE_BYTES + s2 * (TL_ROWS * 4) + sc_lds);
   };
   // row R of an operand tile, 16-byte piece p (0..7) of the 256 k -> byte offset
   auto at = [](int R, int p) { return (R >> 3) * 1024 + ((R & 7) * 8 + (p ^ ((R >> 1) & 7))) * 16; };
   // operands of the 128-k half s2 of stage d
-  auto read_frags = [&](DmFrags& f, int d, int s2) {
-    const uint8_t* base = dm_lds + (d % DM_STAGES) * DM_STAGE;
-    const uint32_t* sc = (const uint32_t*)(base + DM_TILE_BYTES) + s2 * TL_ROWS;
+  // the same for a 256-byte row of E4M3 bytes, piece p in 0..15
+  auto at8 = [](int R, int p) { return (R >> 2) * 1024 + ((R & 3) * 16 + (p ^ (R & 15))) * 16; };
+  auto read_frags = [&](DmFrags<XF8>& f, int d, int s2) {
+    const uint8_t* base = dm_lds + (d % C::STAGES) * C::STAGE;
+    const uint32_t* sc = (const uint32_t*)(base + C::TILE_BYTES) + s2 * TL_ROWS;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int row = wm * 64 + j * 32 + r;
-      f.b[0][j] = *(const u4*)(base + DM_W_BYTES + at(row, 4 * s2 + h));
-      f.b[1][j] = *(const u4*)(base + DM_W_BYTES + at(row, 4 * s2 + 2 + h));
+#pragma unroll
+      for (int kh = 0; kh < 2; ++kh) {
+        if constexpr (XF8) {
+          // of the 64 k of MFMA kh an 8-bit lane group h holds k 16h.. and 32+16h..
+          f.b[kh][j][0] = *(const u4*)(base + DM_W_BYTES + at8(row, 8 * s2 + 4 * kh + h));
+          f.b[kh][j][1] = *(const u4*)(base + DM_W_BYTES + at8(row, 8 * s2 + 4 * kh + 2 + h));
+        } else {
+          f.b[kh][j][0] = *(const u4*)(base + DM_W_BYTES + at(row, 4 * s2 + 2 * kh + h));
+        }
+      }
       f.sb[j] = sc[TL_TN + row];
     }
 #pragma unroll
@@ -418,7 +457,7 @@ __global__ __launch_bounds__(DM_THREADS) void mxn_tile_dma_kernel(
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-  auto multiply = [&](const DmFrags& f) {
+  auto multiply = [&](const DmFrags<XF8>& f) {
 #pragma unroll
     for (int kh = 0; kh < 2; ++kh) {
       const int sh = 16 * kh + 8 * h;
@@ -426,15 +465,21 @@ __global__ __launch_bounds__(DM_THREADS) void mxn_tile_dma_kernel(
       for (int i = 0; i < DM_NT; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
-          acc[i][j] = mfma_fp4_32(f.a[kh][i], f.sa[i] >> sh, f.b[kh][j], f.sb[j] >> sh, acc[i][j]);
+        {
+          if constexpr (XF8)
+            acc[i][j] = mfma_fp4_fp8_32(f.a[kh][i], f.sa[i] >> sh, f.b[kh][j][0], f.b[kh][j][1],
+                                        f.sb[j] >> sh, acc[i][j]);
+          else
+            acc[i][j] = mfma_fp4_32(f.a[kh][i], f.sa[i] >> sh, f.b[kh][j][0], f.sb[j] >> sh, acc[i][j]);
+        }
     }
   };
 
-  DmFrags fa, fb;
-  request(0);
-  request(1);
-  request(2);
-  __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * DM_LOADS));  // stage 0 has landed (this wave's part)
+  DmFrags<XF8> fa, fb;
+#pragma unroll
+  for (int d = 0; d < C::STAGES; ++d) request(d);
+  // stage 0 has landed (this wave's part)
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm((C::STAGES - 1) * C::LOADS));
   __syncthreads();
   read_frags(fa, 0, 0);
 #pragma unroll 1
@@ -443,10 +488,10 @@ __global__ __launch_bounds__(DM_THREADS) void mxn_tile_dma_kernel(
     __builtin_amdgcn_sched_barrier(0);
     multiply(fa);
     __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(DM_LOADS));  // stage d + 1 has landed
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm((C::STAGES - 2) * C::LOADS));  // stage d + 1 has landed
     __syncthreads();
-    // every wave has read both halves of stage d: its buffer takes stage d + 3
-    request(d + 3);
+    // every wave has read both halves of stage d: its buffer takes the next stage to request
+    request(d + C::STAGES);
     read_frags(fa, d + 1, 0);
     __builtin_amdgcn_sched_barrier(0);
     multiply(fb);
@@ -480,36 +525,36 @@ __global__ __launch_bounds__(DM_THREADS) void mxn_tile_dma_kernel(
   }
 }
 
-bool tile_applies(const w4_packed_mx_view& w, const w4_packed_mx_view& x) {
-  // Worth it once the tile grid covers a good part of the chip; below that the
-  // skinny kernel's grid.y walk is faster (measured at K = 4096: N = 4096, M = 256
-  // -> 32 tiles 37 us here, 23 us there; M = 512 -> 64 tiles 31 us here; N = 14336,
-  // M = 256 -> 112 tiles 34 us here, 54 us there).
-  const long long tiles = (long long)((w.N + TL_TN - 1) / TL_TN) * ((x.N + TL_TM - 1) / TL_TM);
-  return x.N >= 128 && tiles >= 64 && w.K % 256 == 0 && (long long)w.N * w.K < (1LL << 32) &&
-         (long long)x.N * x.K < (1LL << 32) && ((uintptr_t)w.q & 15) == 0 &&
-         ((uintptr_t)x.q & 15) == 0 && ((uintptr_t)w.scales & 7) == 0 &&
-         ((uintptr_t)x.scales & 7) == 0;
+// Worth it once the tile grid covers a good part of the chip; below that the
+// skinny kernel's grid.y walk is faster (measured at K = 4096: N = 4096, M = 256
+// -> 32 tiles 37 us here, 23 us there; M = 512 -> 64 tiles 31 us here; N = 14336,
+// M = 256 -> 112 tiles 34 us here, 54 us there).  x_row_bytes: K/2 or K.
+bool tile_applies(const w4_packed_mx_view& w, const void* xq, const uint8_t* xs, int M,
+                  int x_row_bytes) {
+  const long long tiles = (long long)((w.N + TL_TN - 1) / TL_TN) * ((M + TL_TM - 1) / TL_TM);
+  return M >= 128 && tiles >= 64 && w.K % 256 == 0 && (long long)w.N * w.K < (1LL << 32) &&
+         (long long)M * x_row_bytes < (1LL << 32) && ((uintptr_t)w.q & 15) == 0 &&
+         ((uintptr_t)xq & 15) == 0 && ((uintptr_t)w.scales & 7) == 0 && ((uintptr_t)xs & 7) == 0;
 }
 
-hipError_t launch_tile(const w4_packed_mx_view& w, const w4_packed_mx_view& x, w4_half* c,
-                       hipStream_t s) {
-  const int tiles_n = (w.N + TL_TN - 1) / TL_TN, tiles_m = (x.N + TL_TM - 1) / TL_TM;
+template <bool XF8>
+hipError_t launch_tile(const w4_packed_mx_view& w, const void* xq, const uint8_t* xs, int M,
+                       w4_half* c, hipStream_t s) {
+  const int tiles_n = (w.N + TL_TN - 1) / TL_TN, tiles_m = (M + TL_TM - 1) / TL_TM;
   if ((long long)tiles_n * tiles_m > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
+  constexpr int lds_bytes = Dm<XF8>::STAGES * Dm<XF8>::STAGE;
   // more than 64 KB of LDS has to be granted per device, once
   static bool granted[64] = {};
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
   if (dev < 0 || dev >= 64 || !granted[dev]) {
-    const hipError_t e =
-        hipFuncSetAttribute((const void*)mxn_tile_dma_kernel,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, DM_STAGES * DM_STAGE);
+    const hipError_t e = hipFuncSetAttribute((const void*)mxn_tile_dma_kernel<XF8>,
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return e;
     if (dev >= 0 && dev < 64) granted[dev] = true;
   }
-  mxn_tile_dma_kernel<<<dim3((unsigned)(tiles_n * tiles_m)), dim3(DM_THREADS),
-                        DM_STAGES * DM_STAGE, s>>>(w.q, w.scales, x.q, x.scales, c, w.N, w.K, w.B,
-                                                   x.N, tiles_n, tiles_m);
+  mxn_tile_dma_kernel<XF8><<<dim3((unsigned)(tiles_n * tiles_m)), dim3(DM_THREADS), lds_bytes, s>>>(
+      w.q, w.scales, (const uint32_t*)xq, xs, c, w.N, w.K, w.B, M, tiles_n, tiles_m);
   return hipGetLastError();
 }
 
@@ -517,14 +562,14 @@ hipError_t launch_tile(const w4_packed_mx_view& w, const w4_packed_mx_view& x, w
 
 hipError_t launch_gemm_mx_w4a4(const w4_packed_mx_view& w, const w4_packed_mx_view& x,
                                w4_half* c, hipStream_t s) {
-  if (tile_applies(w, x)) return launch_tile(w, x, c, s);
+  if (tile_applies(w, x.q, x.scales, x.N, w.K / 2)) return launch_tile<false>(w, x.q, x.scales, x.N, c, s);
   return launch_skinny<false>(w, x.q, x.scales, x.N, c, s);
 }
 
-// E4M3 activations (K a multiple of 32, rows 16-byte aligned): the skinny kernel
-// for every M (grid.y walks the rows of X).
+// E4M3 activations (K a multiple of 32, rows 16-byte aligned).
 hipError_t launch_gemm_mx_w4a8(const w4_packed_mx_view& w, const w4_act_mx8_view& x, w4_half* c,
                                hipStream_t s) {
+  if (tile_applies(w, x.q, x.scales, x.M, w.K)) return launch_tile<true>(w, x.q, x.scales, x.M, c, s);
   return launch_skinny<true>(w, x.q, x.scales, x.M, c, s);
 }
 

@@ -659,16 +659,15 @@ __global__ __launch_bounds__(64 * NW * KW) void mfma_stream_kernel(
   }
 }
 
-// 4 row tiles x 2 K slices (deeper rings and more chunks per step measured slower).
 
-template <int FMT, int MT>
-static hipError_t launch_stream_mt(const WView& v, const w4_half* x, w4_half* c, int M,
+template <int FMT, int MT, int NW, int KW>
+static hipError_t launch_stream_cfg(const WView& v, const w4_half* x, w4_half* c, int M,
                                    hipStream_t s, w4_half* w_out, bool wvec) {
   const bool gs32 = v.mx || v.gs % 32 == 0;
   int gs_shift = -1;
   if (!v.mx && (v.gs & (v.gs - 1)) == 0) gs_shift = __builtin_ctz((unsigned)v.gs);
-  constexpr int NW = 4, KW = 2;  // 16 waves (KW = 4) measured slower
-  // two chunks per step, two steps in flight; MT = 4 fills the LDS with one chunk per step
+  // two chunks per step, two steps in flight (deeper rings measured slower: 15.2 -> 16-17 us
+  // at N = 11008, M = 16); MT = 4 fills the LDS with one chunk per step
   constexpr int CPS = MT == 4 ? 1 : 2;
   constexpr int DEPTH = MT == 4 ? 4 : 2;
   const dim3 grid((unsigned)((v.N + 16 * NW - 1) / (16 * NW)), (unsigned)((M + 16 * MT - 1) / (16 * MT)));
@@ -702,6 +701,17 @@ static hipError_t launch_stream_mt(const WView& v, const w4_half* x, w4_half* c,
   }
 #undef W4_GO
   return hipGetLastError();
+}
+
+// 4 row tiles x 2 K slices per workgroup; 2 x 4 when that grid would leave half of the
+// chip idle (N = 4096, M = 32: 13.1 vs 16.2 us; K = 11008: 29 vs 38 us).  16 waves
+// measured slower.
+template <int FMT, int MT>
+static hipError_t launch_stream_mt(const WView& v, const w4_half* x, w4_half* c, int M,
+                                   hipStream_t s, w4_half* w_out, bool wvec) {
+  const long long wgs = (long long)((v.N + 63) / 64) * ((M + 16 * MT - 1) / (16 * MT));
+  if (MT < 4 && wgs < 128) return launch_stream_cfg<FMT, MT, 2, 4>(v, x, c, M, s, w_out, wvec);
+  return launch_stream_cfg<FMT, MT, 4, 2>(v, x, c, M, s, w_out, wvec);
 }
 
 template <int FMT>

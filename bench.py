@@ -407,7 +407,22 @@ def extras_w4a4(b, full):
                 rows[-1].update({"a8_us": us8, "a8_TFLOPs": 2.0 * M * N * K / us8 * 1e-6})
         del views
         torch.cuda.empty_cache()
-    return {"w4a4_mxfp4": rows}
+    # the activation quantizers that feed it (FP16 -> MXFP4 / MXFP8), K = 4096
+    capi, st = b.capi, b.stream
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    act = []
+    K = 4096
+    for M in (16, 2048):
+        x = torch.randn(M * K, device="cuda").to(torch.float16)
+        q4 = torch.empty(M * K // 8, dtype=torch.int32, device="cuda")
+        q8 = torch.empty(M * K, dtype=torch.uint8, device="cuda")
+        sc = torch.empty(M * K // 32, dtype=torch.uint8, device="cuda")
+        v4 = capi.packed_mx_view(M, K, K // 32, q4.data_ptr(), sc.data_ptr())
+        v8 = capi.act_mx8_view(M, K, K // 32, q8.data_ptr(), sc.data_ptr())
+        ms4 = _median_events_ms(torch, lambda i: capi.quantize_mx_f16(v4, x.data_ptr(), status.data_ptr(), st), 50, 5)
+        ms8 = _median_events_ms(torch, lambda i: capi.quantize_mx8_f16(v8, x.data_ptr(), status.data_ptr(), st), 50, 5)
+        act.append({"M": M, "K": K, "fp4_us": ms4 * 1e3, "fp8_us": ms8 * 1e3})
+    return {"w4a4_mxfp4": rows, "w4a4_activation_quantizers": act}
 
 
 def extras_quantize(b, full):

@@ -279,3 +279,31 @@ def test_w4a8_prefill_shape_sampled_rows():
     ref = orc.dequant_mx8(xq)[rows] @ _decode(wq, N).T
     assert orc.rel_l2(got[rows], ref) <= TOL
     assert np.isfinite(got).all()
+
+
+def test_w4a4_activation_quantizer_ties_and_boundaries():
+    """FP16 activations on the midpoints between E2M1 magnitudes (and one FP16 ulp either
+    side), block maxima on and beside 6 * 2^e, FP16 subnormals, signed zeros: the device
+    quantizer (FP32 arithmetic for FP16 sources) writes the host quantizer's bytes."""
+    c = w4amd.capi()
+    rows = []
+    mids = np.array([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0])
+    for e in range(-24, 13):
+        top = np.float16(6.0 * 2.0 ** e)
+        if not np.isfinite(top) or top == 0:
+            continue
+        for amax in (top, np.nextafter(top, np.float16(np.inf)), np.nextafter(top, np.float16(0))):
+            if not np.isfinite(amax):
+                continue
+            unit = 2.0 ** e if amax <= top else 2.0 ** (e + 1)
+            m = (mids * unit).astype(np.float16)
+            row = np.concatenate([[amax, -amax], m, np.nextafter(m, np.float16(np.inf)),
+                                  np.nextafter(m, np.float16(0)), -m, [np.float16(0), np.float16(-0.0)]])
+            row = row[np.abs(row.astype(np.float64)) <= float(amax)][:32]
+            rows.append(np.concatenate([row, np.zeros(32 - row.size, np.float16)]))
+    x16 = np.array(rows, np.float16)
+    M, K = x16.shape
+    ref = orc.quantize_mx(x16.astype(np.float64), M, K)
+    _, q, s = _quantize_x_on_device(x16.ravel(), M, K)
+    assert np.array_equal(s.cpu().numpy(), ref.scales)
+    assert np.array_equal(q.cpu().numpy().view(np.uint32), ref.q)

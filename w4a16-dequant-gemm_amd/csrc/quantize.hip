@@ -379,13 +379,16 @@ __device__ __forceinline__ int mx_exponent(double amax, bool* out_of_range) {
 }
 
 // mx.hpp:103-108: index of the nearest E2M1 magnitude, the lower one on ties.
-__device__ __forceinline__ int nearest_e2m1(double a) {
-  const double mags[8] = {0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0};
+// (In FP32 for FP16 sources: the scaled value has 11 significant bits, so every
+// difference below is exact and a tie is a tie.)
+template <typename A>
+__device__ __forceinline__ int nearest_e2m1(A a) {
+  const A mags[8] = {(A)0.0, (A)0.5, (A)1.0, (A)1.5, (A)2.0, (A)3.0, (A)4.0, (A)6.0};
   int best = 0;
-  double dbest = a;
+  A dbest = a;
 #pragma unroll
   for (int i = 1; i < 8; ++i) {
-    const double d = fabs(mags[i] - a);
+    const A d = mags[i] > a ? mags[i] - a : a - mags[i];
     if (d < dbest) {
       best = i;
       dbest = d;
@@ -417,35 +420,51 @@ __global__ __launch_bounds__(QT) void quantize_mx_kernel(const T* __restrict__ s
   const int k0 = b * 32 + j4 * 8;
   const int n = live ? (K - k0 < 0 ? 0 : (K - k0 > 8 ? 8 : K - k0)) : 0;
   const T* base = src + row * (long long)K + k0;
-  double v[8];
-  double amax = 0.0;
+  // FP16 sources work in FP32: scaling by a power of two is exact, and so is
+  // everything the encoders do with an 11-bit significand
+  typedef typename Quot<T>::type A;
+  A v[8];
+  A amax = (A)0;
   bool bad = false;
-  if (FULL) {  // K a multiple of 8 and 16-byte aligned rows: four 16-byte loads
+  if constexpr (FULL) {  // K a multiple of 8 and 16-byte aligned rows: four 16-byte loads
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = 0.0;
-    if (n) load8((const double*)base, v);
+    for (int j = 0; j < 8; ++j) v[j] = (A)0;
+    if (n) load8(base, v);
   } else {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = j < n ? (double)base[j] : 0.0;
+    for (int j = 0; j < 8; ++j) v[j] = j < n ? (A)base[j] : (A)0;
   }
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    bad |= !finite(v[j]);
-    amax = fmax(amax, fabs(v[j]));
+    const A av = v[j] < (A)0 ? -v[j] : v[j];
+    bad |= !(av <= (A)(sizeof(T) == 2 ? 65504.0 : DBL_MAX));
+    amax = av > amax ? av : amax;
   }
   if (bad) atomicOr(status, 1);
-  amax = fmax(amax, __shfl_xor(amax, 1));
-  amax = fmax(amax, __shfl_xor(amax, 2));
+  {
+    const A o1 = __shfl_xor(amax, 1);
+    amax = o1 > amax ? o1 : amax;
+    const A o2 = __shfl_xor(amax, 2);
+    amax = o2 > amax ? o2 : amax;
+  }
   bool range = false;
-  const int e = mx_exponent<F8 ? 448 : 6>(amax, &range);
+  const int e = mx_exponent<F8 ? 448 : 6>((double)amax, &range);
   if (range && j4 == 0) atomicOr(status, 2);
   if (n == 0) return;
-  const double scale = ldexp(1.0, e);
+  A u[8];  // v / 2^e
+  if constexpr (sizeof(T) == 2) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) u[j] = ldexpf(v[j], -e);
+  } else {
+    const double scale = ldexp(1.0, e);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) u[j] = v[j] / scale;
+  }
   if (F8) {
     uint8_t* dst = q8 + row * (long long)K + k0;
     uint32_t c[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) c[j] = encode_e4m3((float)(v[j] / scale));
+    for (int j = 0; j < 8; ++j) c[j] = encode_e4m3((float)u[j]);
     if (n == 8 && ((uintptr_t)dst & 7) == 0) {
       u2 out;
       out[0] = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
@@ -461,8 +480,8 @@ __global__ __launch_bounds__(QT) void quantize_mx_kernel(const T* __restrict__ s
 #pragma unroll
     for (int j = 0; j < 8; ++j)
       if (j < n) {
-        const double u = v[j] / scale;
-        const uint32_t code = (__builtin_signbit(u) ? 8u : 0u) | (uint32_t)nearest_e2m1(fabs(u));
+        const uint32_t code = (__builtin_signbit(u[j]) ? 8u : 0u) |
+                              (uint32_t)nearest_e2m1<A>(u[j] < (A)0 ? -u[j] : u[j]);
         word |= code << (4 * j);
       }
     q[row * (long long)words(K) + b * 4 + j4] = word;
@@ -544,7 +563,11 @@ hipError_t launch_quantize_mx(const void* src, int src_f16, long long rows, int 
   const long long blocks = (rows * B * 4 + QT - 1) / QT;
   if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
   const dim3 grid((unsigned)blocks), block(QT);
-  if (src_f16)
+  const bool vec = K % 8 == 0 && ((uintptr_t)src & 15) == 0;
+  if (src_f16 && vec)
+    quantize_mx_kernel<_Float16, true, false><<<grid, block, 0, s>>>((const _Float16*)src, rows, K,
+                                                                    B, q, nullptr, scales, status);
+  else if (src_f16)
     quantize_mx_kernel<_Float16, false, false><<<grid, block, 0, s>>>((const _Float16*)src, rows, K,
                                                                      B, q, nullptr, scales, status);
   else if (K % 8 == 0 && ((uintptr_t)src & 15) == 0)
@@ -562,7 +585,10 @@ hipError_t launch_quantize_mx8(const void* src, int src_f16, long long rows, int
   const long long blocks = (rows * B * 4 + QT - 1) / QT;
   if (blocks > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
   const dim3 grid((unsigned)blocks), block(QT);
-  if (src_f16)
+  if (src_f16 && K % 8 == 0 && ((uintptr_t)src & 15) == 0)
+    quantize_mx_kernel<_Float16, true, true><<<grid, block, 0, s>>>((const _Float16*)src, rows, K,
+                                                                   B, nullptr, q, scales, status);
+  else if (src_f16)
     quantize_mx_kernel<_Float16, false, true><<<grid, block, 0, s>>>((const _Float16*)src, rows, K,
                                                                     B, nullptr, q, scales, status);
   else

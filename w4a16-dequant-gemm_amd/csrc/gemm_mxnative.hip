@@ -1,5 +1,7 @@
-// W4A4: c[M,N] = X[M,K] * W[N,K]^T with BOTH operands in packed MXFP4, on the
-// gfx950 scaled matrix cores (v_mfma_scale_f32_16x16x128_f8f6f4).
+// W4A4 / W4A8: c[M,N] = X[M,K] * W[N,K]^T with packed MXFP4 weights against
+// activations that are block-scaled too -- packed MXFP4, or E4M3 bytes under the
+// same E8M0 block scales -- on the gfx950 scaled matrix cores
+// (v_mfma_scale_f32_{16x16x128,32x32x64}_f8f6f4).
 //
 // No counterpart in the reference, whose MXFP4 kernels expand the weights to
 // FP16 and keep FP16 activations (mxfused.cuh:166-198, 291-307).  Here nothing

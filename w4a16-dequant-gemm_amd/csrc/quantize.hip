@@ -388,7 +388,7 @@ __device__ __forceinline__ int nearest_e2m1(A a) {
   A dbest = a;
 #pragma unroll
   for (int i = 1; i < 8; ++i) {
-    const A d = mags[i] > a ? mags[i] - a : a - mags[i];
+    const A d = __builtin_elementwise_abs(mags[i] - a);
     if (d < dbest) {
       best = i;
       dbest = d;
@@ -456,9 +456,11 @@ __global__ __launch_bounds__(QT) void quantize_mx_kernel(const T* __restrict__ s
 #pragma unroll
     for (int j = 0; j < 8; ++j) u[j] = ldexpf(v[j], -e);
   } else {
-    const double scale = ldexp(1.0, e);
+    // |e| <= 127, so 2^-e is a normal double and v * 2^-e is the same real number
+    // as v / 2^e, rounded the same way: the host's quotient without the division
+    const double inv = ldexp(1.0, -e);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) u[j] = v[j] / scale;
+    for (int j = 0; j < 8; ++j) u[j] = v[j] * inv;
   }
   if (F8) {
     uint8_t* dst = q8 + row * (long long)K + k0;

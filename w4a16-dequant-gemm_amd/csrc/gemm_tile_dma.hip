@@ -1,0 +1,348 @@
+// Large-M W4A16 GEMM whose operands reach LDS without passing through registers:
+// c[M,N] = X[M,K] * dequant(W)[N,K]^T for W4 weights with FP16 group scales and
+// optional 4-bit zero-points (mma.cuh:63-230 is the reference's tensor-core kernel:
+// it expands each chunk of W to FP16 in shared memory once per block).
+//
+// Here the packed words themselves are what sits in LDS -- a quarter of the bytes
+// of the expanded tile -- and every wave expands the words of its own MFMA
+// operands in registers, straight into the operand layout:
+//   * global_load_lds_dwordx4 moves both operand tiles global -> LDS (no staging
+//     registers, no ds_write); a stage is 128 k: 64 bytes of a W row, 256 bytes of
+//     an X row; three stages of 50 KB; one barrier per stage.
+//   * v_mfma_f32_32x32x16_f16: lane l brings row l%32 and eight consecutive k.
+//     Which eight is free as long as both operands agree, so of a 64-k half lane
+//     half h = l/32 takes k 32h + 8j .. + 7 in MFMA j: its four W words are one
+//     16-byte LDS read, its X operand is 16-byte piece 4h + j of the row's half.
+//   * a word becomes four packed-half registers in natural k order with
+//     v_perm_b32 (byte i to bytes 0 and 2), one mask-and-or that plants the low
+//     nibble in the significand of 1024.0 and the high nibble in that of 64.0
+//     (whose unit in the last place is 1/16), one packed add of -(1024 + z),
+//     -(64 + z) and one packed multiply by the scale: q - z is exact and the
+//     product is rounded once, so the operand is bit for bit the FP16 weight the
+//     one dequant step returns (pack.hpp:58-60).
+// The accumulation is FP32 in the instruction; the output is rounded to FP16 once.
+#include "dq.cuh"
+#include "kernels.h"
+
+namespace w4k {
+namespace {
+
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void* lds_ptr;
+
+constexpr int TD_TN = 256, TD_TM = 128;  // rows of W x rows of X per workgroup
+constexpr int TD_WAVES = 4, TD_THREADS = 64 * TD_WAVES;  // a wave: 64 rows of W x all 128 of X
+constexpr int TD_STAGES = 3;
+constexpr int TD_W_BYTES = TD_TN * 64, TD_X_BYTES = TD_TM * 256;
+constexpr int TD_TILE = TD_W_BYTES + TD_X_BYTES;   // 48 KB
+constexpr int TD_STAGE = TD_TILE + 2 * TD_TN * 4;  // + a scale and a zero-point dword per W row
+constexpr int TD_WI = TD_W_BYTES / 1024 / TD_WAVES;  // 1 KB load instructions of W per wave: 4
+constexpr int TD_XI = TD_X_BYTES / 1024 / TD_WAVES;  // of X: 8
+constexpr int TD_LDS = TD_STAGES * TD_STAGE;
+
+// s_waitcnt vmcnt(N) alone (gfx9 encoding: vmcnt in [3:0] and [15:14])
+constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
+
+extern __shared__ __attribute__((aligned(16))) uint8_t td_lds[];
+
+// Position of 16-byte piece p of row R.  A load instruction writes lane l's 16
+// bytes at 16 l, so the rows of one instruction are contiguous (16 rows of W, 4 of
+// X) and the piece a lane fetches is chosen so that the rows one ds_read_b128
+// touches (8 or 16 consecutive ones, same p) fall on distinct 16-byte bank groups.
+__device__ __forceinline__ int w_key(int R) { return ((R >> 1) ^ (R >> 3)) & 3; }
+__device__ __forceinline__ int w_at(int R, int p) {
+  return (R >> 4) * 1024 + ((R & 15) * 4 + (p ^ w_key(R))) * 16;
+}
+__device__ __forceinline__ int x_at(int R, int p) {
+  return (R >> 2) * 1024 + ((R & 3) * 16 + (p ^ (R & 15))) * 16;
+}
+
+// Eight codes of a packed word -> eight FP16 weights in k order (as an MFMA operand).
+// cneg: packed {-(1024 + z), -(64 + z)}; s2: the group scale in both halves.
+// mask, magic: 0x00F0000F and 0x54006400 held in registers (the three-operand
+// and-or takes no literal).
+__device__ __forceinline__ h8 expand_word(uint32_t w, h2 cneg, h2 s2, uint32_t mask, uint32_t magic) {
+  u4 out;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t p = __builtin_amdgcn_perm(0u, w, 0x0c000c00u | (uint32_t)(i << 16) | (uint32_t)i);
+    const uint32_t v = (p & mask) | magic;
+    out[i] = as_u32((as_h2(v) + cneg) * s2);
+  }
+  return __builtin_bit_cast(h8, out);
+}
+
+// One wave per SIMD, so the three pipes have to overlap inside a wave: a stage is
+// eight steps of 16 k (8 MFMAs each); during the MFMAs of step u the wave reads the
+// X operands of step u + 1 from LDS and expands its W words, in program order
+// between the MFMAs.
+//
+// HOOK: the workgroups of the first m tile also write the expanded weights to
+// w_out (mma.cuh:147-159: the reference's dequant hook), from the operand
+// registers the MFMAs consume.
+template <bool ASYM, bool HOOK>
+__global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
+    const uint32_t* __restrict__ wq, const uint16_t* __restrict__ scales,
+    const uint32_t* __restrict__ zeros, const w4_half* __restrict__ x, w4_half* __restrict__ c,
+    w4_half* __restrict__ w_out, int N, int K, int G, int gs, int M, int tiles_n, int tiles_m) {
+  constexpr int LOADS = TD_WI + TD_XI + (ASYM ? 2 : 1);  // load instructions per wave and stage
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // in an SGPR: LDS addresses go to M0
+  const int r = lane & 31, h = lane >> 5;
+  // Consecutive workgroup ids land on different XCDs (each with its own L2): give
+  // each XCD a contiguous run of the tile order, m fastest, so that its
+  // workgroups share a few W tiles and walk X.
+  int L = blockIdx.x;
+  const int total = tiles_n * tiles_m;
+  if (total % 8 == 0) L = (L & 7) * (total >> 3) + (L >> 3);
+  const int n0 = (L / tiles_m) * TD_TN, m0 = (L % tiles_m) * TD_TM;
+  const int wg = words(G);
+
+  // What this lane fetches (byte offsets; 32 bits: the launcher bounds the operands).
+  // Rows past N or M are clamped to the last one; their results are never stored.
+  uint32_t wo[TD_WI], xo[TD_XI];
+#pragma unroll
+  for (int i = 0; i < TD_WI; ++i) {
+    const int R = (wave + TD_WAVES * i) * 16 + (lane >> 2), n = n0 + R;
+    wo[i] = (uint32_t)(n < N ? n : N - 1) * (uint32_t)(K >> 1) + (((lane & 3) ^ w_key(R)) * 16);
+  }
+#pragma unroll
+  for (int i = 0; i < TD_XI; ++i) {
+    const int R = (wave + TD_WAVES * i) * 4 + (lane >> 4), m = m0 + R;
+    xo[i] = (uint32_t)(m < M ? m : M - 1) * (uint32_t)(K * 2) + (((lane & 15) ^ (R & 15)) * 16);
+  }
+  // per stage: the dword that holds the group scale of W row 64 wave + lane, and
+  // (ASYM) that row's zero-point word
+  const uint32_t sn = (uint32_t)(n0 + wave * 64 + lane < N ? n0 + wave * 64 + lane : N - 1);
+  const uint32_t sc_base = sn * (uint32_t)G, zw_base = sn * (uint32_t)wg;
+  const char* wqb = (const char*)wq;
+  const char* xb = (const char*)x;
+
+  const int stages = K >> 7;
+  // The loads are asm so that the compiler neither tracks them (it would wait for
+  // all of them before any LDS read) nor moves LDS reads across them; the vmcnt
+  // waits below are by hand.  M0 carries the wave-uniform LDS address.
+  auto dma16 = [](const void* gbase, uint32_t goff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(goff), "s"(gbase), "s"(lds_addr)
+                 : "memory", "m0");
+  };
+  auto dma4 = [](const void* gbase, uint32_t goff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1"
+                 :
+                 : "v"(goff), "s"(gbase), "s"(lds_addr)
+                 : "memory", "m0");
+  };
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr)td_lds;
+  // Load instruction `part` (0 .. LOADS - 1) of stage d: a wave issues them two at
+  // a time between the MFMAs of successive steps -- thirteen in a row would hold up
+  // its one instruction stream for as long as four steps take.
+  auto request_part = [&](int d, int part) {
+    const uint32_t dd = (uint32_t)(d < stages ? d : stages - 1);  // past the end: valid, never used
+    const uint32_t st = lds0 + (uint32_t)(d % TD_STAGES) * TD_STAGE;
+    if (part < TD_WI) {
+      dma16(wqb, wo[part] + dd * 64u, st + (wave + TD_WAVES * part) * 1024);
+    } else if (part < TD_WI + TD_XI) {
+      const int i = part - TD_WI;
+      dma16(xb, xo[i] + dd * 256u, st + TD_W_BYTES + (wave + TD_WAVES * i) * 1024);
+    } else {
+      const uint32_t g = (dd * 128u) / (uint32_t)gs;
+      if (part == TD_WI + TD_XI) dma4(scales, ((sc_base + g) >> 1) * 4u, st + TD_TILE + wave * 256);
+      else dma4(zeros, (zw_base + (g >> 3)) * 4u, st + TD_TILE + TD_TN * 4 + wave * 256);
+    }
+  };
+  auto request = [&](int d) {
+#pragma unroll
+    for (int part = 0; part < LOADS; ++part) request_part(d, part);
+  };
+
+  // this lane's rows of the two W tiles of its wave; the parity of their first
+  // scale index says which half of the fetched dword is theirs
+  int wrow[2];
+  uint32_t par[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    wrow[i] = wave * 64 + i * 32 + r;
+    const int n = n0 + wrow[i];
+    par[i] = ((uint32_t)(n < N ? n : N - 1) * (uint32_t)G) & 1u;
+  }
+  const bool hook = HOOK && m0 == 0;
+  uint32_t mask = 0x00F0000Fu, magic = 0x54006400u;
+  asm volatile("" : "+s"(mask));   // opaque: otherwise they come back as literals of two
+  asm volatile("" : "+v"(magic));  // separate instructions
+
+  u4 xv[2][4];            // X operands of the step in hand and of the next: [m tile]
+  u4 wv[2][2];            // packed words of the two 64-k halves: [half][n tile], word = step % 4
+  h8 av[2][2];            // expanded W operands of the step in hand and of the next
+  uint32_t sc[2], zw[2];  // the stage's scale dword and zero-point word per n tile
+  h2 cneg[2], s2v[2];
+  auto read_x = [&](u4* dst, const uint8_t* base, int u) {  // step u = half u/4, MFMA u%4
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      dst[j] = *(const u4*)(base + TD_W_BYTES + x_at(j * 32 + r, 8 * (u >> 2) + 4 * h + (u & 3)));
+  };
+  auto read_w = [&](u4* dst, const uint8_t* base, int s2) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) dst[i] = *(const u4*)(base + w_at(wrow[i], 2 * s2 + h));
+  };
+  auto read_sc = [&](const uint8_t* base) {
+    const uint32_t* p = (const uint32_t*)(base + TD_TILE);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      sc[i] = p[wrow[i]];
+      if (ASYM) zw[i] = p[TD_TN + wrow[i]];
+    }
+  };
+  auto set_group = [&](int d) {
+    const uint32_t g = ((uint32_t)d * 128u) / (uint32_t)gs;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const uint32_t s16 = ((par[i] + g) & 1u) ? (sc[i] >> 16) : (sc[i] & 0xFFFFu);
+      s2v[i] = splat_bits(s16);
+      const uint32_t z = ASYM ? ((zw[i] >> (4 * (g & 7))) & 0xFu) : 8u;
+      cneg[i] = as_h2(0xD400E400u | (z << 20) | z);
+    }
+  };
+  auto expand = [&](h8* dst, int d, int u) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      dst[i] = expand_word(wv[u >> 2][i][u & 3], cneg[i], s2v[i], mask, magic);
+      if (HOOK && hook && d < stages && n0 + wrow[i] < N)
+        *(h8*)(w_out + (size_t)(n0 + wrow[i]) * K + d * 128 + (u >> 2) * 64 + h * 32 + (u & 3) * 8) =
+            dst[i];
+    }
+  };
+
+  f16v acc[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // Stage d + 2 is requested in pieces from step 7 of stage d - 1 (when the barrier
+  // there has freed its buffer) to step 6 of stage d.
+  request(0);
+  request(1);
+  request_part(2, 0);
+  request_part(2, 1);
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm(LOADS + 2));  // stage 0 has landed
+  __syncthreads();
+  read_x(xv[0], td_lds, 0);
+  read_w(wv[0], td_lds, 0);
+  read_sc(td_lds);
+  set_group(0);
+  expand(av[0], 0, 0);
+#pragma unroll 1
+  for (int d = 0; d < stages; ++d) {
+    const uint8_t* base = td_lds + (d % TD_STAGES) * TD_STAGE;
+    const uint8_t* next = td_lds + ((d + 1) % TD_STAGES) * TD_STAGE;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (u == 7) {
+        // every LDS read of stage d has been issued (the X operands of step 7 during
+        // step 6): once all waves are here its buffer can take stage d + 3, and stage
+        // d + 1 has landed for everyone (outstanding: all of stage d + 2)
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(LOADS));
+        __syncthreads();
+        request_part(d + 3, 0);
+        request_part(d + 3, 1);
+        read_x(xv[0], next, 0);
+        read_w(wv[0], next, 0);
+        read_sc(next);
+        set_group(d + 1);
+        expand(av[0], d + 1, 0);
+      } else {
+        if (2 * u + 2 < LOADS) request_part(d + 2, 2 * u + 2);
+        if (2 * u + 3 < LOADS) request_part(d + 2, 2 * u + 3);
+        read_x(xv[(u + 1) & 1], base, u + 1);
+        if (u == 0) read_w(wv[1], base, 1);
+        expand(av[(u + 1) & 1], d, u + 1);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+              av[u & 1][i], __builtin_bit_cast(h8, xv[u & 1][j]), acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // nothing may still be writing LDS at exit
+
+  // lane: m = tile row r, n = 8 q + 4 h + e of each 32 x 32 tile
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int m = m0 + j * 32 + r;
+    if (m >= M) continue;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int nn = n0 + wave * 64 + i * 32 + 8 * q + 4 * h;
+        w4_half* dst = c + (size_t)m * N + nn;
+        if (nn + 3 < N && ((uintptr_t)dst & 7) == 0) {
+          h4 out;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) out[e] = (_Float16)acc[i][j][4 * q + e];
+          *(h4*)dst = out;
+        } else {
+          const int left = N - nn;
+          if (left > 0) dst[0] = __builtin_bit_cast(uint16_t, (_Float16)acc[i][j][4 * q + 0]);
+          if (left > 1) dst[1] = __builtin_bit_cast(uint16_t, (_Float16)acc[i][j][4 * q + 1]);
+          if (left > 2) dst[2] = __builtin_bit_cast(uint16_t, (_Float16)acc[i][j][4 * q + 2]);
+          if (left > 3) dst[3] = __builtin_bit_cast(uint16_t, (_Float16)acc[i][j][4 * q + 3]);
+        }
+      }
+  }
+}
+
+template <bool ASYM, bool HOOK>
+hipError_t launch(const WView& v, const w4_half* x, w4_half* c, w4_half* w_out, int M,
+                  hipStream_t s, int tiles_n, int tiles_m) {
+  // more than 64 KB of LDS has to be granted per device, once
+  static bool granted[64] = {};
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+  if (dev < 0 || dev >= 64 || !granted[dev]) {
+    const hipError_t e = hipFuncSetAttribute((const void*)w4_tile_dma_kernel<ASYM, HOOK>,
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, TD_LDS);
+    if (e != hipSuccess) return e;
+    if (dev >= 0 && dev < 64) granted[dev] = true;
+  }
+  w4_tile_dma_kernel<ASYM, HOOK>
+      <<<dim3((unsigned)(tiles_n * tiles_m)), dim3(TD_THREADS), TD_LDS, s>>>(
+          v.q, (const uint16_t*)v.scales, v.zeros, x, c, w_out, v.N, v.K, v.G, v.gs, M, tiles_n,
+          tiles_m);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+// Takes W4 weights whose groups hold whole stages (gs a multiple of 128, hence K
+// too), operands under 4 GiB (32-bit offsets), 16-byte aligned rows, an even
+// number of scales (they are fetched as dwords) and a tile grid that covers a
+// good part of the chip.  Returns false, launching nothing, otherwise.
+bool try_tile_dma(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
+                  w4_half* w_out, hipError_t* err) {
+  if (v.mx || v.gs % 128 || v.K % 128 || v.K < 128) return false;
+  const long long tiles_n = (v.N + TD_TN - 1) / TD_TN, tiles_m = (M + TD_TM - 1) / TD_TM;
+  if (M < 128 || tiles_n * tiles_m < 64 || tiles_n * tiles_m > 0x7FFFFFFFLL) return false;
+  if ((long long)v.N * v.K / 2 >= (1LL << 32) || (long long)M * v.K * 2 >= (1LL << 32)) return false;
+  if (((long long)v.N * v.G) & 1) return false;
+  if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)v.scales & 3)) return false;
+  if (!v.symmetric && (v.zeros == nullptr || ((uintptr_t)v.zeros & 3))) return false;
+  if (w_out && ((uintptr_t)w_out & 15)) return false;
+  const int tn = (int)tiles_n, tm = (int)tiles_m;
+  if (w_out)
+    *err = v.symmetric ? launch<false, true>(v, x, c, w_out, M, s, tn, tm)
+                       : launch<true, true>(v, x, c, w_out, M, s, tn, tm);
+  else
+    *err = v.symmetric ? launch<false, false>(v, x, c, nullptr, M, s, tn, tm)
+                       : launch<true, false>(v, x, c, nullptr, M, s, tn, tm);
+  return true;
+}
+
+}  // namespace w4k

@@ -39,6 +39,11 @@ hipError_t launch_gemm_simt(const WView& v, const w4_half* x, w4_half* c, int M,
 hipError_t launch_gemm_mfma(const WView& v, const w4_half* x, w4_half* c, int M,
                             hipStream_t s, w4_half* w_out);
 
+// gemm_tile_dma.hip: large-M W4 kernel with direct-to-LDS operand loads; false
+// (nothing launched) when the arguments are not its shape.
+bool try_tile_dma(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
+                  w4_half* w_out, hipError_t* err);
+
 // flash.hip -- one description for the four cache kinds
 struct FlashArgs {
   int kind;  // 0 FP16, 1 W4, 2 FP8

@@ -141,11 +141,11 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   auto request_part = [&](int d, int part) {
     const uint32_t dd = (uint32_t)(d < stages ? d : stages - 1);  // past the end: valid, never used
     const uint32_t st = lds0 + (uint32_t)(d % TD_STAGES) * TD_STAGE;
-    if (part < TD_WI) {
-      dma16(wqb, wo[part] + dd * 64u, st + (wave + TD_WAVES * part) * 1024);
+    if (part < TD_WI) {  // the stage's offset goes into the scalar base: no vector arithmetic
+      dma16(wqb + dd * 64u, wo[part], st + (wave + TD_WAVES * part) * 1024);
     } else if (part < TD_WI + TD_XI) {
       const int i = part - TD_WI;
-      dma16(xb, xo[i] + dd * 256u, st + TD_W_BYTES + (wave + TD_WAVES * i) * 1024);
+      dma16(xb + dd * 256u, xo[i], st + TD_W_BYTES + (wave + TD_WAVES * i) * 1024);
     } else {
       const uint32_t g = (dd * 128u) / (uint32_t)gs;
       if (part == TD_WI + TD_XI) dma4(scales, ((sc_base + g) >> 1) * 4u, st + TD_TILE + wave * 256);
@@ -267,12 +267,51 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
         for (int j = 0; j < 4; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
               av[u & 1][i], __builtin_bit_cast(h8, xv[u & 1][j]), acc[i][j], 0, 0, 0);
+      if (u < 7) {
+        // LDS reads first, then the expansion spread evenly under the MFMAs: a wave
+        // can issue about six vector instructions in the shadow of one MFMA
+        if (u == 0) __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
+        else __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
   }
   __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // nothing may still be writing LDS at exit
 
-  // lane: m = tile row r, n = 8 q + 4 h + e of each 32 x 32 tile
+  // A lane holds, of each 32 x 32 tile, n = 8 q + 4 h + e for m = tile row r.  Whole
+  // tiles go through LDS (free by now) so that every store instruction writes eight
+  // whole 128-byte lines instead of 16 bytes of each of 32: a wave lays its 128 (m)
+  // x 64 (n) block out in rows of 144 bytes and reads it back 16 bytes a lane.
+  const bool whole = m0 + TD_TM <= M && n0 + TD_TN <= N && (N & 7) == 0 && ((uintptr_t)c & 15) == 0;
+  if (whole) {
+    constexpr int PITCH = 144;
+    __syncthreads();  // no wave reads a stage buffer any more, no load is landing in one
+    uint8_t* mine = td_lds + wave * (TD_TM * PITCH);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          h4 out;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) out[e] = (_Float16)acc[i][j][4 * q + e];
+          *(h4*)(mine + (j * 32 + r) * PITCH + i * 64 + q * 16 + h * 8) = out;
+        }
+    w4_half* cw = c + (size_t)m0 * N + n0 + wave * 64;
+#pragma unroll
+    for (int it = 0; it < TD_TM / 8; ++it) {
+      const int row = it * 8 + (lane >> 3), piece = lane & 7;
+      const u4 v = *(const u4*)(mine + row * PITCH + piece * 16);
+      *(u4*)(cw + (size_t)row * N + piece * 8) = v;
+    }
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int m = m0 + j * 32 + r;

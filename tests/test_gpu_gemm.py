@@ -37,10 +37,12 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         (1, 64, 11008, 128), (1, 32, 2080, 32), (1, 16, 14336, 64), (1, 24, 5120, 48), (1, 8, 16384, 8),
         (2, 16, 11008, 128), (4, 8, 5120, 32), (3, 24, 14336, 64), (4, 16, 8192, 128),
         # the large-M kernel with direct-to-LDS loads (gs % 128 == 0, at least 64 tiles of 128 x 256):
-        # ragged tiles, 3 / 4 / 10 / 2 stages, groups of two stages; then an odd number of scales,
+        # ragged tiles, 4 / 3 / 10 / 2 stages, groups of two stages; then an odd number of scales,
         # which it leaves to the register-staged kernel
         (1030, 2050, 512, 128), (2048, 1024, 384, 128), (1024, 2048, 1280, 256), (1000, 2304, 256, 128),
-        (1025, 2049, 384, 128)]
+        (1025, 2049, 384, 128),
+        # the same kernel with two and four groups per 128-k stage
+        (1030, 2050, 512, 64), (1024, 2048, 384, 32), (2048, 1030, 256, 32), (900, 2304, 640, 64)]
 TOL, CROSS = 1e-3, 2e-3  # rel L2 vs the FP64 oracle; between two gated paths
 
 

@@ -980,7 +980,7 @@ template <int MX>
 static hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M,
                              hipStream_t s, w4_half* w_out) {
   hipError_t terr = hipSuccess;
-  if (!MX && try_tile_dma(v, x, c, M, s, w_out, &terr)) return terr;
+  if (try_tile_dma(v, x, c, M, s, w_out, &terr)) return terr;
   if (try_tile<MX>(v, x, c, M, s, w_out, &terr)) return terr;
   // Rows of packed words are 16-byte aligned when K % 32 == 0 (one dwordx4 per lane
   // slice); K % 8 == 0 still gives whole words and 16-byte aligned activation rows.

@@ -35,7 +35,7 @@ constexpr int TD_WAVES = 4, TD_THREADS = 64 * TD_WAVES;  // a wave: 64 rows of W
 constexpr int TD_STAGES = 3;
 constexpr int TD_W_BYTES = TD_TN * 64, TD_X_BYTES = TD_TM * 256;
 constexpr int TD_TILE = TD_W_BYTES + TD_X_BYTES;   // 48 KB
-constexpr int TD_STAGE = TD_TILE + 2 * TD_TN * 4;  // + a scale and a zero-point dword per W row
+constexpr int TD_STAGE = TD_TILE + 3 * TD_TN * 4;  // + two scale dwords and a zero-point word per W row
 constexpr int TD_WI = TD_W_BYTES / 1024 / TD_WAVES;  // 1 KB load instructions of W per wave: 4
 constexpr int TD_XI = TD_X_BYTES / 1024 / TD_WAVES;  // of X: 8
 constexpr int TD_LDS = TD_STAGES * TD_STAGE;
@@ -80,12 +80,19 @@ __device__ __forceinline__ h8 expand_word(uint32_t w, h2 cneg, h2 s2, uint32_t m
 // HOOK: the workgroups of the first m tile also write the expanded weights to
 // w_out (mma.cuh:147-159: the reference's dequant hook), from the operand
 // registers the MFMAs consume.
-template <bool ASYM, bool HOOK>
+//
+// FMT: 0 W4 symmetric, 1 W4 with zero-points, 2 MXFP4.  GSM says how the groups
+// lie in a 128-k stage: 0 one group (gs a multiple of 128), 1 two (gs = 64), 2 four
+// (gs = 32, and the 32-blocks of MXFP4).  A lane's share of a 64-k half is 32
+// consecutive k, so even then it has one scale per half.  G: scales per row.
+template <int FMT, int GSM, bool HOOK>
 __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
-    const uint32_t* __restrict__ wq, const uint16_t* __restrict__ scales,
+    const uint32_t* __restrict__ wq, const void* __restrict__ scales,
     const uint32_t* __restrict__ zeros, const w4_half* __restrict__ x, w4_half* __restrict__ c,
     w4_half* __restrict__ w_out, int N, int K, int G, int gs, int M, int tiles_n, int tiles_m) {
-  constexpr int LOADS = TD_WI + TD_XI + (ASYM ? 2 : 1);  // load instructions per wave and stage
+  constexpr bool ASYM = FMT == 1, MX = FMT == 2;
+  constexpr int NSC = (!MX && GSM == 2) ? 2 : 1;           // scale dwords per row and stage
+  constexpr int LOADS = TD_WI + TD_XI + NSC + (ASYM ? 1 : 0);  // load instructions per wave and stage
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // in an SGPR: LDS addresses go to M0
   const int r = lane & 31, h = lane >> 5;
@@ -138,23 +145,32 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   // Load instruction `part` (0 .. LOADS - 1) of stage d: a wave issues them two at
   // a time between the MFMAs of successive steps -- thirteen in a row would hold up
   // its one instruction stream for as long as four steps take.
-  auto request_part = [&](int d, int part) {
+  auto request_part = [&](int d, uint32_t buf, int part) {  // buf: byte offset of the stage's buffer
     const uint32_t dd = (uint32_t)(d < stages ? d : stages - 1);  // past the end: valid, never used
-    const uint32_t st = lds0 + (uint32_t)(d % TD_STAGES) * TD_STAGE;
+    const uint32_t st = lds0 + buf;
     if (part < TD_WI) {  // the stage's offset goes into the scalar base: no vector arithmetic
       dma16(wqb + dd * 64u, wo[part], st + (wave + TD_WAVES * part) * 1024);
     } else if (part < TD_WI + TD_XI) {
       const int i = part - TD_WI;
       dma16(xb + dd * 256u, xo[i], st + TD_W_BYTES + (wave + TD_WAVES * i) * 1024);
     } else {
-      const uint32_t g = (dd * 128u) / (uint32_t)gs;
-      if (part == TD_WI + TD_XI) dma4(scales, ((sc_base + g) >> 1) * 4u, st + TD_TILE + wave * 256);
-      else dma4(zeros, (zw_base + (g >> 3)) * 4u, st + TD_TILE + TD_TN * 4 + wave * 256);
+      // the stage's scales of this wave's row 64 wave + lane: the dword with the one
+      // FP16 scale (GSM 0), the dword of its two (GSM 1), the two dwords of its four
+      // (GSM 2), the four E8M0 bytes (MXFP4); then the zero-point word
+      const int k = part - TD_WI - TD_XI;
+      const uint32_t g = MX ? dd * 4u : GSM == 0 ? (dd * 128u) / (uint32_t)gs : dd * (2u * GSM);
+      if (k < NSC) {
+        const uint32_t off = MX ? sc_base + g : GSM == 0 ? ((sc_base + g) >> 1) * 4u
+                                                        : (sc_base + g) * 2u + 4u * k;
+        dma4(scales, off, st + TD_TILE + k * (TD_TN * 4) + wave * 256);
+      } else {
+        dma4(zeros, (zw_base + (g >> 3)) * 4u, st + TD_TILE + 2 * (TD_TN * 4) + wave * 256);
+      }
     }
   };
-  auto request = [&](int d) {
+  auto request = [&](int d, uint32_t buf) {
 #pragma unroll
-    for (int part = 0; part < LOADS; ++part) request_part(d, part);
+    for (int part = 0; part < LOADS; ++part) request_part(d, buf, part);
   };
 
   // this lane's rows of the two W tiles of its wave; the parity of their first
@@ -175,39 +191,75 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   u4 xv[2][4];            // X operands of the step in hand and of the next: [m tile]
   u4 wv[2][2];            // packed words of the two 64-k halves: [half][n tile], word = step % 4
   h8 av[2][2];            // expanded W operands of the step in hand and of the next
-  uint32_t sc[2], zw[2];  // the stage's scale dword and zero-point word per n tile
-  h2 cneg[2], s2v[2];
-  auto read_x = [&](u4* dst, const uint8_t* base, int u) {  // step u = half u/4, MFMA u%4
+  uint32_t sc[2][NSC], zw[2];  // the stage's scale dwords and zero-point word per n tile
+  // what expansion needs, per [half][n tile]: -(1024 + z), -(64 + z) and the scale in
+  // both halves of a register (MXFP4: the scale as a float)
+  h2 cneg[2][2], s2v[2][2];
+  float sf[2][2];
+  // Where this lane reads inside a stage buffer, worked out once: the X piece of
+  // step u in m tile 0 (tile j is 8 KB further), its four words of half s2 in n tile
+  // 0 (tile 1 is 2 KB further), its scale dword.  A read is then one add of the
+  // buffer's offset and an immediate.
+  uint32_t xoff[8], woff[2];
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      dst[j] = *(const u4*)(base + TD_W_BYTES + x_at(j * 32 + r, 8 * (u >> 2) + 4 * h + (u & 3)));
-  };
-  auto read_w = [&](u4* dst, const uint8_t* base, int s2) {
+  for (int u = 0; u < 8; ++u) xoff[u] = TD_W_BYTES + x_at(r, 8 * (u >> 2) + 4 * h + (u & 3));
 #pragma unroll
-    for (int i = 0; i < 2; ++i) dst[i] = *(const u4*)(base + w_at(wrow[i], 2 * s2 + h));
+  for (int s2 = 0; s2 < 2; ++s2) woff[s2] = w_at(wrow[0], 2 * s2 + h);
+  const uint32_t scoff = TD_TILE + wrow[0] * 4;
+  auto read_x = [&](u4* dst, uint32_t buf, int u) {  // step u = half u/4, MFMA u%4
+    const uint8_t* p = td_lds + (buf + xoff[u]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dst[j] = *(const u4*)(p + j * 8192);
   };
-  auto read_sc = [&](const uint8_t* base) {
-    const uint32_t* p = (const uint32_t*)(base + TD_TILE);
+  auto read_w = [&](u4* dst, uint32_t buf, int s2) {
+    const uint8_t* p = td_lds + (buf + woff[s2]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) dst[i] = *(const u4*)(p + i * 2048);
+  };
+  auto read_sc = [&](uint32_t buf) {
+    const uint8_t* p = td_lds + (buf + scoff);
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      sc[i] = p[wrow[i]];
-      if (ASYM) zw[i] = p[TD_TN + wrow[i]];
+#pragma unroll
+      for (int k = 0; k < NSC; ++k) sc[i][k] = *(const uint32_t*)(p + k * (TD_TN * 4) + i * 128);
+      if (ASYM) zw[i] = *(const uint32_t*)(p + 2 * (TD_TN * 4) + i * 128);
     }
   };
   auto set_group = [&](int d) {
-    const uint32_t g = ((uint32_t)d * 128u) / (uint32_t)gs;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const uint32_t s16 = ((par[i] + g) & 1u) ? (sc[i] >> 16) : (sc[i] & 0xFFFFu);
-      s2v[i] = splat_bits(s16);
-      const uint32_t z = ASYM ? ((zw[i] >> (4 * (g & 7))) & 0xFu) : 8u;
-      cneg[i] = as_h2(0xD400E400u | (z << 20) | z);
-    }
+    for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        if constexpr (MX) {  // block 4 d + 2 s2 + h of the row
+          sf[s2][i] = mx_scale((sc[i][0] >> (8 * (2 * s2 + h))) & 0xFFu);
+        } else {
+          uint32_t g, s16;
+          if constexpr (GSM == 0) {
+            g = ((uint32_t)d * 128u) / (uint32_t)gs;
+            s16 = ((par[i] + g) & 1u) ? (sc[i][0] >> 16) : (sc[i][0] & 0xFFFFu);
+          } else if constexpr (GSM == 1) {
+            g = 2u * d + s2;
+            s16 = s2 ? (sc[i][0] >> 16) : (sc[i][0] & 0xFFFFu);
+          } else {
+            g = 4u * d + 2 * s2 + h;
+            s16 = h ? (sc[i][s2] >> 16) : (sc[i][s2] & 0xFFFFu);
+          }
+          s2v[s2][i] = splat_bits(s16);
+          const uint32_t z = ASYM ? ((zw[i] >> (4 * (g & 7))) & 0xFu) : 8u;
+          cneg[s2][i] = as_h2(0xD400E400u | (z << 20) | z);
+        }
+      }
   };
   auto expand = [&](h8* dst, int d, int u) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
-      dst[i] = expand_word(wv[u >> 2][i][u & 3], cneg[i], s2v[i], mask, magic);
+      if constexpr (MX) {
+        h2 n4[4];
+        dq_mx(wv[u >> 2][i][u & 3], sf[u >> 2][i], n4);
+        dst[i] = __builtin_bit_cast(h8, u4{as_u32(n4[0]), as_u32(n4[1]), as_u32(n4[2]), as_u32(n4[3])});
+      } else {
+        dst[i] = expand_word(wv[u >> 2][i][u & 3], cneg[u >> 2][i], s2v[u >> 2][i], mask, magic);
+      }
       if (HOOK && hook && d < stages && n0 + wrow[i] < N)
         *(h8*)(w_out + (size_t)(n0 + wrow[i]) * K + d * 128 + (u >> 2) * 64 + h * 32 + (u & 3) * 8) =
             dst[i];
@@ -223,22 +275,22 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
   // Stage d + 2 is requested in pieces from step 7 of stage d - 1 (when the barrier
-  // there has freed its buffer) to step 6 of stage d.
-  request(0);
-  request(1);
-  request_part(2, 0);
-  request_part(2, 1);
+  // there has freed its buffer) to step 6 of stage d.  b0, b1, b2: byte offsets of
+  // the buffers of stages d, d + 1, d + 2 (d + 3 takes b0 again).
+  uint32_t b0 = 0, b1 = TD_STAGE, b2 = 2 * TD_STAGE;
+  request(0, b0);
+  request(1, b1);
+  request_part(2, b2, 0);
+  request_part(2, b2, 1);
   __builtin_amdgcn_s_waitcnt(waitcnt_vm(LOADS + 2));  // stage 0 has landed
   __syncthreads();
-  read_x(xv[0], td_lds, 0);
-  read_w(wv[0], td_lds, 0);
-  read_sc(td_lds);
+  read_x(xv[0], b0, 0);
+  read_w(wv[0], b0, 0);
+  read_sc(b0);
   set_group(0);
   expand(av[0], 0, 0);
 #pragma unroll 1
   for (int d = 0; d < stages; ++d) {
-    const uint8_t* base = td_lds + (d % TD_STAGES) * TD_STAGE;
-    const uint8_t* next = td_lds + ((d + 1) % TD_STAGES) * TD_STAGE;
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       if (u == 7) {
@@ -247,18 +299,20 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
         // d + 1 has landed for everyone (outstanding: all of stage d + 2)
         __builtin_amdgcn_s_waitcnt(waitcnt_vm(LOADS));
         __syncthreads();
-        request_part(d + 3, 0);
-        request_part(d + 3, 1);
-        read_x(xv[0], next, 0);
-        read_w(wv[0], next, 0);
-        read_sc(next);
+        request_part(d + 3, b0, 0);
+        request_part(d + 3, b0, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        read_x(xv[0], b1, 0);
+        read_w(wv[0], b1, 0);
+        read_sc(b1);
         set_group(d + 1);
         expand(av[0], d + 1, 0);
       } else {
-        if (2 * u + 2 < LOADS) request_part(d + 2, 2 * u + 2);
-        if (2 * u + 3 < LOADS) request_part(d + 2, 2 * u + 3);
-        read_x(xv[(u + 1) & 1], base, u + 1);
-        if (u == 0) read_w(wv[1], base, 1);
+        if (2 * u + 2 < LOADS) request_part(d + 2, b2, 2 * u + 2);
+        if (2 * u + 3 < LOADS) request_part(d + 2, b2, 2 * u + 3);
+        __builtin_amdgcn_sched_barrier(0);
+        read_x(xv[(u + 1) & 1], b0, u + 1);
+        if (u == 0) read_w(wv[1], b0, 1);
         expand(av[(u + 1) & 1], d, u + 1);
       }
 #pragma unroll
@@ -267,19 +321,34 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
         for (int j = 0; j < 4; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
               av[u & 1][i], __builtin_bit_cast(h8, xv[u & 1][j]), acc[i][j], 0, 0, 0);
-      if (u < 7) {
-        // LDS reads first, then the expansion spread evenly under the MFMAs: a wave
-        // can issue about six vector instructions in the shadow of one MFMA
+      // LDS reads first, then the expansion spread evenly under the MFMAs: a wave
+      // can issue about six vector instructions in the shadow of one MFMA
+      if (u == 7) {
+        // the words to expand have only just been asked for: three MFMAs cover that
+        __builtin_amdgcn_sched_group_barrier(0x100, 6 + 2 * NSC + (ASYM ? 2 : 0), 0);
+#pragma unroll
+        for (int k = 0; k < 3; ++k) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+#pragma unroll
+        for (int k = 0; k < 5; ++k) {
+          __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+      } else {
         if (u == 0) __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
         else __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+          if (u == 0) __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+          else __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
         }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
+    const uint32_t first = b0;
+    b0 = b1;
+    b1 = b2;
+    b2 = first;
   }
   __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // nothing may still be writing LDS at exit
 
@@ -338,7 +407,7 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   }
 }
 
-template <bool ASYM, bool HOOK>
+template <int FMT, int GSM, bool HOOK>
 hipError_t launch(const WView& v, const w4_half* x, w4_half* c, w4_half* w_out, int M,
                   hipStream_t s, int tiles_n, int tiles_m) {
   // more than 64 KB of LDS has to be granted per device, once
@@ -346,41 +415,61 @@ hipError_t launch(const WView& v, const w4_half* x, w4_half* c, w4_half* w_out, 
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
   if (dev < 0 || dev >= 64 || !granted[dev]) {
-    const hipError_t e = hipFuncSetAttribute((const void*)w4_tile_dma_kernel<ASYM, HOOK>,
+    const hipError_t e = hipFuncSetAttribute((const void*)w4_tile_dma_kernel<FMT, GSM, HOOK>,
                                              hipFuncAttributeMaxDynamicSharedMemorySize, TD_LDS);
     if (e != hipSuccess) return e;
     if (dev >= 0 && dev < 64) granted[dev] = true;
   }
-  w4_tile_dma_kernel<ASYM, HOOK>
+  w4_tile_dma_kernel<FMT, GSM, HOOK>
       <<<dim3((unsigned)(tiles_n * tiles_m)), dim3(TD_THREADS), TD_LDS, s>>>(
-          v.q, (const uint16_t*)v.scales, v.zeros, x, c, w_out, v.N, v.K, v.G, v.gs, M, tiles_n,
+          v.q, v.scales, v.zeros, x, c, w_out, v.N, v.K, v.mx ? v.B : v.G, v.gs, M, tiles_n,
           tiles_m);
   return hipGetLastError();
 }
 
+template <int FMT, int GSM>
+hipError_t launch_hook(const WView& v, const w4_half* x, w4_half* c, w4_half* w_out, int M,
+                       hipStream_t s, int tn, int tm) {
+  return w_out ? launch<FMT, GSM, true>(v, x, c, w_out, M, s, tn, tm)
+               : launch<FMT, GSM, false>(v, x, c, nullptr, M, s, tn, tm);
+}
+
+template <int FMT>
+hipError_t launch_gsm(int gsm, const WView& v, const w4_half* x, w4_half* c, w4_half* w_out,
+                      int M, hipStream_t s, int tn, int tm) {
+  if (gsm == 0) return launch_hook<FMT, 0>(v, x, c, w_out, M, s, tn, tm);
+  if (gsm == 1) return launch_hook<FMT, 1>(v, x, c, w_out, M, s, tn, tm);
+  return launch_hook<FMT, 2>(v, x, c, w_out, M, s, tn, tm);
+}
+
 }  // namespace
 
-// Takes W4 weights whose groups hold whole stages (gs a multiple of 128, hence K
-// too), operands under 4 GiB (32-bit offsets), 16-byte aligned rows, an even
-// number of scales (they are fetched as dwords) and a tile grid that covers a
-// good part of the chip.  Returns false, launching nothing, otherwise.
+// Takes MXFP4 weights and W4 weights whose groups tile a 128-k stage (gs 32, 64 or a
+// multiple of 128), K a multiple of 128, operands under 4 GiB (32-bit offsets),
+// 16-byte aligned rows, scales that can be fetched as aligned dwords, and a tile
+// grid that covers a good part of the chip.  Returns false, launching nothing,
+// otherwise.
 bool try_tile_dma(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                   w4_half* w_out, hipError_t* err) {
-  if (v.mx || v.gs % 128 || v.K % 128 || v.K < 128) return false;
+  if (v.K % 128 || v.K < 128) return false;
+  int gsm = 2;
+  if (!v.mx) {
+    if (v.gs % 128 == 0) gsm = 0;
+    else if (v.gs == 64) gsm = 1;
+    else if (v.gs != 32) return false;
+  }
   const long long tiles_n = (v.N + TD_TN - 1) / TD_TN, tiles_m = (M + TD_TM - 1) / TD_TM;
   if (M < 128 || tiles_n * tiles_m < 64 || tiles_n * tiles_m > 0x7FFFFFFFLL) return false;
   if ((long long)v.N * v.K / 2 >= (1LL << 32) || (long long)M * v.K * 2 >= (1LL << 32)) return false;
-  if (((long long)v.N * v.G) & 1) return false;
+  // one FP16 scale per stage: the dword around it must lie inside the array
+  if (gsm == 0 && (((long long)v.N * v.G) & 1)) return false;
   if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)v.scales & 3)) return false;
-  if (!v.symmetric && (v.zeros == nullptr || ((uintptr_t)v.zeros & 3))) return false;
+  if (!v.mx && !v.symmetric && (v.zeros == nullptr || ((uintptr_t)v.zeros & 3))) return false;
   if (w_out && ((uintptr_t)w_out & 15)) return false;
   const int tn = (int)tiles_n, tm = (int)tiles_m;
-  if (w_out)
-    *err = v.symmetric ? launch<false, true>(v, x, c, w_out, M, s, tn, tm)
-                       : launch<true, true>(v, x, c, w_out, M, s, tn, tm);
-  else
-    *err = v.symmetric ? launch<false, false>(v, x, c, nullptr, M, s, tn, tm)
-                       : launch<true, false>(v, x, c, nullptr, M, s, tn, tm);
+  if (v.mx) *err = launch_hook<2, 2>(v, x, c, w_out, M, s, tn, tm);
+  else if (v.symmetric) *err = launch_gsm<0>(gsm, v, x, c, w_out, M, s, tn, tm);
+  else *err = launch_gsm<1>(gsm, v, x, c, w_out, M, s, tn, tm);
   return true;
 }
 

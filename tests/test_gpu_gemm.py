@@ -42,7 +42,9 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         (1030, 2050, 512, 128), (2048, 1024, 384, 128), (1024, 2048, 1280, 256), (1000, 2304, 256, 128),
         (1025, 2049, 384, 128),
         # the same kernel with two and four groups per 128-k stage
-        (1030, 2050, 512, 64), (1024, 2048, 384, 32), (2048, 1030, 256, 32), (900, 2304, 640, 64)]
+        (1030, 2050, 512, 64), (1024, 2048, 384, 32), (2048, 1030, 256, 32), (900, 2304, 640, 64),
+        # a thin grid of its tiles (2 x 8, 1 x 9)
+        (130, 2000, 256, 128), (100, 2100, 384, 32)]
 TOL, CROSS = 1e-3, 2e-3  # rel L2 vs the FP64 oracle; between two gated paths
 
 

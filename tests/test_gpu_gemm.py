@@ -44,7 +44,11 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         # the same kernel with two and four groups per 128-k stage
         (1030, 2050, 512, 64), (1024, 2048, 384, 32), (2048, 1030, 256, 32), (900, 2304, 640, 64),
         # a thin grid of its tiles (2 x 8, 1 x 9)
-        (130, 2000, 256, 128), (100, 2100, 384, 32)]
+        (130, 2000, 256, 128), (100, 2100, 384, 32),
+        # M <= 16 with more 16-row tiles than compute units: two, three and four tiles per
+        # workgroup share one copy of the activations (the last workgroups have fewer)
+        (16, 4128, 2048, 128), (7, 8208, 4096, 64), (9, 12304, 2048, 32), (12, 4144, 4096, 96),
+        (1, 8192, 2048, 128)]
 TOL, CROSS = 1e-3, 2e-3  # rel L2 vs the FP64 oracle; between two gated paths
 
 

@@ -1,0 +1,316 @@
+// Decode-batch W4A16 GEMM for M <= 16 with the activations fetched once per
+// workgroup: c[M,N] = X[M,K] * dequant(W)[N,K]^T, K = 2048 or 4096 (mma.cuh:63-230 is
+// the reference's kernel for this path; it stages x in shared memory per block).
+//
+// At these shapes a 16-row tile of W is 16 KB to 32 KB of codes, and the MFMAs
+// that consume it want 64 KB to 128 KB of FP16 activations as operands.  With one
+// tile per workgroup the activations, not the weights, were what the memory path
+// spent its time on (measured at M = 8, N = 11008, K = 4096: 15.1 us; with constant
+// activations 9.0 us; with constant weights instead 11.3 us).  So a workgroup
+// takes T tiles and brings its activations in once:
+//   * 8 waves split K (wave w owns k in [K/8 w, K/8 (w + 1))), as in the kernels of
+//     gemm_mfma.hip; a wave needs only its own slice of x.
+//   * global_load_lds_dwordx4 moves that slice into the wave's own 8 or 16 KB of
+//     LDS: a load instruction takes 4 rows x 256 contiguous bytes (whole cache
+//     lines; operand loads straight into registers would take 64 bytes of each of
+//     16 rows), pieces XOR-swizzled by the row so that the reads back are
+//     conflict-free.  No other wave touches the region: no barrier.
+//   * the slice is read back once into registers as MFMA B operands and serves
+//     all T tiles; the codes of all T tiles are requested before anything is
+//     consumed.
+//   * a word is expanded in natural k order (see gemm_tile_dma.hip) straight into
+//     the A operand of v_mfma_f32_16x16x32_f16.
+// Partial sums of the eight waves meet in LDS in wave order (no atomics).
+#include "dq.cuh"
+#include "kernels.h"
+
+namespace w4k {
+namespace {
+
+typedef __attribute__((address_space(3))) void* lds_ptr;
+constexpr int DR_WAVES = 8, DR_THREADS = 64 * DR_WAVES;
+constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
+extern __shared__ __attribute__((aligned(16))) uint8_t dr_lds[];
+
+// Eight codes of a packed word -> eight FP16 weights in k order.  cneg: packed
+// {-(1024 + z), -(64 + z)}; s2: the group scale in both halves; mask, magic:
+// 0x00F0000F and 0x54006400 in registers.
+__device__ __forceinline__ h8 expand_word(uint32_t w, h2 cneg, h2 s2, uint32_t mask, uint32_t magic) {
+  u4 out;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t p = __builtin_amdgcn_perm(0u, w, 0x0c000c00u | (uint32_t)(i << 16) | (uint32_t)i);
+    const uint32_t v = (p & mask) | magic;
+    out[i] = as_u32((as_h2(v) + cneg) * s2);
+  }
+  return __builtin_bit_cast(h8, out);
+}
+
+// FMT: 0 W4 symmetric, 1 W4 with zero-points, 2 MXFP4.  K = 1024 CH.  POW2: gs is a
+// power of two (shift gs_shift); GS128: it is 128.  T tiles of
+// 16 rows per workgroup: tile g + gridDim.x t for t < T (tiles past the end are
+// computed on the last tile's rows and not stored).
+template <int FMT, int CH, bool POW2, bool GS128, int T>
+__global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
+    const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
+    const int gs_shift, const int tiles) {
+  constexpr bool MX = FMT == 2;
+  constexpr int K = 1024 * CH, WPR = K / 8;
+  constexpr int XBYTES = 16 * 128 * CH * 2;  // a wave's slice of x: 16 rows x 128 CH k
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane & 15, b = lane >> 4;
+  const int kw = wave * (128 * CH) + 32 * b;  // first k of this lane
+
+  // rows of W this lane reads, per tile
+  size_t nrow[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    const int tile = min((int)blockIdx.x + (int)gridDim.x * t, tiles - 1);
+    nrow[t] = (size_t)(tile * 16 + r);
+  }
+  // Scales: a lane's CH chunks lie 128 k apart.  With groups of 128 (VEC) they are
+  // CH consecutive FP16 scales of the row, one 4- or 8-byte load, and their
+  // zero-points sit in one word; MXFP4's CH bytes are 4 apart in 8 or 16 consecutive
+  // ones.  Other group sizes load them one by one.
+  constexpr bool VEC = MX || (POW2 && GS128);
+  uint32_t sc[T][CH], zw[T][CH];
+  int gidx[CH];
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    const int k = kw + 128 * i;
+    gidx[i] = MX ? (k >> 5) : GS128 ? (k >> 7) : POW2 ? (k >> gs_shift) : k / p.gs;
+  }
+  u4 qw[T][CH];
+  auto load_tile = [&](int t) {
+    const uint32_t* qr = p.q + nrow[t] * WPR + (kw >> 3);
+#pragma unroll
+    for (int i = 0; i < CH; ++i) qw[t][i] = __builtin_nontemporal_load((const u4*)(qr + 16 * i));
+  };
+  auto load_scales = [&](int t) {
+    if constexpr (MX) {  // bytes 4 CH wave .. + 4 CH - 1 of the row; this lane's are b + 4 i
+      const uint8_t* sp = (const uint8_t*)p.scales + nrow[t] * p.B + wave * (4 * CH);
+      uint32_t w[CH];
+      if constexpr (CH == 4) {
+        const u4 v = *(const u4*)sp;
+#pragma unroll
+        for (int i = 0; i < CH; ++i) w[i] = v[i];
+      } else {
+        const u2 v = *(const u2*)sp;
+#pragma unroll
+        for (int i = 0; i < CH; ++i) w[i] = v[i];
+      }
+#pragma unroll
+      for (int i = 0; i < CH; ++i) sc[t][i] = (w[i] >> (8 * b)) & 0xFFu;
+    } else if constexpr (VEC) {
+      const uint16_t* sp = (const uint16_t*)p.scales + nrow[t] * p.G + wave * CH;
+      if constexpr (CH == 4) {
+        const u2 v = *(const u2*)sp;
+        sc[t][0] = v[0] & 0xFFFFu, sc[t][1] = v[0] >> 16, sc[t][2] = v[1] & 0xFFFFu, sc[t][3] = v[1] >> 16;
+      } else {
+        const uint32_t v = *(const uint32_t*)sp;
+        sc[t][0] = v & 0xFFFFu, sc[t][1] = v >> 16;
+      }
+      if (FMT == 1) {
+        const uint32_t z = p.zeros[nrow[t] * words(p.G) + ((wave * CH) >> 3)];
+#pragma unroll
+        for (int i = 0; i < CH; ++i) zw[t][i] = z;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < CH; ++i) {
+        sc[t][i] = ((const uint16_t*)p.scales)[nrow[t] * p.G + gidx[i]];
+        if (FMT == 1) zw[t][i] = p.zeros[nrow[t] * words(p.G) + (gidx[i] >> 3)];
+      }
+    }
+  };
+  // vector loads the scales of all tiles take (between the x slice and the wait)
+  constexpr int SLOADS = T * (VEC ? ((FMT == 1) ? 2 : 1) : ((FMT == 1) ? 2 * CH : CH));
+  load_tile(0);
+
+  // This wave's slice of x -> its LDS region: block (i, rq) = 128-k chunk i of rows
+  // 4 rq .. 4 rq + 3; lane l fetches row 4 rq + l/16, 16-byte piece (l%16) ^ row of
+  // the chunk's 256 bytes.  Rows past M repeat row M - 1 (their columns of the
+  // product are never stored).
+  const uint32_t region = (uint32_t)(uintptr_t)(lds_ptr)dr_lds + (uint32_t)wave * XBYTES;
+  const char* xb = (const char*)x + (size_t)wave * (256 * CH);
+#pragma unroll
+  for (int i = 0; i < CH; ++i)
+#pragma unroll
+    for (int rq = 0; rq < 4; ++rq) {
+      const int row = 4 * rq + (lane >> 4);
+      const uint32_t off = (uint32_t)min(row, M - 1) * (uint32_t)(K * 2) + (uint32_t)i * 256u +
+                           (uint32_t)(((lane & 15) ^ row) * 16);
+      const uint32_t dst = region + (uint32_t)(i * 4 + rq) * 1024u;
+      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :
+                   : "v"(off), "s"(xb), "s"(dst)
+                   : "memory", "m0");
+    }
+#pragma unroll
+  for (int t = 0; t < T; ++t) load_scales(t);
+#pragma unroll
+  for (int t = 1; t < T; ++t) load_tile(t);
+  __builtin_amdgcn_sched_barrier(0);  // every request above is issued before the wait below
+
+  // everything up to and including the x slice has landed once at most the loads
+  // issued after it are outstanding
+  static_assert(SLOADS + CH * (T - 1) < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm(SLOADS + CH * (T - 1)));
+  // B operands: MFMA j of chunk i contracts k = kw + 128 i + 8 j .. + 7 = piece 4 b + j
+  u4 xv[CH][4];
+  {
+    const uint8_t* mine = dr_lds + wave * XBYTES;
+#pragma unroll
+    for (int i = 0; i < CH; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        xv[i][j] = *(const u4*)(mine + (i * 4 + (r >> 2)) * 1024 + ((r & 3) * 16 + ((4 * b + j) ^ r)) * 16);
+  }
+
+  uint32_t mask = 0x00F0000Fu, magic = 0x54006400u;
+  asm volatile("" : "+s"(mask));   // opaque: as literals they cost two instructions
+  asm volatile("" : "+v"(magic));  // instead of one and-or
+  f4* red = (f4*)(dr_lds + DR_WAVES * XBYTES);  // [2][DR_WAVES][64]
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      h2 cneg, s2;
+      float sf = 0.f;
+      if (MX) {
+        sf = mx_scale(sc[t][i]);
+      } else {
+        const uint32_t z = FMT == 1 ? ((zw[t][i] >> (4 * (gidx[i] & 7))) & 0xFu) : 8u;
+        cneg = as_h2(0xD400E400u | (z << 20) | z);
+        s2 = splat_bits(sc[t][i]);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        h8 a;
+        if (MX) {
+          h2 n4[4];
+          dq_mx(qw[t][i][j], sf, n4);
+          a = __builtin_bit_cast(h8, u4{as_u32(n4[0]), as_u32(n4[1]), as_u32(n4[2]), as_u32(n4[3])});
+        } else {
+          a = expand_word(qw[t][i][j], cneg, s2, mask, magic);
+        }
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(h8, xv[i][j]), acc, 0, 0, 0);
+      }
+    }
+    // fixed-order combine of the 8 K slices; the buffer alternates so that one
+    // barrier per tile is enough
+    f4* mine = red + (t & 1) * (DR_WAVES * 64);
+    mine[wave * 64 + lane] = acc;
+    __syncthreads();
+    const int tile = (int)blockIdx.x + (int)gridDim.x * t;
+    if (wave == (t & 7) && tile < tiles) {
+      f4 s = mine[lane];
+#pragma unroll
+      for (int w = 1; w < DR_WAVES; ++w) s += mine[w * 64 + lane];
+      if (r < M) {  // lane: activation row r, weight rows 16 tile + 4 b .. + 3
+        uint16_t hv[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const _Float16 hh = (_Float16)s[e];
+          hv[e] = __builtin_bit_cast(uint16_t, hh);
+        }
+        *(u2*)(c + (size_t)r * p.N + tile * 16 + 4 * b) =
+            u2{hv[0] | ((uint32_t)hv[1] << 16), hv[2] | ((uint32_t)hv[3] << 16)};
+      }
+    }
+  }
+}
+
+template <int FMT, int CH, bool POW2, bool GS128, int T>
+hipError_t launch_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
+                    int tiles, unsigned grid) {
+  constexpr int lds_bytes = DR_WAVES * (16 * 128 * CH * 2) + 2 * DR_WAVES * 64 * 16;
+  // more than 64 KB of LDS has to be granted per device, once
+  static bool granted[64] = {};
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+  if (dev < 0 || dev >= 64 || !granted[dev]) {
+    const hipError_t e =
+        hipFuncSetAttribute((const void*)mfma_decode_resident_kernel<FMT, CH, POW2, GS128, T>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return e;
+    if (dev >= 0 && dev < 64) granted[dev] = true;
+  }
+  mfma_decode_resident_kernel<FMT, CH, POW2, GS128, T>
+      <<<grid, DR_THREADS, lds_bytes, s>>>(v, x, c, M, sh, tiles);
+  return hipGetLastError();
+}
+
+template <int FMT, int CH, bool POW2, bool GS128>
+hipError_t launch_ch(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
+                     int tiles, int T) {
+  const unsigned grid = (unsigned)((tiles + T - 1) / T);
+  switch (T) {
+    case 2: return launch_t<FMT, CH, POW2, GS128, 2>(v, x, c, M, s, sh, tiles, grid);
+    case 3: return launch_t<FMT, CH, POW2, GS128, 3>(v, x, c, M, s, sh, tiles, grid);
+    default: return launch_t<FMT, CH, POW2, GS128, 4>(v, x, c, M, s, sh, tiles, grid);
+  }
+}
+
+template <int FMT>
+hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
+                      int tiles, int T) {
+  const bool pow2 = !v.mx && (v.gs & (v.gs - 1)) == 0;
+  const int sh = pow2 ? __builtin_ctz((unsigned)v.gs) : 0;
+  // the 8-byte scale loads of the gs = 128 form need the scale array 8-byte aligned
+  const bool gs128 = !v.mx && v.gs == 128 && ((uintptr_t)v.scales & 7) == 0;
+  if (v.K == 4096) {
+    if (gs128) return launch_ch<FMT, 4, true, true>(v, x, c, M, s, sh, tiles, T);
+    return pow2 ? launch_ch<FMT, 4, true, false>(v, x, c, M, s, sh, tiles, T)
+                : launch_ch<FMT, 4, false, false>(v, x, c, M, s, sh, tiles, T);
+  }
+  if (gs128) return launch_ch<FMT, 2, true, true>(v, x, c, M, s, sh, tiles, T);
+  return pow2 ? launch_ch<FMT, 2, true, false>(v, x, c, M, s, sh, tiles, T)
+              : launch_ch<FMT, 2, false, false>(v, x, c, M, s, sh, tiles, T);
+}
+
+// Compute units of the current device (per-device cache); 0 on error.
+int device_cus() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < 64 && cached[dev]) return cached[dev];
+  int n = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < 64) cached[dev] = n;
+  return n;
+}
+
+// M <= 16, K = 2048 or 4096, whole 16-row tiles, a lane's 32-k slice inside one
+// group, 16-byte aligned operands, and two to four tiles per compute unit (with
+// one tile per workgroup there is nothing to share).
+int decode_resident_tiles(const WView& v, const w4_half* x, const w4_half* c, int M) {
+  if (M > 16 || M < 1 || v.N % 16 || (v.K != 2048 && v.K != 4096)) return 0;
+  if (!v.mx && v.gs % 32) return 0;
+  if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)c & 7)) return 0;
+  if (v.mx && ((uintptr_t)v.scales & 15)) return 0;  // a slice's scale bytes are one vector load
+  const int cus = device_cus();
+  if (cus < 1) return 0;
+  const int T = (v.N / 16 + cus - 1) / cus;
+  return (T >= 2 && T <= 4) ? T : 0;
+}
+
+}  // namespace
+
+bool decode_resident_applies(const WView& v, const w4_half* x, const w4_half* c, int M) {
+  return decode_resident_tiles(v, x, c, M) != 0;
+}
+
+// Precondition: decode_resident_applies(v, x, c, M); no hook.
+hipError_t launch_decode_resident(const WView& v, const w4_half* x, w4_half* c, int M,
+                                  hipStream_t s) {
+  const int T = decode_resident_tiles(v, x, c, M);
+  if (T == 0) return hipErrorInvalidValue;
+  const int tiles = v.N / 16;
+  if (v.mx) return launch_fmt<2>(v, x, c, M, s, tiles, T);
+  return v.symmetric ? launch_fmt<0>(v, x, c, M, s, tiles, T) : launch_fmt<1>(v, x, c, M, s, tiles, T);
+}
+
+}  // namespace w4k

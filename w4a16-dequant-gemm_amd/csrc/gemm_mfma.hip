@@ -990,7 +990,11 @@ static hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M
   if (aligned) {
     // Measured on N = 4096 .. 14336, K = 4096 .. 11008: the K-split kernel wins for
     // M <= 16 unless N is large enough to give the streaming kernel a full grid.
-    const bool ksplit = M <= 8 || (M <= 16 && v.N < 8192);
+    // Shapes of the kernel that shares the activations among several tiles: hooked
+    // calls take the K-split kernel, which adds in the same order.
+    const bool resident = wvec && decode_resident_applies(v, x, c, M);
+    if (resident && w_out == nullptr) return launch_decode_resident(v, x, c, M, s);
+    const bool ksplit = M <= 8 || (M <= 16 && v.N < 8192) || resident;
     if (ksplit && wvec &&
         (MX ? try_decode_unrolled<2>(v, x, c, M, s, w_out, &terr)
             : v.symmetric ? try_decode_unrolled<0>(v, x, c, M, s, w_out, &terr)

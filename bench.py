@@ -310,6 +310,25 @@ def extras_gemm(b, full):
                          "fused_TFLOPs": flop / fused_ms * 1e-9, "two_pass_ms": two_ms,
                          "two_pass_TFLOPs": flop / two_ms * 1e-9, "hipblaslt_only_TFLOPs": flop / blas_ms * 1e-9,
                          "frac_of_mfma_peak": flop / fused_ms * 1e-9 / MFMA_F16_PEAK_TFLOPS}
+    # the same kernel on the other formats it takes, and on a thin and a large grid
+    rows = []
+    del views
+    fmts = [("w4_asym_gs128", lambda: b.rand_w4(N, K, 128, False, 1), capi.gemm),
+            ("w4_sym_gs32", lambda: b.rand_w4(N, K, 32, True, 1), capi.gemm),
+            ("mxfp4", lambda: b.rand_mx(N, K, 1), capi.gemm_mx)]
+    for name, make, fn in fmts:
+        v = make()
+        ms = _median_events_ms(torch, lambda i: fn(v[0][0], x.data_ptr(), c.data_ptr(), M, st, 0), steps, 3)
+        rows.append({"weights": name, "M": M, "us": ms * 1e3, "TFLOPs": flop / ms * 1e-9})
+        del v
+    v = b.rand_w4(N, K, 128, True, 1)
+    for M2 in (256, 4096) if full else (256,):
+        x2 = torch.randn(M2 * K, device="cuda").to(torch.float16)
+        c2 = torch.empty(M2 * N, dtype=torch.float16, device="cuda")
+        ms = _median_events_ms(torch, lambda i: capi.gemm(v[0][0], x2.data_ptr(), c2.data_ptr(), M2, st, 0),
+                               steps, 3)
+        rows.append({"weights": "w4_sym_gs128", "M": M2, "us": ms * 1e3, "TFLOPs": 2.0 * M2 * N * K / ms * 1e-9})
+    out["c4_prefill_other"] = rows
     return out
 
 

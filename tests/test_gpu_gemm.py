@@ -48,7 +48,11 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         # M <= 16 with more 16-row tiles than compute units: two, three and four tiles per
         # workgroup share one copy of the activations (the last workgroups have fewer)
         (16, 4128, 2048, 128), (7, 8208, 4096, 64), (9, 12304, 2048, 32), (12, 4144, 4096, 96),
-        (1, 8192, 2048, 128)]
+        (1, 8192, 2048, 128),
+        # the same with two and four 16-row tiles of activations (17 <= M <= 64), which pass
+        # through the wave's LDS region in phases
+        (17, 4128, 4096, 128), (32, 8208, 2048, 64), (33, 4144, 4096, 32), (64, 12304, 2048, 128),
+        (50, 4128, 2048, 96)]
 TOL, CROSS = 1e-3, 2e-3  # rel L2 vs the FP64 oracle; between two gated paths
 
 

@@ -47,16 +47,23 @@ __device__ __forceinline__ h8 expand_word(uint32_t w, h2 cneg, h2 s2, uint32_t m
 }
 
 // FMT: 0 W4 symmetric, 1 W4 with zero-points, 2 MXFP4.  K = 1024 CH.  POW2: gs is a
-// power of two (shift gs_shift); GS128: it is 128.  T tiles of
-// 16 rows per workgroup: tile g + gridDim.x t for t < T (tiles past the end are
-// computed on the last tile's rows and not stored).
-template <int FMT, int CH, bool POW2, bool GS128, int T>
+// power of two (shift gs_shift); GS128: it is 128.  T tiles of 16 rows per
+// workgroup: tile g + gridDim.x t for t < T (tiles past the end are computed on
+// the last tile's rows and not stored).  MT tiles of 16 activation rows (M <= 16 MT).
+//
+// A wave's LDS region holds 16 KB: with MT > 1 its slice of x goes through it in MT
+// phases of CP = 4 / MT chunks of 128 k (all MT row tiles of a chunk at a time); the
+// next phase is requested as soon as the current one sits in registers, so it
+// lands while the current one multiplies.
+template <int FMT, int CH, bool POW2, bool GS128, int T, int MT>
 __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
     const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
     const int gs_shift, const int tiles) {
   constexpr bool MX = FMT == 2;
   constexpr int K = 1024 * CH, WPR = K / 8;
-  constexpr int XBYTES = 16 * 128 * CH * 2;  // a wave's slice of x: 16 rows x 128 CH k
+  constexpr int CP = (4 / MT) < CH ? (4 / MT) : CH;  // chunks per phase
+  constexpr int PH = CH / CP;                         // phases
+  constexpr int XBYTES = MT * CP * 4096;              // the wave's LDS region
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, b = lane >> 4;
@@ -124,123 +131,168 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
       }
     }
   };
-  // vector loads the scales of all tiles take (between the x slice and the wait)
+  // vector loads the scales of all tiles take (between the first x request and the wait)
   constexpr int SLOADS = T * (VEC ? ((FMT == 1) ? 2 : 1) : ((FMT == 1) ? 2 * CH : CH));
   load_tile(0);
 
-  // This wave's slice of x -> its LDS region: block (i, rq) = 128-k chunk i of rows
-  // 4 rq .. 4 rq + 3; lane l fetches row 4 rq + l/16, 16-byte piece (l%16) ^ row of
-  // the chunk's 256 bytes.  Rows past M repeat row M - 1 (their columns of the
-  // product are never stored).
+  // Phase ph of this wave's slice of x -> its LDS region: block (mt, cc, rq) = rows
+  // 16 mt + 4 rq .. + 3 of the 128-k chunk CP ph + cc; lane l fetches row l/16 of the
+  // four, 16-byte piece (l%16) ^ (row % 16) of the chunk's 256 bytes.  Rows past M
+  // repeat row M - 1 (their columns of the product are never stored).
   const uint32_t region = (uint32_t)(uintptr_t)(lds_ptr)dr_lds + (uint32_t)wave * XBYTES;
   const char* xb = (const char*)x + (size_t)wave * (256 * CH);
+  auto request_x = [&](int ph) {
 #pragma unroll
-  for (int i = 0; i < CH; ++i)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int rq = 0; rq < 4; ++rq) {
-      const int row = 4 * rq + (lane >> 4);
-      const uint32_t off = (uint32_t)min(row, M - 1) * (uint32_t)(K * 2) + (uint32_t)i * 256u +
-                           (uint32_t)(((lane & 15) ^ row) * 16);
-      const uint32_t dst = region + (uint32_t)(i * 4 + rq) * 1024u;
-      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
-                   :
-                   : "v"(off), "s"(xb), "s"(dst)
-                   : "memory", "m0");
-    }
+      for (int cc = 0; cc < CP; ++cc)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          const int r16 = 4 * rq + (lane >> 4), row = 16 * mt + r16;
+          const uint32_t off = (uint32_t)min(row, M - 1) * (uint32_t)(K * 2) +
+                               (uint32_t)(ph * CP + cc) * 256u + (uint32_t)(((lane & 15) ^ r16) * 16);
+          const uint32_t dst = region + (uint32_t)((mt * CP + cc) * 4 + rq) * 1024u;
+          asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                       :
+                       : "v"(off), "s"(xb), "s"(dst)
+                       : "memory", "m0");
+        }
+  };
+  request_x(0);
 #pragma unroll
   for (int t = 0; t < T; ++t) load_scales(t);
 #pragma unroll
   for (int t = 1; t < T; ++t) load_tile(t);
   __builtin_amdgcn_sched_barrier(0);  // every request above is issued before the wait below
 
-  // everything up to and including the x slice has landed once at most the loads
-  // issued after it are outstanding
-  static_assert(SLOADS + CH * (T - 1) < 64, "vmcnt is a 6-bit counter");
-  __builtin_amdgcn_s_waitcnt(waitcnt_vm(SLOADS + CH * (T - 1)));
-  // B operands: MFMA j of chunk i contracts k = kw + 128 i + 8 j .. + 7 = piece 4 b + j
-  u4 xv[CH][4];
-  {
-    const uint8_t* mine = dr_lds + wave * XBYTES;
-#pragma unroll
-    for (int i = 0; i < CH; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        xv[i][j] = *(const u4*)(mine + (i * 4 + (r >> 2)) * 1024 + ((r & 3) * 16 + ((4 * b + j) ^ r)) * 16);
-  }
-
   uint32_t mask = 0x00F0000Fu, magic = 0x54006400u;
   asm volatile("" : "+s"(mask));   // opaque: as literals they cost two instructions
   asm volatile("" : "+v"(magic));  // instead of one and-or
-  f4* red = (f4*)(dr_lds + DR_WAVES * XBYTES);  // [2][DR_WAVES][64]
+  f4 acc[T][MT];
 #pragma unroll
-  for (int t = 0; t < T; ++t) {
-    f4 acc = f4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < T; ++t)
 #pragma unroll
-    for (int i = 0; i < CH; ++i) {
-      h2 cneg, s2;
-      float sf = 0.f;
-      if (MX) {
-        sf = mx_scale(sc[t][i]);
-      } else {
-        const uint32_t z = FMT == 1 ? ((zw[t][i] >> (4 * (gidx[i] & 7))) & 0xFu) : 8u;
-        cneg = as_h2(0xD400E400u | (z << 20) | z);
-        s2 = splat_bits(sc[t][i]);
-      }
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f4{0.f, 0.f, 0.f, 0.f};
+
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        h8 a;
-        if (MX) {
-          h2 n4[4];
-          dq_mx(qw[t][i][j], sf, n4);
-          a = __builtin_bit_cast(h8, u4{as_u32(n4[0]), as_u32(n4[1]), as_u32(n4[2]), as_u32(n4[3])});
-        } else {
-          a = expand_word(qw[t][i][j], cneg, s2, mask, magic);
-        }
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(h8, xv[i][j]), acc, 0, 0, 0);
-      }
+  for (int ph = 0; ph < PH; ++ph) {
+    // Phase 0 has landed once at most the loads issued after it are outstanding;
+    // later phases are the youngest requests of the wave.
+    static_assert(SLOADS + CH * (T - 1) < 64, "vmcnt is a 6-bit counter");
+    if (ph == 0) __builtin_amdgcn_s_waitcnt(waitcnt_vm(SLOADS + CH * (T - 1)));
+    else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    // B operands: MFMA j of chunk i contracts k = kw + 128 i + 8 j .. + 7 = piece 4 b + j
+    u4 xv[MT][CP][4];
+    {
+      const uint8_t* mine = dr_lds + wave * XBYTES;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int cc = 0; cc < CP; ++cc)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            xv[mt][cc][j] = *(const u4*)(mine + ((mt * CP + cc) * 4 + (r >> 2)) * 1024 +
+                                         ((r & 3) * 16 + ((4 * b + j) ^ r)) * 16);
     }
-    // fixed-order combine of the 8 K slices; the buffer alternates so that one
-    // barrier per tile is enough
-    f4* mine = red + (t & 1) * (DR_WAVES * 64);
-    mine[wave * 64 + lane] = acc;
-    __syncthreads();
-    const int tile = (int)blockIdx.x + (int)gridDim.x * t;
-    if (wave == (t & 7) && tile < tiles) {
-      f4 s = mine[lane];
+    if (ph + 1 < PH) {
+      // the region is free once these reads have returned: ask for the next phase now
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+      __builtin_amdgcn_sched_barrier(0);
+      request_x(ph + 1);
+    }
 #pragma unroll
-      for (int w = 1; w < DR_WAVES; ++w) s += mine[w * 64 + lane];
-      if (r < M) {  // lane: activation row r, weight rows 16 tile + 4 b .. + 3
-        uint16_t hv[4];
+    for (int t = 0; t < T; ++t)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const _Float16 hh = (_Float16)s[e];
-          hv[e] = __builtin_bit_cast(uint16_t, hh);
+      for (int cc = 0; cc < CP; ++cc) {
+        const int i = ph * CP + cc;
+        h2 cneg, s2;
+        float sf = 0.f;
+        if (MX) {
+          sf = mx_scale(sc[t][i]);
+        } else {
+          const uint32_t z = FMT == 1 ? ((zw[t][i] >> (4 * (gidx[i] & 7))) & 0xFu) : 8u;
+          cneg = as_h2(0xD400E400u | (z << 20) | z);
+          s2 = splat_bits(sc[t][i]);
         }
-        *(u2*)(c + (size_t)r * p.N + tile * 16 + 4 * b) =
-            u2{hv[0] | ((uint32_t)hv[1] << 16), hv[2] | ((uint32_t)hv[3] << 16)};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          h8 a;
+          if (MX) {
+            h2 n4[4];
+            dq_mx(qw[t][i][j], sf, n4);
+            a = __builtin_bit_cast(h8, u4{as_u32(n4[0]), as_u32(n4[1]), as_u32(n4[2]), as_u32(n4[3])});
+          } else {
+            a = expand_word(qw[t][i][j], cneg, s2, mask, magic);
+          }
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(h8, xv[mt][cc][j]),
+                                                                acc[t][mt], 0, 0, 0);
+        }
       }
+  }
+
+  // Fixed-order combine of the 8 K slices.  The x regions are free once every wave
+  // is here; entry (t, mt) of wave w goes to red[w][t MT + mt]; wave w then sums
+  // the entries e = w, w + 8, ... in wave order and stores them.
+  constexpr int E = T * MT;
+  static_assert(E * 1024 <= XBYTES || E <= 8 * (XBYTES / 1024) , "reduction buffer fits the x regions");
+  __syncthreads();
+  f4* red = (f4*)dr_lds;  // [DR_WAVES][E][64]
+#pragma unroll
+  for (int t = 0; t < T; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) red[(wave * E + t * MT + mt) * 64 + lane] = acc[t][mt];
+  __syncthreads();
+  for (int e = wave; e < E; e += DR_WAVES) {
+    const int t = e / MT, mt = e % MT;
+    const int tile = (int)blockIdx.x + (int)gridDim.x * t;
+    if (tile >= tiles) continue;
+    f4 s = red[e * 64 + lane];
+#pragma unroll
+    for (int w = 1; w < DR_WAVES; ++w) s += red[(w * E + e) * 64 + lane];
+    const int m = 16 * mt + r;
+    if (m < M) {  // lane: activation row m, weight rows 16 tile + 4 b .. + 3
+      uint16_t hv[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const _Float16 hh = (_Float16)s[k];
+        hv[k] = __builtin_bit_cast(uint16_t, hh);
+      }
+      *(u2*)(c + (size_t)m * p.N + tile * 16 + 4 * b) =
+          u2{hv[0] | ((uint32_t)hv[1] << 16), hv[2] | ((uint32_t)hv[3] << 16)};
     }
   }
 }
 
-template <int FMT, int CH, bool POW2, bool GS128, int T>
+template <int FMT, int CH, bool POW2, bool GS128, int T, int MT>
 hipError_t launch_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
                     int tiles, unsigned grid) {
-  constexpr int lds_bytes = DR_WAVES * (16 * 128 * CH * 2) + 2 * DR_WAVES * 64 * 16;
+  constexpr int CP = (4 / MT) < CH ? (4 / MT) : CH;
+  constexpr int lds_bytes = DR_WAVES * MT * CP * 4096;
+  static_assert(DR_WAVES * T * MT * 1024 <= lds_bytes, "the reduction reuses the x regions");
   // more than 64 KB of LDS has to be granted per device, once
   static bool granted[64] = {};
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
   if (dev < 0 || dev >= 64 || !granted[dev]) {
     const hipError_t e =
-        hipFuncSetAttribute((const void*)mfma_decode_resident_kernel<FMT, CH, POW2, GS128, T>,
+        hipFuncSetAttribute((const void*)mfma_decode_resident_kernel<FMT, CH, POW2, GS128, T, MT>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return e;
     if (dev >= 0 && dev < 64) granted[dev] = true;
   }
-  mfma_decode_resident_kernel<FMT, CH, POW2, GS128, T>
+  mfma_decode_resident_kernel<FMT, CH, POW2, GS128, T, MT>
       <<<grid, DR_THREADS, lds_bytes, s>>>(v, x, c, M, sh, tiles);
   return hipGetLastError();
+}
+
+template <int FMT, int CH, bool POW2, bool GS128, int T>
+hipError_t launch_mt(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
+                     int tiles, unsigned grid) {
+  if (M <= 16) return launch_t<FMT, CH, POW2, GS128, T, 1>(v, x, c, M, s, sh, tiles, grid);
+  if (M <= 32) return launch_t<FMT, CH, POW2, GS128, T, 2>(v, x, c, M, s, sh, tiles, grid);
+  return launch_t<FMT, CH, POW2, GS128, T, 4>(v, x, c, M, s, sh, tiles, grid);
 }
 
 template <int FMT, int CH, bool POW2, bool GS128>
@@ -248,9 +300,9 @@ hipError_t launch_ch(const WView& v, const w4_half* x, w4_half* c, int M, hipStr
                      int tiles, int T) {
   const unsigned grid = (unsigned)((tiles + T - 1) / T);
   switch (T) {
-    case 2: return launch_t<FMT, CH, POW2, GS128, 2>(v, x, c, M, s, sh, tiles, grid);
-    case 3: return launch_t<FMT, CH, POW2, GS128, 3>(v, x, c, M, s, sh, tiles, grid);
-    default: return launch_t<FMT, CH, POW2, GS128, 4>(v, x, c, M, s, sh, tiles, grid);
+    case 2: return launch_mt<FMT, CH, POW2, GS128, 2>(v, x, c, M, s, sh, tiles, grid);
+    case 3: return launch_mt<FMT, CH, POW2, GS128, 3>(v, x, c, M, s, sh, tiles, grid);
+    default: return launch_mt<FMT, CH, POW2, GS128, 4>(v, x, c, M, s, sh, tiles, grid);
   }
 }
 
@@ -283,18 +335,22 @@ int device_cus() {
   return n;
 }
 
-// M <= 16, K = 2048 or 4096, whole 16-row tiles, a lane's 32-k slice inside one
+// M <= 64, K = 2048 or 4096, whole 16-row tiles, a lane's 32-k slice inside one
 // group, 16-byte aligned operands, and two to four tiles per compute unit (with
 // one tile per workgroup there is nothing to share).
 int decode_resident_tiles(const WView& v, const w4_half* x, const w4_half* c, int M) {
-  if (M > 16 || M < 1 || v.N % 16 || (v.K != 2048 && v.K != 4096)) return 0;
+  if (M > 64 || M < 1 || v.N % 16 || (v.K != 2048 && v.K != 4096)) return 0;
   if (!v.mx && v.gs % 32) return 0;
   if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)c & 7)) return 0;
   if (v.mx && ((uintptr_t)v.scales & 15)) return 0;  // a slice's scale bytes are one vector load
   const int cus = device_cus();
   if (cus < 1) return 0;
   const int T = (v.N / 16 + cus - 1) / cus;
-  return (T >= 2 && T <= 4) ? T : 0;
+  if (T < 2 || T > 4) return 0;
+  // the one combination that does not fit the register file: four tiles, four row
+  // tiles, zero-points and per-chunk scale loads
+  if (T == 4 && M > 32 && !v.mx && !v.symmetric && v.gs != 128) return 0;
+  return T;
 }
 
 }  // namespace

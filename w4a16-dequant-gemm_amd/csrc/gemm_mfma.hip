@@ -450,10 +450,25 @@ static hipError_t launch_decode_mt(const WView& v, const w4_half* x, w4_half* c,
   return hipGetLastError();
 }
 
+// Hooked calls of the shapes the resident-activation kernel takes with 17 <= M <= 64
+// (gs % 32 == 0, 16-byte aligned rows): same K split, same order of additions.
+template <int FMT, int MT>
+static hipError_t launch_decode_hooked_mt(const WView& v, const w4_half* x, w4_half* c, int M,
+                                          hipStream_t s, w4_half* w_out) {
+  int gs_shift = -1;
+  if (!v.mx && (v.gs & (v.gs - 1)) == 0) gs_shift = __builtin_ctz((unsigned)v.gs);
+  const dim3 grid((unsigned)((v.N + 15) / 16), (unsigned)((M + 16 * MT - 1) / (16 * MT)));
+  mfma_decode_kernel<FMT, MT, 1, 1, true, true, true>
+      <<<grid, DEC_WAVES * 64, 0, s>>>(v, x, c, M, w_out, gs_shift);
+  return hipGetLastError();
+}
+
 template <int FMT>
 static hipError_t launch_decode(const WView& v, const w4_half* x, w4_half* c, int M,
                                 hipStream_t s, w4_half* w_out, bool wvec) {
-  return launch_decode_mt<FMT, 1>(v, x, c, M, s, w_out, wvec);  // M <= 16
+  if (M <= 16) return launch_decode_mt<FMT, 1>(v, x, c, M, s, w_out, wvec);
+  if (M <= 32) return launch_decode_hooked_mt<FMT, 2>(v, x, c, M, s, w_out);
+  return launch_decode_hooked_mt<FMT, 4>(v, x, c, M, s, w_out);
 }
 
 // ---- streaming decode-batch kernel --------------------------------------------------
@@ -990,8 +1005,8 @@ static hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M
   if (aligned) {
     // Measured on N = 4096 .. 14336, K = 4096 .. 11008: the K-split kernel wins for
     // M <= 16 unless N is large enough to give the streaming kernel a full grid.
-    // Shapes of the kernel that shares the activations among several tiles: hooked
-    // calls take the K-split kernel, which adds in the same order.
+    // Shapes of the kernel that shares the activations among several tiles (M <= 64):
+    // hooked calls take the K-split kernel, which adds in the same order.
     const bool resident = wvec && decode_resident_applies(v, x, c, M);
     if (resident && w_out == nullptr) return launch_decode_resident(v, x, c, M, s);
     const bool ksplit = M <= 8 || (M <= 16 && v.N < 8192) || resident;

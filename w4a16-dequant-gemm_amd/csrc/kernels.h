@@ -44,7 +44,7 @@ hipError_t launch_gemm_mfma(const WView& v, const w4_half* x, w4_half* c, int M,
 bool try_tile_dma(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                   w4_half* w_out, hipError_t* err);
 
-// gemm_decode_resident.hip: M <= 16 with the activations fetched once per workgroup
+// gemm_decode_resident.hip: M <= 64 with the activations fetched once per workgroup
 // (several 16-row tiles each).  Same order of additions as the K-split decode
 // kernels of gemm_mfma.hip, which serve the hooked calls of these shapes.
 bool decode_resident_applies(const WView& v, const w4_half* x, const w4_half* c, int M);

@@ -52,7 +52,9 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         # the same with two and four 16-row tiles of activations (17 <= M <= 64), which pass
         # through the wave's LDS region in phases
         (17, 4128, 4096, 128), (32, 8208, 2048, 64), (33, 4144, 4096, 32), (64, 12304, 2048, 128),
-        (50, 4128, 2048, 96)]
+        (50, 4128, 2048, 96),
+        # more than four tiles per compute unit: four per workgroup, more workgroups than units
+        (8, 16416, 2048, 128)]
 TOL, CROSS = 1e-3, 2e-3  # rel L2 vs the FP64 oracle; between two gated paths
 
 

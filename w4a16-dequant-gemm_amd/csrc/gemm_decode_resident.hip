@@ -47,7 +47,8 @@ __device__ __forceinline__ h8 expand_word(uint32_t w, h2 cneg, h2 s2, uint32_t m
 }
 
 // FMT: 0 W4 symmetric, 1 W4 with zero-points, 2 MXFP4.  K = 1024 CH.  POW2: gs is a
-// power of two (shift gs_shift); GS128: it is 128.  T tiles of 16 rows per
+// power of two (shift gs_shift); GSV: 1, 2, 3 for gs = 128, 64, 32 with scale arrays
+// aligned for vector loads, else 0.  T tiles of 16 rows per
 // workgroup: tile g + gridDim.x t for t < T (tiles past the end are computed on
 // the last tile's rows and not stored).  MT tiles of 16 activation rows (M <= 16 MT).
 //
@@ -55,7 +56,7 @@ __device__ __forceinline__ h8 expand_word(uint32_t w, h2 cneg, h2 s2, uint32_t m
 // phases of CP = 4 / MT chunks of 128 k (all MT row tiles of a chunk at a time); the
 // next phase is requested as soon as the current one sits in registers, so it
 // lands while the current one multiplies.
-template <int FMT, int CH, bool POW2, bool GS128, int T, int MT>
+template <int FMT, int CH, bool POW2, int GSV, int T, int MT>
 __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
     const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
     const int gs_shift, const int tiles) {
@@ -76,17 +77,20 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
     const int tile = min((int)blockIdx.x + (int)gridDim.x * t, tiles - 1);
     nrow[t] = (size_t)(tile * 16 + r);
   }
-  // Scales: a lane's CH chunks lie 128 k apart.  With groups of 128 (VEC) they are
-  // CH consecutive FP16 scales of the row, one 4- or 8-byte load, and their
-  // zero-points sit in one word; MXFP4's CH bytes are 4 apart in 8 or 16 consecutive
-  // ones.  Other group sizes load them one by one.
-  constexpr bool VEC = MX || (POW2 && GS128);
+  // Scales: a lane's CH chunks lie 128 k apart; chunk i of lane group b is group
+  // (CH wave + i) (128 / gs) + b / (gs / 32) of the row.  With gs = 128, 64 or 32 (GSV)
+  // the wave's groups are CH, 2 CH or 4 CH consecutive FP16 scales: one or two vector
+  // loads and a per-lane pick, and their zero-points sit in one or two words;
+  // MXFP4's CH bytes are 4 apart in 4 CH consecutive ones.  Other group sizes load
+  // them one by one.
+  constexpr bool VEC = MX || GSV != 0;
+  constexpr int PER = MX ? 4 : GSV == 1 ? 1 : GSV == 2 ? 2 : 4;  // groups per 128-k chunk
   uint32_t sc[T][CH], zw[T][CH];
   int gidx[CH];
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
     const int k = kw + 128 * i;
-    gidx[i] = MX ? (k >> 5) : GS128 ? (k >> 7) : POW2 ? (k >> gs_shift) : k / p.gs;
+    gidx[i] = MX ? (k >> 5) : GSV ? (k >> (8 - GSV)) : POW2 ? (k >> gs_shift) : k / p.gs;
   }
   u4 qw[T][CH];
   auto load_tile = [&](int t) {
@@ -110,18 +114,48 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
 #pragma unroll
       for (int i = 0; i < CH; ++i) sc[t][i] = (w[i] >> (8 * b)) & 0xFFu;
     } else if constexpr (VEC) {
-      const uint16_t* sp = (const uint16_t*)p.scales + nrow[t] * p.G + wave * CH;
-      if constexpr (CH == 4) {
+      // HALVES consecutive scales = HALVES / 2 dwords; this lane's scale of chunk i is
+      // half PER i + (b >> (GSV == 2 ? 1 : 0 ...)) of them
+      constexpr int HALVES = PER * CH, DW = HALVES / 2;
+      const uint32_t* sp = (const uint32_t*)((const uint16_t*)p.scales + nrow[t] * p.G + wave * HALVES);
+      uint32_t w[DW];
+      if constexpr (DW == 1) {
+        w[0] = *sp;
+      } else if constexpr (DW == 2) {
         const u2 v = *(const u2*)sp;
-        sc[t][0] = v[0] & 0xFFFFu, sc[t][1] = v[0] >> 16, sc[t][2] = v[1] & 0xFFFFu, sc[t][3] = v[1] >> 16;
+        w[0] = v[0], w[1] = v[1];
       } else {
-        const uint32_t v = *(const uint32_t*)sp;
-        sc[t][0] = v & 0xFFFFu, sc[t][1] = v >> 16;
+#pragma unroll
+        for (int q = 0; q < DW / 4; ++q) {
+          const u4 v = *(const u4*)(sp + 4 * q);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[4 * q + e] = v[e];
+        }
+      }
+      const int sub = GSV == 1 ? 0 : GSV == 2 ? (b >> 1) : b;  // group of the chunk this lane is in
+#pragma unroll
+      for (int i = 0; i < CH; ++i) {
+        // half index PER i + sub: dword (PER i + sub) / 2, upper half if odd
+        uint32_t d;
+        if constexpr (PER == 4) d = (sub & 2) ? w[2 * i + 1] : w[2 * i];
+        else if constexpr (PER == 2) d = w[i];
+        else d = w[i >> 1];
+        const bool hi = PER == 1 ? (i & 1) : (sub & 1);
+        sc[t][i] = hi ? (d >> 16) : (d & 0xFFFFu);
       }
       if (FMT == 1) {
-        const uint32_t z = p.zeros[nrow[t] * words(p.G) + ((wave * CH) >> 3)];
+        // groups PER CH wave .. + PER CH - 1: one zero-point word per eight
+        constexpr int ZW = (HALVES + 7) / 8;
+        const uint32_t* zp = p.zeros + nrow[t] * words(p.G) + ((wave * HALVES) >> 3);
+        uint32_t z[ZW];
+        if constexpr (ZW == 2) {
+          const u2 v = *(const u2*)zp;
+          z[0] = v[0], z[1] = v[1];
+        } else {
+          z[0] = *zp;
+        }
 #pragma unroll
-        for (int i = 0; i < CH; ++i) zw[t][i] = z;
+        for (int i = 0; i < CH; ++i) zw[t][i] = z[ZW == 2 ? (i >> 1) : 0];
       }
     } else {
 #pragma unroll
@@ -132,7 +166,8 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
     }
   };
   // vector loads the scales of all tiles take (between the first x request and the wait)
-  constexpr int SLOADS = T * (VEC ? ((FMT == 1) ? 2 : 1) : ((FMT == 1) ? 2 * CH : CH));
+  constexpr int SVEC = MX ? 1 : (PER * CH / 2 + 3) / 4;  // vector loads of a tile's scales
+  constexpr int SLOADS = T * (VEC ? SVEC + ((FMT == 1) ? 1 : 0) : ((FMT == 1) ? 2 * CH : CH));
   load_tile(0);
 
   // Phase ph of this wave's slice of x -> its LDS region: block (mt, cc, rq) = rows
@@ -265,7 +300,7 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
   }
 }
 
-template <int FMT, int CH, bool POW2, bool GS128, int T, int MT>
+template <int FMT, int CH, bool POW2, int GSV, int T, int MT>
 hipError_t launch_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
                     int tiles, unsigned grid) {
   constexpr int CP = (4 / MT) < CH ? (4 / MT) : CH;
@@ -277,33 +312,33 @@ hipError_t launch_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStre
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
   if (dev < 0 || dev >= 64 || !granted[dev]) {
     const hipError_t e =
-        hipFuncSetAttribute((const void*)mfma_decode_resident_kernel<FMT, CH, POW2, GS128, T, MT>,
+        hipFuncSetAttribute((const void*)mfma_decode_resident_kernel<FMT, CH, POW2, GSV, T, MT>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return e;
     if (dev >= 0 && dev < 64) granted[dev] = true;
   }
-  mfma_decode_resident_kernel<FMT, CH, POW2, GS128, T, MT>
+  mfma_decode_resident_kernel<FMT, CH, POW2, GSV, T, MT>
       <<<grid, DR_THREADS, lds_bytes, s>>>(v, x, c, M, sh, tiles);
   return hipGetLastError();
 }
 
-template <int FMT, int CH, bool POW2, bool GS128, int T>
+template <int FMT, int CH, bool POW2, int GSV, int T>
 hipError_t launch_mt(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
                      int tiles, unsigned grid) {
-  if (M <= 16) return launch_t<FMT, CH, POW2, GS128, T, 1>(v, x, c, M, s, sh, tiles, grid);
-  if (M <= 32) return launch_t<FMT, CH, POW2, GS128, T, 2>(v, x, c, M, s, sh, tiles, grid);
-  return launch_t<FMT, CH, POW2, GS128, T, 4>(v, x, c, M, s, sh, tiles, grid);
+  if (M <= 16) return launch_t<FMT, CH, POW2, GSV, T, 1>(v, x, c, M, s, sh, tiles, grid);
+  if (M <= 32) return launch_t<FMT, CH, POW2, GSV, T, 2>(v, x, c, M, s, sh, tiles, grid);
+  return launch_t<FMT, CH, POW2, GSV, T, 4>(v, x, c, M, s, sh, tiles, grid);
 }
 
-template <int FMT, int CH, bool POW2, bool GS128>
+template <int FMT, int CH, bool POW2, int GSV>
 hipError_t launch_ch(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
                      int tiles, int T) {
   const unsigned grid = (unsigned)((tiles + T - 1) / T);
   switch (T) {
-    case 1: return launch_mt<FMT, CH, POW2, GS128, 1>(v, x, c, M, s, sh, tiles, grid);
-    case 2: return launch_mt<FMT, CH, POW2, GS128, 2>(v, x, c, M, s, sh, tiles, grid);
-    case 3: return launch_mt<FMT, CH, POW2, GS128, 3>(v, x, c, M, s, sh, tiles, grid);
-    default: return launch_mt<FMT, CH, POW2, GS128, 4>(v, x, c, M, s, sh, tiles, grid);
+    case 1: return launch_mt<FMT, CH, POW2, GSV, 1>(v, x, c, M, s, sh, tiles, grid);
+    case 2: return launch_mt<FMT, CH, POW2, GSV, 2>(v, x, c, M, s, sh, tiles, grid);
+    case 3: return launch_mt<FMT, CH, POW2, GSV, 3>(v, x, c, M, s, sh, tiles, grid);
+    default: return launch_mt<FMT, CH, POW2, GSV, 4>(v, x, c, M, s, sh, tiles, grid);
   }
 }
 
@@ -312,16 +347,24 @@ hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
                       int tiles, int T) {
   const bool pow2 = !v.mx && (v.gs & (v.gs - 1)) == 0;
   const int sh = pow2 ? __builtin_ctz((unsigned)v.gs) : 0;
-  // the 8-byte scale loads of the gs = 128 form need the scale array 8-byte aligned
-  const bool gs128 = !v.mx && v.gs == 128 && ((uintptr_t)v.scales & 7) == 0;
-  if (v.K == 4096) {
-    if (gs128) return launch_ch<FMT, 4, true, true>(v, x, c, M, s, sh, tiles, T);
-    return pow2 ? launch_ch<FMT, 4, true, false>(v, x, c, M, s, sh, tiles, T)
-                : launch_ch<FMT, 4, false, false>(v, x, c, M, s, sh, tiles, T);
+  // the vector loads of the scales (and of two zero-point words) need aligned arrays
+  int gsv = 0;
+  if (!v.mx && ((uintptr_t)v.scales & 15) == 0 && (v.symmetric || ((uintptr_t)v.zeros & 7) == 0))
+    gsv = v.gs == 128 ? 1 : v.gs == 64 ? 2 : v.gs == 32 ? 3 : 0;
+#define W4_GO(CHV)                                                                          \
+  switch (gsv) {                                                                            \
+    case 1: return launch_ch<FMT, CHV, true, 1>(v, x, c, M, s, sh, tiles, T);               \
+    case 2: return launch_ch<FMT, CHV, true, 2>(v, x, c, M, s, sh, tiles, T);               \
+    case 3: return launch_ch<FMT, CHV, true, 3>(v, x, c, M, s, sh, tiles, T);               \
+    default:                                                                                \
+      return pow2 ? launch_ch<FMT, CHV, true, 0>(v, x, c, M, s, sh, tiles, T)               \
+                  : launch_ch<FMT, CHV, false, 0>(v, x, c, M, s, sh, tiles, T);             \
   }
-  if (gs128) return launch_ch<FMT, 2, true, true>(v, x, c, M, s, sh, tiles, T);
-  return pow2 ? launch_ch<FMT, 2, true, false>(v, x, c, M, s, sh, tiles, T)
-              : launch_ch<FMT, 2, false, false>(v, x, c, M, s, sh, tiles, T);
+  if (v.K == 4096) {
+    W4_GO(4)
+  }
+  W4_GO(2)
+#undef W4_GO
 }
 
 // Compute units of the current device (per-device cache); 0 on error.
@@ -353,7 +396,7 @@ int decode_resident_tiles(const WView& v, const w4_half* x, const w4_half* c, in
   if (T > 4) T = 4;
   // the one combination that does not fit the register file: four tiles, four row
   // tiles, zero-points and per-chunk scale loads
-  if (T == 4 && M > 32 && !v.mx && !v.symmetric && v.gs != 128) T = 3;
+  if (T == 4 && M > 32 && !v.mx && !v.symmetric && v.gs != 128 && v.gs != 64 && v.gs != 32) T = 3;
   return T;
 }
 

@@ -312,117 +312,6 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void mfma_decode_kernel(
   }
 }
 
-// Unrolled form of the kernel above for the common decode shapes: M <= 16,
-// K = 1024 * CH (one round: wave w owns k in [128 CH w, 128 CH (w + 1))), whole
-// row tiles, one group per lane slice, no hook.  No bounds logic at all, so few
-// instructions stand between the start of a wave and its requests.
-template <int FMT, int CH, bool POW2>
-__global__ __launch_bounds__(DEC_WAVES * 64) void mfma_decode_unrolled_kernel(
-    const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
-    const int gs_shift) {
-  constexpr bool MX = FMT == 2;
-  constexpr int K = 1024 * CH, WPR = K / 8;
-  __shared__ f4 red[DEC_WAVES][64];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int r = lane & 15, b = lane >> 4;
-  const int n0 = blockIdx.x * 16;
-  const int kw = wave * (128 * CH) + 32 * b;  // first k of this lane
-  const size_t n = (size_t)(n0 + r);
-  const uint16_t* xr = x + (size_t)min(r, M - 1) * K + kw;
-  const uint32_t* qr = p.q + n * WPR + (kw >> 3);
-
-  // Activations are requested in two halves that share registers, so that enough
-  // workgroups fit on a CU for the whole grid to be resident at once.
-  constexpr int HALF = CH / 2;
-  u4 xv[HALF][4], qw[CH];
-  uint32_t sc[CH], zw[CH], zsh[CH];
-#pragma unroll
-  for (int i = 0; i < HALF; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) xv[i][j] = *(const u4*)(xr + 128 * i + 8 * j);
-#pragma unroll
-  for (int i = 0; i < CH; ++i) {
-    const int k = kw + 128 * i;
-    const int g = MX ? (k >> 5) : POW2 ? (k >> gs_shift) : k / p.gs;
-    zsh[i] = 4u * (uint32_t)(g & 7);
-    if (MX) {
-      sc[i] = ((const uint8_t*)p.scales)[n * p.B + g];
-    } else {
-      sc[i] = ((const uint16_t*)p.scales)[n * p.G + g];
-      if (FMT == 1) zw[i] = p.zeros[n * words(p.G) + (g >> 3)];
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < CH; ++i) qw[i] = __builtin_nontemporal_load((const u4*)(qr + 16 * i));
-
-  f4 acc = f4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    if (half == 1) {
-      __builtin_amdgcn_sched_barrier(0);  // the second half reuses the registers of the first
-#pragma unroll
-      for (int i = 0; i < HALF; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) xv[i][j] = *(const u4*)(xr + 128 * (HALF + i) + 8 * j);
-    }
-#pragma unroll
-    for (int ii = 0; ii < HALF; ++ii) {
-      const int i = half * HALF + ii;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        h2 d[4], nat[4];
-        if (MX) {
-          dq_mx(qw[i][j], mx_scale(sc[i]), nat);
-        } else {
-          const int z = FMT == 1 ? (int)((zw[i] >> zsh[i]) & 0xFu) : 8;
-          dq_w4(qw[i][j], w4_group((uint16_t)sc[i], z), d);
-          to_natural(d, nat);
-        }
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(pack_h8(nat), __builtin_bit_cast(h8, xv[ii][j]),
-                                                     acc, 0, 0, 0);
-      }
-    }
-  }
-  red[wave][lane] = acc;
-  __syncthreads();
-  if (wave == 0) {
-    f4 s = red[0][lane];
-#pragma unroll
-    for (int w = 1; w < DEC_WAVES; ++w) s += red[w][lane];
-    if (r < M) {  // lane: activation row r, weight rows n0 + 4 b .. + 3
-      uint16_t hv[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const _Float16 h = (_Float16)s[i];
-        hv[i] = __builtin_bit_cast(uint16_t, h);
-      }
-      *(u2*)(c + (size_t)r * p.N + n0 + 4 * b) =
-          u2{hv[0] | ((uint32_t)hv[1] << 16), hv[2] | ((uint32_t)hv[3] << 16)};
-    }
-  }
-}
-
-template <int FMT>
-static bool try_decode_unrolled(const WView& v, const w4_half* x, w4_half* c, int M,
-                                hipStream_t s, w4_half* w_out, hipError_t* err) {
-  if (w_out || M > 16 || v.N % 16 || ((uintptr_t)c & 7)) return false;
-  if (!v.mx && v.gs % 32) return false;
-  if (v.K != 2048 && v.K != 4096) return false;
-  const bool pow2 = !v.mx && (v.gs & (v.gs - 1)) == 0;
-  const int sh = pow2 ? __builtin_ctz((unsigned)v.gs) : 0;
-  const unsigned grid = (unsigned)(v.N / 16);
-#define W4_GO(CH, P2) \
-  mfma_decode_unrolled_kernel<FMT, CH, P2><<<grid, DEC_WAVES * 64, 0, s>>>(v, x, c, M, sh)
-  if (v.K == 4096) {
-    if (pow2) W4_GO(4, true); else W4_GO(4, false);
-  } else {
-    if (pow2) W4_GO(2, true); else W4_GO(2, false);
-  }
-#undef W4_GO
-  *err = hipGetLastError();
-  return true;
-}
-
 // One chunk per wave and round, one row tile per workgroup: the fastest of the
 // (NT, CH) combinations measured for M <= 16 (N = 4096 .. 14336, K = 4096 .. 11008).
 template <int FMT, int MT>
@@ -1010,11 +899,6 @@ static hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M
     const bool resident = wvec && decode_resident_applies(v, x, c, M);
     if (resident && w_out == nullptr) return launch_decode_resident(v, x, c, M, s);
     const bool ksplit = M <= 8 || (M <= 16 && v.N < 8192) || resident;
-    if (ksplit && wvec &&
-        (MX ? try_decode_unrolled<2>(v, x, c, M, s, w_out, &terr)
-            : v.symmetric ? try_decode_unrolled<0>(v, x, c, M, s, w_out, &terr)
-                          : try_decode_unrolled<1>(v, x, c, M, s, w_out, &terr)))
-      return terr;
     if (ksplit) {
       if (MX) return launch_decode<2>(v, x, c, M, s, w_out, wvec);
       return v.symmetric ? launch_decode<0>(v, x, c, M, s, w_out, wvec)

@@ -54,7 +54,9 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         (17, 4128, 4096, 128), (32, 8208, 2048, 64), (33, 4144, 4096, 32), (64, 12304, 2048, 128),
         (50, 4128, 2048, 96),
         # more than four tiles per compute unit: four per workgroup, more workgroups than units
-        (8, 16416, 2048, 128)]
+        (8, 16416, 2048, 128),
+        # 65 <= M <= 256: two to four passes of that kernel over the weights (grid.y)
+        (65, 4128, 2048, 128), (128, 2048, 4096, 64), (100, 96, 2048, 32), (250, 2048, 4096, 128)]
 TOL, CROSS = 1e-3, 2e-3  # rel L2 vs the FP64 oracle; between two gated paths
 
 

@@ -69,6 +69,7 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, b = lane >> 4;
   const int kw = wave * (128 * CH) + 32 * b;  // first k of this lane
+  const int m0 = (int)blockIdx.y * (16 * MT);  // grid.y walks the activation rows 16 MT at a time
 
   // rows of W this lane reads, per tile
   size_t nrow[T];
@@ -183,7 +184,7 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
       for (int cc = 0; cc < CP; ++cc)
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
-          const int r16 = 4 * rq + (lane >> 4), row = 16 * mt + r16;
+          const int r16 = 4 * rq + (lane >> 4), row = m0 + 16 * mt + r16;
           const uint32_t off = (uint32_t)min(row, M - 1) * (uint32_t)(K * 2) +
                                (uint32_t)(ph * CP + cc) * 256u + (uint32_t)(((lane & 15) ^ r16) * 16);
           const uint32_t dst = region + (uint32_t)((mt * CP + cc) * 4 + rq) * 1024u;
@@ -286,7 +287,7 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
     f4 s = red[e * 64 + lane];
 #pragma unroll
     for (int w = 1; w < DR_WAVES; ++w) s += red[(w * E + e) * 64 + lane];
-    const int m = 16 * mt + r;
+    const int m = m0 + 16 * mt + r;
     if (m < M) {  // lane: activation row m, weight rows 16 tile + 4 b .. + 3
       uint16_t hv[4];
 #pragma unroll
@@ -318,7 +319,8 @@ hipError_t launch_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStre
     if (dev >= 0 && dev < 64) granted[dev] = true;
   }
   mfma_decode_resident_kernel<FMT, CH, POW2, GSV, T, MT>
-      <<<grid, DR_THREADS, lds_bytes, s>>>(v, x, c, M, sh, tiles);
+      <<<dim3(grid, (unsigned)((M + 16 * MT - 1) / (16 * MT))), DR_THREADS, lds_bytes, s>>>(v, x, c, M, sh,
+                                                                                          tiles);
   return hipGetLastError();
 }
 
@@ -379,15 +381,21 @@ int device_cus() {
   return n;
 }
 
-// M <= 64, K = 2048 or 4096, whole 16-row tiles, a lane's 32-k slice inside one
-// group, 16-byte aligned operands.  Returns the tiles per workgroup, 0 if the
-// shape is not this kernel's.  (One tile per workgroup shares nothing, but the
-// coalesced fetch of x alone is worth it: N = K = 4096, M = 64: 22 -> 9 us.)
+// K = 2048 or 4096, whole 16-row tiles, a lane's 32-k slice inside one group,
+// 16-byte aligned operands, and M <= 64 -- or up to 256 rows in passes of 64
+// (grid.y) as long as the passes together stay under what the large-M kernel
+// takes, whose workgroups walk all of K alone (about 44 us at K = 4096 whatever M;
+// a pass here measured 8.6 / 13.7 / 16.5 us at N = 4096 / 11008 / 14336).  Returns
+// the tiles per workgroup, 0 if the shape is not this kernel's.
 int decode_resident_tiles(const WView& v, const w4_half* x, const w4_half* c, int M) {
-  if (M > 64 || M < 1 || v.N % 16 || (v.K != 2048 && v.K != 4096)) return 0;
+  if (M > 256 || M < 1 || v.N % 16 || (v.K != 2048 && v.K != 4096)) return 0;
   if (!v.mx && v.gs % 32) return 0;
   if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)c & 7)) return 0;
   if (v.mx && ((uintptr_t)v.scales & 15)) return 0;  // a slice's scale bytes are one vector load
+  if (M > 64) {
+    const double passes = (M + 63) / 64, pass_us = 5.0 + v.N / 1235.0;
+    if (passes * pass_us >= (v.K == 4096 ? 44.0 : 26.0)) return 0;
+  }
   const int cus = device_cus();
   if (cus < 1) return 0;
   // tiles per workgroup: enough that one workgroup per compute unit covers N, at

@@ -884,20 +884,23 @@ template <int MX>
 static hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M,
                              hipStream_t s, w4_half* w_out) {
   hipError_t terr = hipSuccess;
-  if (try_tile_dma(v, x, c, M, s, w_out, &terr)) return terr;
-  if (try_tile<MX>(v, x, c, M, s, w_out, &terr)) return terr;
+  // Shapes of the kernel that fetches the activations once per workgroup (M <= 256):
+  // hooked calls take the K-split kernel, which adds in the same order.
+  const bool wvec = (v.K % 32 == 0) && (((uintptr_t)v.q) & 15) == 0;
+  const bool resident = wvec && decode_resident_applies(v, x, c, M) &&
+                        (w_out == nullptr || ((uintptr_t)w_out & 15) == 0);
+  if (resident && w_out == nullptr) return launch_decode_resident(v, x, c, M, s);
+  if (!resident) {
+    if (try_tile_dma(v, x, c, M, s, w_out, &terr)) return terr;
+    if (try_tile<MX>(v, x, c, M, s, w_out, &terr)) return terr;
+  }
   // Rows of packed words are 16-byte aligned when K % 32 == 0 (one dwordx4 per lane
   // slice); K % 8 == 0 still gives whole words and 16-byte aligned activation rows.
-  const bool wvec = (v.K % 32 == 0) && (((uintptr_t)v.q) & 15) == 0;
   const bool aligned = (v.K % 8 == 0) && (((uintptr_t)x) & 15) == 0 &&
                        (w_out == nullptr || ((uintptr_t)w_out & 15) == 0);
   if (aligned) {
     // Measured on N = 4096 .. 14336, K = 4096 .. 11008: the K-split kernel wins for
     // M <= 16 unless N is large enough to give the streaming kernel a full grid.
-    // Shapes of the kernel that shares the activations among several tiles (M <= 64):
-    // hooked calls take the K-split kernel, which adds in the same order.
-    const bool resident = wvec && decode_resident_applies(v, x, c, M);
-    if (resident && w_out == nullptr) return launch_decode_resident(v, x, c, M, s);
     const bool ksplit = M <= 8 || (M <= 16 && v.N < 8192) || resident;
     if (ksplit) {
       if (MX) return launch_decode<2>(v, x, c, M, s, w_out, wvec);

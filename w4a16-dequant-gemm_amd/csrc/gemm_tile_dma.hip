@@ -30,15 +30,15 @@ namespace {
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
-constexpr int TD_TN = 256, TD_TM = 128;  // rows of W x rows of X per workgroup
+constexpr int TD_TN = 256;  // rows of W per workgroup; rows of X: the TM template parameter (128 or 64)
 constexpr int TD_WAVES = 4, TD_THREADS = 64 * TD_WAVES;  // a wave: 64 rows of W x all 128 of X
 constexpr int TD_STAGES = 3;
-constexpr int TD_W_BYTES = TD_TN * 64, TD_X_BYTES = TD_TM * 256;
-constexpr int TD_TILE = TD_W_BYTES + TD_X_BYTES;   // 48 KB
-constexpr int TD_STAGE = TD_TILE + 3 * TD_TN * 4;  // + two scale dwords and a zero-point word per W row
+constexpr int TD_W_BYTES = TD_TN * 64;
+// a stage: the W tile, TM rows of X, two scale dwords and a zero-point word per W row
+constexpr int td_tile(int tm) { return TD_W_BYTES + tm * 256; }
+constexpr int td_stage(int tm) { return td_tile(tm) + 3 * TD_TN * 4; }
 constexpr int TD_WI = TD_W_BYTES / 1024 / TD_WAVES;  // 1 KB load instructions of W per wave: 4
-constexpr int TD_XI = TD_X_BYTES / 1024 / TD_WAVES;  // of X: 8
-constexpr int TD_LDS = TD_STAGES * TD_STAGE;
+constexpr int td_lds_bytes(int tm) { return TD_STAGES * td_stage(tm); }
 
 // s_waitcnt vmcnt(N) alone (gfx9 encoding: vmcnt in [3:0] and [15:14])
 constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
@@ -85,13 +85,19 @@ __device__ __forceinline__ h8 expand_word(uint32_t w, h2 cneg, h2 s2, uint32_t m
 // lie in a 128-k stage: 0 one group (gs a multiple of 128), 1 two (gs = 64), 2 four
 // (gs = 32, and the 32-blocks of MXFP4).  A lane's share of a 64-k half is 32
 // consecutive k, so even then it has one scale per half.  G: scales per row.
-template <int FMT, int GSM, bool HOOK>
+// TM: rows of X per workgroup, 128 or 64 (a wave: 64 rows of W x all TM of X).  The
+// smaller tile halves a workgroup's walk over K when the grid of the larger one
+// would leave most of the chip idle.
+template <int FMT, int GSM, bool HOOK, int TM>
 __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
     const uint32_t* __restrict__ wq, const void* __restrict__ scales,
     const uint32_t* __restrict__ zeros, const w4_half* __restrict__ x, w4_half* __restrict__ c,
     w4_half* __restrict__ w_out, int N, int K, int G, int gs, int M, int tiles_n, int tiles_m) {
   constexpr bool ASYM = FMT == 1, MX = FMT == 2;
   constexpr int NSC = (!MX && GSM == 2) ? 2 : 1;           // scale dwords per row and stage
+  constexpr int TD_TM = TM, MJ = TM / 32;                  // 32-row tiles of X per wave
+  constexpr int TD_TILE = td_tile(TM), TD_STAGE = td_stage(TM);
+  constexpr int TD_XI = TM * 256 / 1024 / TD_WAVES;        // 1 KB load instructions of X per wave
   constexpr int LOADS = TD_WI + TD_XI + NSC + (ASYM ? 1 : 0);  // load instructions per wave and stage
   const int t = threadIdx.x, lane = t & 63;
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // in an SGPR: LDS addresses go to M0
@@ -188,7 +194,7 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   asm volatile("" : "+s"(mask));   // opaque: otherwise they come back as literals of two
   asm volatile("" : "+v"(magic));  // separate instructions
 
-  u4 xv[2][4];            // X operands of the step in hand and of the next: [m tile]
+  u4 xv[2][MJ];           // X operands of the step in hand and of the next: [m tile]
   u4 wv[2][2];            // packed words of the two 64-k halves: [half][n tile], word = step % 4
   h8 av[2][2];            // expanded W operands of the step in hand and of the next
   uint32_t sc[2][NSC], zw[2];  // the stage's scale dwords and zero-point word per n tile
@@ -209,7 +215,7 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   auto read_x = [&](u4* dst, uint32_t buf, int u) {  // step u = half u/4, MFMA u%4
     const uint8_t* p = td_lds + (buf + xoff[u]);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) dst[j] = *(const u4*)(p + j * 8192);
+    for (int j = 0; j < MJ; ++j) dst[j] = *(const u4*)(p + j * 8192);
   };
   auto read_w = [&](u4* dst, uint32_t buf, int s2) {
     const uint8_t* p = td_lds + (buf + woff[s2]);
@@ -266,11 +272,11 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
     }
   };
 
-  f16v acc[2][4];
+  f16v acc[2][MJ];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < MJ; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
@@ -318,29 +324,36 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < MJ; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
               av[u & 1][i], __builtin_bit_cast(h8, xv[u & 1][j]), acc[i][j], 0, 0, 0);
       // LDS reads first, then the expansion spread evenly under the MFMAs: a wave
       // can issue about six vector instructions in the shadow of one MFMA
+      constexpr int NM = 2 * MJ;  // MFMAs of a step
       if (u == 7) {
-        // the words to expand have only just been asked for: three MFMAs cover that
-        __builtin_amdgcn_sched_group_barrier(0x100, 6 + 2 * NSC + (ASYM ? 2 : 0), 0);
+        // the words to expand have only just been asked for: the first MFMAs cover that
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 + MJ + 2 * NSC + (ASYM ? 2 : 0), 0);
 #pragma unroll
-        for (int k = 0; k < 3; ++k) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        for (int k = 0; k < NM / 2 - 1; ++k) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
 #pragma unroll
-        for (int k = 0; k < 5; ++k) {
-          __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
+        for (int k = 0; k < NM / 2 + 1; ++k) {
+          if (MJ == 4) __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
+          else __builtin_amdgcn_sched_group_barrier(0x002, 16, 0);
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         }
       } else {
-        if (u == 0) __builtin_amdgcn_sched_group_barrier(0x100, 6, 0);
-        else __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+        if (u == 0) __builtin_amdgcn_sched_group_barrier(0x100, MJ + 2, 0);
+        else __builtin_amdgcn_sched_group_barrier(0x100, MJ, 0);
 #pragma unroll
-        for (int k = 0; k < 8; ++k) {
+        for (int k = 0; k < NM; ++k) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          if (u == 0) __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
-          else __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+          if (MJ == 4) {
+            if (u == 0) __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
+            else __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+          } else {
+            if (u == 0) __builtin_amdgcn_sched_group_barrier(0x002, 12, 0);
+            else __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
+          }
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -362,7 +375,7 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
     __syncthreads();  // no wave reads a stage buffer any more, no load is landing in one
     uint8_t* mine = td_lds + wave * (TD_TM * PITCH);
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < MJ; ++j)
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -382,7 +395,7 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
     return;
   }
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < MJ; ++j) {
     const int m = m0 + j * 32 + r;
     if (m >= M) continue;
 #pragma unroll
@@ -407,39 +420,42 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   }
 }
 
-template <int FMT, int GSM, bool HOOK>
+template <int FMT, int GSM, bool HOOK, int TM>
 hipError_t launch(const WView& v, const w4_half* x, w4_half* c, w4_half* w_out, int M,
                   hipStream_t s, int tiles_n, int tiles_m) {
+  constexpr int TD_LDS = td_lds_bytes(TM);
   // more than 64 KB of LDS has to be granted per device, once
   static bool granted[64] = {};
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
   if (dev < 0 || dev >= 64 || !granted[dev]) {
-    const hipError_t e = hipFuncSetAttribute((const void*)w4_tile_dma_kernel<FMT, GSM, HOOK>,
+    const hipError_t e = hipFuncSetAttribute((const void*)w4_tile_dma_kernel<FMT, GSM, HOOK, TM>,
                                              hipFuncAttributeMaxDynamicSharedMemorySize, TD_LDS);
     if (e != hipSuccess) return e;
     if (dev >= 0 && dev < 64) granted[dev] = true;
   }
-  w4_tile_dma_kernel<FMT, GSM, HOOK>
+  w4_tile_dma_kernel<FMT, GSM, HOOK, TM>
       <<<dim3((unsigned)(tiles_n * tiles_m)), dim3(TD_THREADS), TD_LDS, s>>>(
           v.q, v.scales, v.zeros, x, c, w_out, v.N, v.K, v.mx ? v.B : v.G, v.gs, M, tiles_n,
           tiles_m);
   return hipGetLastError();
 }
 
+// tm_rows: 128 or 64 rows of X per workgroup (the hooked kernels exist for 128 only)
 template <int FMT, int GSM>
 hipError_t launch_hook(const WView& v, const w4_half* x, w4_half* c, w4_half* w_out, int M,
-                       hipStream_t s, int tn, int tm) {
-  return w_out ? launch<FMT, GSM, true>(v, x, c, w_out, M, s, tn, tm)
-               : launch<FMT, GSM, false>(v, x, c, nullptr, M, s, tn, tm);
+                       hipStream_t s, int tn, int tm, int tm_rows) {
+  if (w_out) return launch<FMT, GSM, true, 128>(v, x, c, w_out, M, s, tn, tm);
+  return tm_rows == 64 ? launch<FMT, GSM, false, 64>(v, x, c, nullptr, M, s, tn, tm)
+                       : launch<FMT, GSM, false, 128>(v, x, c, nullptr, M, s, tn, tm);
 }
 
 template <int FMT>
 hipError_t launch_gsm(int gsm, const WView& v, const w4_half* x, w4_half* c, w4_half* w_out,
-                      int M, hipStream_t s, int tn, int tm) {
-  if (gsm == 0) return launch_hook<FMT, 0>(v, x, c, w_out, M, s, tn, tm);
-  if (gsm == 1) return launch_hook<FMT, 1>(v, x, c, w_out, M, s, tn, tm);
-  return launch_hook<FMT, 2>(v, x, c, w_out, M, s, tn, tm);
+                      int M, hipStream_t s, int tn, int tm, int tm_rows) {
+  if (gsm == 0) return launch_hook<FMT, 0>(v, x, c, w_out, M, s, tn, tm, tm_rows);
+  if (gsm == 1) return launch_hook<FMT, 1>(v, x, c, w_out, M, s, tn, tm, tm_rows);
+  return launch_hook<FMT, 2>(v, x, c, w_out, M, s, tn, tm, tm_rows);
 }
 
 }  // namespace
@@ -458,8 +474,14 @@ bool try_tile_dma(const WView& v, const w4_half* x, w4_half* c, int M, hipStream
     else if (v.gs == 64) gsm = 1;
     else if (v.gs != 32) return false;
   }
-  const long long tiles_n = (v.N + TD_TN - 1) / TD_TN, tiles_m = (M + TD_TM - 1) / TD_TM;
-  if (M < 96 || tiles_n * tiles_m < 8 || tiles_n * tiles_m > 0x7FFFFFFFLL) return false;
+  // 64-row tiles of X when that grid still fits the chip's 256 compute units in one
+  // round: half the walk over K per workgroup (hooked and unhooked calls add in the
+  // same order either way: a wave's sums do not depend on how many rows of X its
+  // workgroup holds)
+  const long long tiles_n = (v.N + TD_TN - 1) / TD_TN;
+  const int tm_rows = (w_out == nullptr && tiles_n * ((M + 63) / 64) <= 256) ? 64 : 128;
+  const long long tiles_m = (M + tm_rows - 1) / tm_rows;
+  if (M < 96 || tiles_n * ((M + 127) / 128) < 8 || tiles_n * tiles_m > 0x7FFFFFFFLL) return false;
   if ((long long)v.N * v.K / 2 >= (1LL << 32) || (long long)M * v.K * 2 >= (1LL << 32)) return false;
   // one FP16 scale per stage: the dword around it must lie inside the array
   if (gsm == 0 && (((long long)v.N * v.G) & 1)) return false;
@@ -467,9 +489,9 @@ bool try_tile_dma(const WView& v, const w4_half* x, w4_half* c, int M, hipStream
   if (!v.mx && !v.symmetric && (v.zeros == nullptr || ((uintptr_t)v.zeros & 3))) return false;
   if (w_out && ((uintptr_t)w_out & 15)) return false;
   const int tn = (int)tiles_n, tm = (int)tiles_m;
-  if (v.mx) *err = launch_hook<2, 2>(v, x, c, w_out, M, s, tn, tm);
-  else if (v.symmetric) *err = launch_gsm<0>(gsm, v, x, c, w_out, M, s, tn, tm);
-  else *err = launch_gsm<1>(gsm, v, x, c, w_out, M, s, tn, tm);
+  if (v.mx) *err = launch_hook<2, 2>(v, x, c, w_out, M, s, tn, tm, tm_rows);
+  else if (v.symmetric) *err = launch_gsm<0>(gsm, v, x, c, w_out, M, s, tn, tm, tm_rows);
+  else *err = launch_gsm<1>(gsm, v, x, c, w_out, M, s, tn, tm, tm_rows);
   return true;
 }
 

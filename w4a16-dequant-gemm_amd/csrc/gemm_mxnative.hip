@@ -501,6 +501,35 @@ __global__ __launch_bounds__(DM_THREADS) void mxn_tile_dma_kernel(
   }
   __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // nothing may still be writing LDS at exit
 
+  // A lane holds, of each 32 x 32 tile, n = 8 q + 4 h + e for m = tile row r.  Whole
+  // tiles go through LDS (free by now) so that every store instruction writes eight
+  // whole 128-byte lines instead of 16 bytes of each of 32: a wave lays its 64 (m)
+  // x 64 (n) block out in rows of 144 bytes and reads it back 16 bytes a lane.
+  const bool whole = m0 + TL_TM <= M && n0 + TL_TN <= N && (N & 7) == 0 && ((uintptr_t)c & 15) == 0;
+  if (whole) {
+    constexpr int PITCH = 144;
+    __syncthreads();  // no wave reads a stage buffer any more, no load is landing in one
+    uint8_t* mine = dm_lds + wave * (64 * PITCH);
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int i = 0; i < DM_NT; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          h4 out;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) out[e] = (_Float16)acc[i][j][4 * q + e];
+          *(h4*)(mine + (j * 32 + r) * PITCH + i * 64 + q * 16 + h * 8) = out;
+        }
+    w4_half* cw = c + (size_t)(m0 + wm * 64) * N + n0 + wn * (32 * DM_NT);
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int row = it * 8 + (lane >> 3), piece = lane & 7;
+      const u4 v = *(const u4*)(mine + row * PITCH + piece * 16);
+      *(u4*)(cw + (size_t)row * N + piece * 8) = v;
+    }
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int m = m0 + wm * 64 + j * 32 + r;

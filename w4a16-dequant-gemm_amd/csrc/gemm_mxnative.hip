@@ -556,6 +556,226 @@ __global__ __launch_bounds__(DM_THREADS) void mxn_tile_dma_kernel(
   }
 }
 
+// The same tile for packed-MXFP4 activations with one wave per SIMD: 4 waves, each
+// 64 rows of W x all 128 rows of X (2 x 4 tiles of 32x32x64).  A stage (256 k) is
+// four steps of 64 k; during the eight MFMAs of a step the wave reads the next
+// step's six operands from LDS, and the fifteen load instructions of a stage are
+// issued four per step instead of in a row (a wave has one instruction stream to
+// keep its SIMD's matrix pipe fed).  Stage d + 2 is requested from the last step of
+// stage d - 1, when the barrier there has freed its buffer.
+constexpr int D4_WAVES = 4, D4_THREADS = 64 * D4_WAVES;
+constexpr int D4_TILE = DM_W_BYTES + TL_TM * 128;           // 48 KB
+constexpr int D4_STAGE = D4_TILE + 2 * TL_ROWS * 4;         // + two scale dwords per row
+constexpr int D4_STAGES = 3;
+constexpr int D4_WI = DM_W_BYTES / 1024 / D4_WAVES;         // 8
+constexpr int D4_XI = TL_TM * 128 / 1024 / D4_WAVES;        // 4
+constexpr int D4_LOADS = D4_WI + D4_XI + 3;                 // + two dwords of W scales, one of X scales
+
+__global__ __launch_bounds__(D4_THREADS) void mxn_tile4_kernel(
+    const uint32_t* __restrict__ wq, const uint8_t* __restrict__ ws,
+    const uint32_t* __restrict__ xq, const uint8_t* __restrict__ xs, w4_half* __restrict__ c,
+    int N, int K, int B, int M, int tiles_n, int tiles_m) {
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // in an SGPR: LDS addresses go to M0
+  const int r = lane & 31, h = lane >> 5;
+  int L = blockIdx.x;
+  const int total = tiles_n * tiles_m;
+  if (total % 8 == 0) L = (L & 7) * (total >> 3) + (L >> 3);  // a run of the tile order per XCD
+  const int n0 = (L / tiles_m) * TL_TN, m0 = (L % tiles_m) * TL_TM;
+  const int wk = K >> 3;
+
+  // what this lane fetches: row l/8 of an 8-row block, swizzled 16-byte piece
+  const int row8 = lane >> 3;
+  uint32_t wo[D4_WI], xo[D4_XI];
+#pragma unroll
+  for (int i = 0; i < D4_WI; ++i) {
+    const int R = (wave + D4_WAVES * i) * 8 + row8, n = n0 + R;
+    wo[i] = ((uint32_t)(n < N ? n : N - 1) * (uint32_t)wk) * 4u + (((lane & 7) ^ ((R >> 1) & 7)) * 16);
+  }
+#pragma unroll
+  for (int i = 0; i < D4_XI; ++i) {
+    const int R = (wave + D4_WAVES * i) * 8 + row8, m = m0 + R;
+    xo[i] = ((uint32_t)(m < M ? m : M - 1) * (uint32_t)wk) * 4u + (((lane & 7) ^ ((R >> 1) & 7)) * 16);
+  }
+  // scale dwords: W rows 64 wave + lane, both 128-k halves; X rows 64 (wave & 1) + lane, half wave / 2
+  const int swrow = n0 + wave * 64 + lane, sxrow = m0 + (wave & 1) * 64 + lane;
+  const uint32_t swo = (uint32_t)(swrow < N ? swrow : N - 1) * (uint32_t)B;
+  const uint32_t sxo = (uint32_t)(sxrow < M ? sxrow : M - 1) * (uint32_t)B + (uint32_t)(wave >> 1) * 4u;
+  const char* wqb = (const char*)wq;
+  const char* xqb = (const char*)xq;
+  const int stages = K >> 8;
+  auto dma16 = [](const void* gbase, uint32_t goff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(goff), "s"(gbase), "s"(lds_addr)
+                 : "memory", "m0");
+  };
+  auto dma4 = [](const void* gbase, uint32_t goff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1"
+                 :
+                 : "v"(goff), "s"(gbase), "s"(lds_addr)
+                 : "memory", "m0");
+  };
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr)dm_lds;
+  auto request_part = [&](int d, uint32_t buf, int part) {  // buf: byte offset of the stage's buffer
+    const uint32_t dd = (uint32_t)(d < stages ? d : stages - 1);  // past the end: valid, never used
+    const uint32_t st = lds0 + buf;
+    if (part < D4_WI) {
+      dma16(wqb + dd * 128u, wo[part], st + (wave + D4_WAVES * part) * 1024);
+    } else if (part < D4_WI + D4_XI) {
+      const int i = part - D4_WI;
+      dma16(xqb + dd * 128u, xo[i], st + DM_W_BYTES + (wave + D4_WAVES * i) * 1024);
+    } else if (part < D4_WI + D4_XI + 2) {
+      const int s2 = part - D4_WI - D4_XI;
+      dma4(ws + dd * 8u + s2 * 4u, swo, st + D4_TILE + s2 * (TL_ROWS * 4) + wave * 256);
+    } else {
+      dma4(xs + dd * 8u, sxo, st + D4_TILE + (wave >> 1) * (TL_ROWS * 4) + TL_TN * 4 + (wave & 1) * 256);
+    }
+  };
+  auto request = [&](int d, uint32_t buf) {
+#pragma unroll
+    for (int part = 0; part < D4_LOADS; ++part) request_part(d, buf, part);
+  };
+
+  // where this lane reads inside a stage buffer: piece 2 u + h of its row in W tile
+  // 0 and X tile 0 (the next tile is 4 KB further), its rows' scale dwords
+  auto at = [](int R, int p) { return (R >> 3) * 1024 + ((R & 7) * 8 + (p ^ ((R >> 1) & 7))) * 16; };
+  uint32_t woff[4], xoff[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    woff[u] = at(wave * 64 + r, 2 * u + h);
+    xoff[u] = DM_W_BYTES + at(r, 2 * u + h);
+  }
+  const uint32_t saoff = D4_TILE + (wave * 64 + r) * 4, sboff = D4_TILE + (TL_TN + r) * 4;
+
+  u4 wv[2][2], xv[2][4];          // operands of the step in hand and of the next
+  uint32_t sa[2][2], sb[2][4];    // scale dwords of the 128-k half in hand and of the next
+  auto read_ops = [&](int slot, uint32_t buf, int u) {
+    const uint8_t* pw = dm_lds + (buf + woff[u]);
+    const uint8_t* px = dm_lds + (buf + xoff[u]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) wv[slot][i] = *(const u4*)(pw + i * 4096);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) xv[slot][j] = *(const u4*)(px + j * 4096);
+  };
+  auto read_scales = [&](int slot, uint32_t buf, int s2) {
+    const uint8_t* pa = dm_lds + (buf + saoff + s2 * (TL_ROWS * 4));
+    const uint8_t* pb = dm_lds + (buf + sboff + s2 * (TL_ROWS * 4));
+#pragma unroll
+    for (int i = 0; i < 2; ++i) sa[slot][i] = *(const uint32_t*)(pa + i * 128);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sb[slot][j] = *(const uint32_t*)(pb + j * 128);
+  };
+
+  f16v acc[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // b0, b1, b2: byte offsets of the buffers of stages d, d + 1, d + 2
+  uint32_t b0 = 0, b1 = D4_STAGE, b2 = 2 * D4_STAGE;
+  request(0, b0);
+  request(1, b1);
+#pragma unroll
+  for (int part = 0; part < 4; ++part) request_part(2, b2, part);
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm(D4_LOADS + 4));  // stage 0 has landed
+  __syncthreads();
+  read_ops(0, b0, 0);
+  read_scales(0, b0, 0);
+#pragma unroll 1
+  for (int d = 0; d < stages; ++d) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      // step u = half u / 2, MFMA u % 2 of it; operand slot u % 2, scale slot (u / 2) % 2
+      if (u == 3) {
+        // every LDS read of stage d has been issued: once all waves are here its buffer
+        // can take stage d + 3, and stage d + 1 has landed for everyone
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(D4_LOADS));
+        __syncthreads();
+#pragma unroll
+        for (int part = 0; part < 4; ++part) request_part(d + 3, b0, part);
+        __builtin_amdgcn_sched_barrier(0);
+        read_ops(0, b1, 0);
+        read_scales(0, b1, 0);
+      } else {
+#pragma unroll
+        for (int part = 4 * u + 4; part < 4 * u + 8; ++part)
+          if (part < D4_LOADS) request_part(d + 2, b2, part);
+        __builtin_amdgcn_sched_barrier(0);
+        read_ops((u + 1) & 1, b0, u + 1);
+        if (u == 1) read_scales(1, b0, 1);
+      }
+      const int sh = 16 * (u & 1) + 8 * h, ss = u >> 1;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = mfma_fp4_32(wv[u & 1][i], sa[ss][i] >> sh, xv[u & 1][j], sb[ss][j] >> sh, acc[i][j]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    const uint32_t first = b0;
+    b0 = b1;
+    b1 = b2;
+    b2 = first;
+  }
+  __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // nothing may still be writing LDS at exit
+
+  // lane: m = tile row r, n = 8 q + 4 h + e of each 32 x 32 tile; whole tiles leave
+  // through LDS as full 128-byte lines
+  const bool whole = m0 + TL_TM <= M && n0 + TL_TN <= N && (N & 7) == 0 && ((uintptr_t)c & 15) == 0;
+  if (whole) {
+    constexpr int PITCH = 144;
+    __syncthreads();  // no wave reads a stage buffer any more, no load is landing in one
+    uint8_t* mine = dm_lds + wave * (TL_TM * PITCH);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          h4 out;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) out[e] = (_Float16)acc[i][j][4 * q + e];
+          *(h4*)(mine + (j * 32 + r) * PITCH + i * 64 + q * 16 + h * 8) = out;
+        }
+    w4_half* cw = c + (size_t)m0 * N + n0 + wave * 64;
+#pragma unroll
+    for (int it = 0; it < TL_TM / 8; ++it) {
+      const int row = it * 8 + (lane >> 3), piece = lane & 7;
+      const u4 v = *(const u4*)(mine + row * PITCH + piece * 16);
+      *(u4*)(cw + (size_t)row * N + piece * 8) = v;
+    }
+    return;
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int m = m0 + j * 32 + r;
+    if (m >= M) continue;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int nn = n0 + wave * 64 + i * 32 + 8 * q + 4 * h;
+        w4_half* dst = c + (size_t)m * N + nn;
+        if (nn + 3 < N && ((uintptr_t)dst & 7) == 0) {
+          h4 out;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) out[e] = (_Float16)acc[i][j][4 * q + e];
+          *(h4*)dst = out;
+        } else {
+          const int left = N - nn;
+          if (left > 0) dst[0] = __builtin_bit_cast(uint16_t, (_Float16)acc[i][j][4 * q + 0]);
+          if (left > 1) dst[1] = __builtin_bit_cast(uint16_t, (_Float16)acc[i][j][4 * q + 1]);
+          if (left > 2) dst[2] = __builtin_bit_cast(uint16_t, (_Float16)acc[i][j][4 * q + 2]);
+          if (left > 3) dst[3] = __builtin_bit_cast(uint16_t, (_Float16)acc[i][j][4 * q + 3]);
+        }
+      }
+  }
+}
+
 // Worth it once the tile grid covers a good part of the chip; below that the
 // skinny kernel's grid.y walk is faster (measured at K = 4096: N = 4096, M = 256
 // -> 32 tiles 37 us here, 23 us there; M = 512 -> 64 tiles 31 us here; N = 14336,
@@ -573,19 +793,31 @@ hipError_t launch_tile(const w4_packed_mx_view& w, const void* xq, const uint8_t
                        w4_half* c, hipStream_t s) {
   const int tiles_n = (w.N + TL_TN - 1) / TL_TN, tiles_m = (M + TL_TM - 1) / TL_TM;
   if ((long long)tiles_n * tiles_m > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
-  constexpr int lds_bytes = Dm<XF8>::STAGES * Dm<XF8>::STAGE;
   // more than 64 KB of LDS has to be granted per device, once
   static bool granted[64] = {};
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
-  if (dev < 0 || dev >= 64 || !granted[dev]) {
-    const hipError_t e = hipFuncSetAttribute((const void*)mxn_tile_dma_kernel<XF8>,
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64) granted[dev] = true;
+  const bool grant = dev < 0 || dev >= 64 || !granted[dev];
+  if constexpr (XF8) {
+    constexpr int lds_bytes = Dm<true>::STAGES * Dm<true>::STAGE;
+    if (grant) {
+      const hipError_t e = hipFuncSetAttribute((const void*)mxn_tile_dma_kernel<true>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+      if (e != hipSuccess) return e;
+    }
+    mxn_tile_dma_kernel<true><<<dim3((unsigned)(tiles_n * tiles_m)), dim3(DM_THREADS), lds_bytes, s>>>(
+        w.q, w.scales, (const uint32_t*)xq, xs, c, w.N, w.K, w.B, M, tiles_n, tiles_m);
+  } else {
+    constexpr int lds_bytes = D4_STAGES * D4_STAGE;
+    if (grant) {
+      const hipError_t e = hipFuncSetAttribute((const void*)mxn_tile4_kernel,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+      if (e != hipSuccess) return e;
+    }
+    mxn_tile4_kernel<<<dim3((unsigned)(tiles_n * tiles_m)), dim3(D4_THREADS), lds_bytes, s>>>(
+        w.q, w.scales, (const uint32_t*)xq, xs, c, w.N, w.K, w.B, M, tiles_n, tiles_m);
   }
-  mxn_tile_dma_kernel<XF8><<<dim3((unsigned)(tiles_n * tiles_m)), dim3(DM_THREADS), lds_bytes, s>>>(
-      w.q, w.scales, (const uint32_t*)xq, xs, c, w.N, w.K, w.B, M, tiles_n, tiles_m);
+  if (dev >= 0 && dev < 64) granted[dev] = true;
   return hipGetLastError();
 }
 

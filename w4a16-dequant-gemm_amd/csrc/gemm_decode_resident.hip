@@ -61,14 +61,23 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
     const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
     const int gs_shift, const int tiles) {
   constexpr bool MX = FMT == 2;
-  constexpr int K = 1024 * CH, WPR = K / 8;
+  // K: any multiple of 128 with ceil(K / 128 / 8) == CH; wave w owns the 128-k chunks
+  // [CH w, CH (w + 1)) that exist (the last waves may own fewer: chunks past the end
+  // are fetched from a clamped address and meet zero activations)
+  const int K = p.K, WPR = K >> 3, nchunks = K >> 7;
+  constexpr bool EXACT = CH == 2 || CH == 4;  // K = 1024 CH by the launcher: every chunk exists
   constexpr int CP = (4 / MT) < CH ? (4 / MT) : CH;  // chunks per phase
-  constexpr int PH = CH / CP;                         // phases
+  constexpr int PH = (CH + CP - 1) / CP;              // phases (the last may be partial)
   constexpr int XBYTES = MT * CP * 4096;              // the wave's LDS region
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 15, b = lane >> 4;
   const int kw = wave * (128 * CH) + 32 * b;  // first k of this lane
+  // chunk i of this wave, clamped to the last one of the row
+  auto chunk_k = [&](int i) {
+    const int cidx = wave * CH + i;
+    return (EXACT || cidx < nchunks) ? kw + 128 * i : (nchunks - 1) * 128 + 32 * b;
+  };
   const int m0 = (int)blockIdx.y * (16 * MT);  // grid.y walks the activation rows 16 MT at a time
 
   // rows of W this lane reads, per tile
@@ -84,23 +93,26 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
   // loads and a per-lane pick, and their zero-points sit in one or two words;
   // MXFP4's CH bytes are 4 apart in 4 CH consecutive ones.  Other group sizes load
   // them one by one.
-  constexpr bool VEC = MX || GSV != 0;
+  constexpr bool VEC = (MX && EXACT) || GSV != 0;
   constexpr int PER = MX ? 4 : GSV == 1 ? 1 : GSV == 2 ? 2 : 4;  // groups per 128-k chunk
   uint32_t sc[T][CH], zw[T][CH];
   int gidx[CH];
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
-    const int k = kw + 128 * i;
+    const int k = chunk_k(i);
     gidx[i] = MX ? (k >> 5) : GSV ? (k >> (8 - GSV)) : POW2 ? (k >> gs_shift) : k / p.gs;
   }
   u4 qw[T][CH];
   auto load_tile = [&](int t) {
-    const uint32_t* qr = p.q + nrow[t] * WPR + (kw >> 3);
+    const uint32_t* qr = p.q + nrow[t] * WPR;
 #pragma unroll
-    for (int i = 0; i < CH; ++i) qw[t][i] = __builtin_nontemporal_load((const u4*)(qr + 16 * i));
+    for (int i = 0; i < CH; ++i) qw[t][i] = __builtin_nontemporal_load((const u4*)(qr + (chunk_k(i) >> 3)));
   };
   auto load_scales = [&](int t) {
-    if constexpr (MX) {  // bytes 4 CH wave .. + 4 CH - 1 of the row; this lane's are b + 4 i
+    if constexpr (MX && !EXACT) {
+#pragma unroll
+      for (int i = 0; i < CH; ++i) sc[t][i] = ((const uint8_t*)p.scales)[nrow[t] * p.B + gidx[i]];
+    } else if constexpr (MX) {  // bytes 4 CH wave .. + 4 CH - 1 of the row; this lane's are b + 4 i
       const uint8_t* sp = (const uint8_t*)p.scales + nrow[t] * p.B + wave * (4 * CH);
       uint32_t w[CH];
       if constexpr (CH == 4) {
@@ -168,6 +180,7 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
   };
   // vector loads the scales of all tiles take (between the first x request and the wait)
   constexpr int SVEC = MX ? 1 : (PER * CH / 2 + 3) / 4;  // vector loads of a tile's scales
+  static_assert(EXACT || GSV == 0, "vector scale loads assume K = 1024 CH");
   constexpr int SLOADS = T * (VEC ? SVEC + ((FMT == 1) ? 1 : 0) : ((FMT == 1) ? 2 * CH : CH));
   load_tile(0);
 
@@ -176,7 +189,7 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
   // four, 16-byte piece (l%16) ^ (row % 16) of the chunk's 256 bytes.  Rows past M
   // repeat row M - 1 (their columns of the product are never stored).
   const uint32_t region = (uint32_t)(uintptr_t)(lds_ptr)dr_lds + (uint32_t)wave * XBYTES;
-  const char* xb = (const char*)x + (size_t)wave * (256 * CH);
+  const char* xb = (const char*)x;
   auto request_x = [&](int ph) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -184,9 +197,12 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
       for (int cc = 0; cc < CP; ++cc)
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
+          if (ph * CP + cc >= CH) continue;
           const int r16 = 4 * rq + (lane >> 4), row = m0 + 16 * mt + r16;
+          const int cidx = wave * CH + ph * CP + cc;  // a chunk past the end repeats the last one
           const uint32_t off = (uint32_t)min(row, M - 1) * (uint32_t)(K * 2) +
-                               (uint32_t)(ph * CP + cc) * 256u + (uint32_t)(((lane & 15) ^ r16) * 16);
+                               (uint32_t)((EXACT || cidx < nchunks) ? cidx : nchunks - 1) * 256u +
+                               (uint32_t)(((lane & 15) ^ r16) * 16);
           const uint32_t dst = region + (uint32_t)((mt * CP + cc) * 4 + rq) * 1024u;
           asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
                        :
@@ -226,9 +242,12 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
 #pragma unroll
         for (int cc = 0; cc < CP; ++cc)
 #pragma unroll
-          for (int j = 0; j < 4; ++j)
+          for (int j = 0; j < 4; ++j) {
+            if (ph * CP + cc >= CH) continue;
             xv[mt][cc][j] = *(const u4*)(mine + ((mt * CP + cc) * 4 + (r >> 2)) * 1024 +
                                          ((r & 3) * 16 + ((4 * b + j) ^ r)) * 16);
+            if (!EXACT && wave * CH + ph * CP + cc >= nchunks) xv[mt][cc][j] = u4{0u, 0u, 0u, 0u};
+          }
     }
     if (ph + 1 < PH) {
       // the region is free once these reads have returned: ask for the next phase now
@@ -241,6 +260,7 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
 #pragma unroll
       for (int cc = 0; cc < CP; ++cc) {
         const int i = ph * CP + cc;
+        if (i >= CH) continue;
         h2 cneg, s2;
         float sf = 0.f;
         if (MX) {
@@ -301,6 +321,17 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
   }
 }
 
+// Chunks of 128 k per wave for the K this kernel is built for, else 0: K = 2048 and
+// 4096 exactly, and any multiple of 128 whose eighth rounds up to 8, 11 or 14 chunks
+// (7296 .. 8192, 10368 .. 11264, 13440 .. 14336: the long sides of the usual MLP shapes).
+int resident_chunks(int K) {
+  if (K == 2048) return 2;
+  if (K == 4096) return 4;
+  if (K % 128) return 0;
+  const int per_wave = (K / 128 + DR_WAVES - 1) / DR_WAVES;
+  return (per_wave == 8 || per_wave == 11 || per_wave == 14) ? per_wave : 0;
+}
+
 template <int FMT, int CH, bool POW2, int GSV, int T, int MT>
 hipError_t launch_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
                     int tiles, unsigned grid) {
@@ -336,11 +367,15 @@ template <int FMT, int CH, bool POW2, int GSV>
 hipError_t launch_ch(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
                      int tiles, int T) {
   const unsigned grid = (unsigned)((tiles + T - 1) / T);
-  switch (T) {
-    case 1: return launch_mt<FMT, CH, POW2, GSV, 1>(v, x, c, M, s, sh, tiles, grid);
-    case 2: return launch_mt<FMT, CH, POW2, GSV, 2>(v, x, c, M, s, sh, tiles, grid);
-    case 3: return launch_mt<FMT, CH, POW2, GSV, 3>(v, x, c, M, s, sh, tiles, grid);
-    default: return launch_mt<FMT, CH, POW2, GSV, 4>(v, x, c, M, s, sh, tiles, grid);
+  if constexpr (CH > 4) {  // long K: one tile per workgroup (the codes of a tile fill the registers)
+    return launch_mt<FMT, CH, POW2, GSV, 1>(v, x, c, M, s, sh, tiles, grid);
+  } else {
+    switch (T) {
+      case 1: return launch_mt<FMT, CH, POW2, GSV, 1>(v, x, c, M, s, sh, tiles, grid);
+      case 2: return launch_mt<FMT, CH, POW2, GSV, 2>(v, x, c, M, s, sh, tiles, grid);
+      case 3: return launch_mt<FMT, CH, POW2, GSV, 3>(v, x, c, M, s, sh, tiles, grid);
+      default: return launch_mt<FMT, CH, POW2, GSV, 4>(v, x, c, M, s, sh, tiles, grid);
+    }
   }
 }
 
@@ -351,7 +386,8 @@ hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
   const int sh = pow2 ? __builtin_ctz((unsigned)v.gs) : 0;
   // the vector loads of the scales (and of two zero-point words) need aligned arrays
   int gsv = 0;
-  if (!v.mx && ((uintptr_t)v.scales & 15) == 0 && (v.symmetric || ((uintptr_t)v.zeros & 7) == 0))
+  if (!v.mx && (v.K == 2048 || v.K == 4096) && ((uintptr_t)v.scales & 15) == 0 &&
+      (v.symmetric || ((uintptr_t)v.zeros & 7) == 0))
     gsv = v.gs == 128 ? 1 : v.gs == 64 ? 2 : v.gs == 32 ? 3 : 0;
 #define W4_GO(CHV)                                                                          \
   switch (gsv) {                                                                            \
@@ -362,10 +398,18 @@ hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
       return pow2 ? launch_ch<FMT, CHV, true, 0>(v, x, c, M, s, sh, tiles, T)               \
                   : launch_ch<FMT, CHV, false, 0>(v, x, c, M, s, sh, tiles, T);             \
   }
-  if (v.K == 4096) {
-    W4_GO(4)
+#define W4_LONG(CHV)                                                                        \
+  return pow2 ? launch_ch<FMT, CHV, true, 0>(v, x, c, M, s, sh, tiles, T)                   \
+              : launch_ch<FMT, CHV, false, 0>(v, x, c, M, s, sh, tiles, T);
+  switch (resident_chunks(v.K)) {
+    case 2: W4_GO(2)
+    case 4: W4_GO(4)
+    case 8: W4_LONG(8)
+    case 11: W4_LONG(11)
+    case 14: W4_LONG(14)
+    default: return hipErrorInvalidValue;
   }
-  W4_GO(2)
+#undef W4_LONG
 #undef W4_GO
 }
 
@@ -381,20 +425,21 @@ int device_cus() {
   return n;
 }
 
-// K = 2048 or 4096, whole 16-row tiles, a lane's 32-k slice inside one group,
-// 16-byte aligned operands, and M <= 64 -- or up to 256 rows in passes of 64
+// A K this kernel is built for, whole 16-row tiles, a lane's 32-k slice inside one
+// group, 16-byte aligned operands, and M <= 64 -- or up to 256 rows in passes of 64
 // (grid.y) as long as the passes together stay under what the large-M kernel
 // takes, whose workgroups walk all of K alone (about 44 us at K = 4096 whatever M;
 // a pass here measured 8.6 / 13.7 / 16.5 us at N = 4096 / 11008 / 14336).  Returns
 // the tiles per workgroup, 0 if the shape is not this kernel's.
 int decode_resident_tiles(const WView& v, const w4_half* x, const w4_half* c, int M) {
-  if (M > 256 || M < 1 || v.N % 16 || (v.K != 2048 && v.K != 4096)) return 0;
+  if (M > 256 || M < 1 || v.N % 16 || resident_chunks(v.K) == 0) return 0;
   if (!v.mx && v.gs % 32) return 0;
   if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)c & 7)) return 0;
   if (v.mx && ((uintptr_t)v.scales & 15)) return 0;  // a slice's scale bytes are one vector load
   if (M > 64) {
     const double passes = (M + 63) / 64, pass_us = 5.0 + v.N / 1235.0;
-    if (passes * pass_us >= (v.K == 4096 ? 44.0 : 26.0)) return 0;
+    // both sides grow with K alike; at K = 2048 the fixed part of a pass weighs more
+    if (passes * pass_us >= (v.K == 2048 ? 35.6 : 44.0)) return 0;
   }
   const int cus = device_cus();
   if (cus < 1) return 0;
@@ -402,6 +447,7 @@ int decode_resident_tiles(const WView& v, const w4_half* x, const w4_half* c, in
   // most four (more workgroups than compute units beyond that)
   int T = (v.N / 16 + cus - 1) / cus;
   if (T > 4) T = 4;
+  if (resident_chunks(v.K) > 4) T = 1;
   // the one combination that does not fit the register file: four tiles, four row
   // tiles, zero-points and per-chunk scale loads
   if (T == 4 && M > 32 && !v.mx && !v.symmetric && v.gs != 128 && v.gs != 64 && v.gs != 32) T = 3;

@@ -55,8 +55,10 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         (50, 4128, 2048, 96),
         # more than four tiles per compute unit: four per workgroup, more workgroups than units
         (8, 16416, 2048, 128),
-        # 65 <= M <= 256: two to four passes of that kernel over the weights (grid.y)
+        # 65 <= M <= 256: two or three passes of that kernel over the weights (grid.y) while that is
+        # the cheaper way (four passes at N = 2048 are not: the tile kernel takes that one)
         (65, 4128, 2048, 128), (128, 2048, 4096, 64), (100, 96, 2048, 32), (250, 2048, 4096, 128),
+        (130, 512, 4096, 128),
         # long K (8, 11 and 14 chunks of 128 per wave; the last waves own fewer when K / 128 is no
         # multiple of 8: 86 chunks at K = 11008, 57 at K = 7296, 81 at K = 10368)
         (16, 256, 11008, 128), (64, 512, 14336, 64), (5, 128, 8192, 32), (33, 96, 7296, 128),

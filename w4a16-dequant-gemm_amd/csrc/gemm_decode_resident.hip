@@ -428,18 +428,19 @@ int device_cus() {
 // A K this kernel is built for, whole 16-row tiles, a lane's 32-k slice inside one
 // group, 16-byte aligned operands, and M <= 64 -- or up to 256 rows in passes of 64
 // (grid.y) as long as the passes together stay under what the large-M kernel
-// takes, whose workgroups walk all of K alone (about 44 us at K = 4096 whatever M;
-// a pass here measured 8.6 / 13.7 / 16.5 us at N = 4096 / 11008 / 14336).  Returns
-// the tiles per workgroup, 0 if the shape is not this kernel's.
+// takes, whose workgroups walk all of K alone.  Returns the tiles per workgroup, 0
+// if the shape is not this kernel's.
 int decode_resident_tiles(const WView& v, const w4_half* x, const w4_half* c, int M) {
   if (M > 256 || M < 1 || v.N % 16 || resident_chunks(v.K) == 0) return 0;
   if (!v.mx && v.gs % 32) return 0;
   if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)c & 7)) return 0;
   if (v.mx && ((uintptr_t)v.scales & 15)) return 0;  // a slice's scale bytes are one vector load
   if (M > 64) {
-    const double passes = (M + 63) / 64, pass_us = 5.0 + v.N / 1235.0;
-    // both sides grow with K alike; at K = 2048 the fixed part of a pass weighs more
-    if (passes * pass_us >= (v.K == 2048 ? 35.6 : 44.0)) return 0;
+    // measured at K = 4096: a pass here 8.6 / 13.7 / 16.5 us at N = 4096 / 11008 / 14336, the
+    // large-M kernel on its thinnest grids 25 / 37 / 41 us; both grow with K alike, the
+    // fixed part of a pass weighs more at K = 2048
+    const double passes = (M + 63) / 64, pass_us = 5.0 + v.N / 1235.0, tile_us = 18.0 + v.N / 590.0;
+    if (passes * pass_us >= tile_us * (v.K == 2048 ? 0.8 : 1.0)) return 0;
   }
   const int cus = device_cus();
   if (cus < 1) return 0;

@@ -30,15 +30,14 @@ namespace {
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
-constexpr int TD_TN = 256;  // rows of W per workgroup; rows of X: the TM template parameter (128 or 64)
+// rows of W (TN: 256 or 128) and of X (TM: 128 or 64) per workgroup are template parameters
 constexpr int TD_WAVES = 4, TD_THREADS = 64 * TD_WAVES;  // a wave: 64 rows of W x all 128 of X
 constexpr int TD_STAGES = 3;
-constexpr int TD_W_BYTES = TD_TN * 64;
-// a stage: the W tile, TM rows of X, two scale dwords and a zero-point word per W row
-constexpr int td_tile(int tm) { return TD_W_BYTES + tm * 256; }
-constexpr int td_stage(int tm) { return td_tile(tm) + 3 * TD_TN * 4; }
-constexpr int TD_WI = TD_W_BYTES / 1024 / TD_WAVES;  // 1 KB load instructions of W per wave: 4
-constexpr int td_lds_bytes(int tm) { return TD_STAGES * td_stage(tm); }
+// a stage: TN rows of W (64 bytes each), TM rows of X (256 bytes each), two scale dwords and a
+// zero-point word per W row
+constexpr int td_tile(int tm, int tn) { return tn * 64 + tm * 256; }
+constexpr int td_stage(int tm, int tn) { return td_tile(tm, tn) + 3 * tn * 4; }
+constexpr int td_lds_bytes(int tm, int tn) { return TD_STAGES * td_stage(tm, tn); }
 
 // s_waitcnt vmcnt(N) alone (gfx9 encoding: vmcnt in [3:0] and [15:14])
 constexpr int waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
@@ -88,7 +87,8 @@ __device__ __forceinline__ h8 expand_word(uint32_t w, h2 cneg, h2 s2, uint32_t m
 // TM: rows of X per workgroup, 128 or 64 (a wave: 64 rows of W x all TM of X).  The
 // smaller tile halves a workgroup's walk over K when the grid of the larger one
 // would leave most of the chip idle.
-template <int FMT, int GSM, bool HOOK, int TM>
+// TN: rows of W per workgroup, 256 or 128 (a wave: TN / 4 of them = NI tiles of 32).
+template <int FMT, int GSM, bool HOOK, int TM, int TN>
 __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
     const uint32_t* __restrict__ wq, const void* __restrict__ scales,
     const uint32_t* __restrict__ zeros, const w4_half* __restrict__ x, w4_half* __restrict__ c,
@@ -96,7 +96,10 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   constexpr bool ASYM = FMT == 1, MX = FMT == 2;
   constexpr int NSC = (!MX && GSM == 2) ? 2 : 1;           // scale dwords per row and stage
   constexpr int TD_TM = TM, MJ = TM / 32;                  // 32-row tiles of X per wave
-  constexpr int TD_TILE = td_tile(TM), TD_STAGE = td_stage(TM);
+  constexpr int TD_TN = TN, NI = TN / 128;                 // 32-row tiles of W per wave
+  constexpr int TD_W_BYTES = TN * 64;
+  constexpr int TD_WI = TD_W_BYTES / 1024 / TD_WAVES;      // 1 KB load instructions of W per wave
+  constexpr int TD_TILE = td_tile(TM, TN), TD_STAGE = td_stage(TM, TN);
   constexpr int TD_XI = TM * 256 / 1024 / TD_WAVES;        // 1 KB load instructions of X per wave
   constexpr int LOADS = TD_WI + TD_XI + NSC + (ASYM ? 1 : 0);  // load instructions per wave and stage
   const int t = threadIdx.x, lane = t & 63;
@@ -126,7 +129,10 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   }
   // per stage: the dword that holds the group scale of W row 64 wave + lane, and
   // (ASYM) that row's zero-point word
-  const uint32_t sn = (uint32_t)(n0 + wave * 64 + lane < N ? n0 + wave * 64 + lane : N - 1);
+  // (TN = 128: waves 2 and 3 repeat the fetches of waves 0 and 1, which keeps the count of
+  // load instructions the same for every wave)
+  const int srow = (NI == 2 ? wave : (wave & 1)) * 64 + lane;
+  const uint32_t sn = (uint32_t)(n0 + srow < N ? n0 + srow : N - 1);
   const uint32_t sc_base = sn * (uint32_t)G, zw_base = sn * (uint32_t)wg;
   const char* wqb = (const char*)wq;
   const char* xb = (const char*)x;
@@ -168,9 +174,10 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
       if (k < NSC) {
         const uint32_t off = MX ? sc_base + g : GSM == 0 ? ((sc_base + g) >> 1) * 4u
                                                         : (sc_base + g) * 2u + 4u * k;
-        dma4(scales, off, st + TD_TILE + k * (TD_TN * 4) + wave * 256);
+        dma4(scales, off, st + TD_TILE + k * (TD_TN * 4) + (NI == 2 ? wave : (wave & 1)) * 256);
       } else {
-        dma4(zeros, (zw_base + (g >> 3)) * 4u, st + TD_TILE + 2 * (TD_TN * 4) + wave * 256);
+        dma4(zeros, (zw_base + (g >> 3)) * 4u,
+             st + TD_TILE + 2 * (TD_TN * 4) + (NI == 2 ? wave : (wave & 1)) * 256);
       }
     }
   };
@@ -181,11 +188,11 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
 
   // this lane's rows of the two W tiles of its wave; the parity of their first
   // scale index says which half of the fetched dword is theirs
-  int wrow[2];
-  uint32_t par[2];
+  int wrow[NI];
+  uint32_t par[NI];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    wrow[i] = wave * 64 + i * 32 + r;
+  for (int i = 0; i < NI; ++i) {
+    wrow[i] = wave * (32 * NI) + i * 32 + r;
     const int n = n0 + wrow[i];
     par[i] = ((uint32_t)(n < N ? n : N - 1) * (uint32_t)G) & 1u;
   }
@@ -195,13 +202,13 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   asm volatile("" : "+v"(magic));  // separate instructions
 
   u4 xv[2][MJ];           // X operands of the step in hand and of the next: [m tile]
-  u4 wv[2][2];            // packed words of the two 64-k halves: [half][n tile], word = step % 4
-  h8 av[2][2];            // expanded W operands of the step in hand and of the next
-  uint32_t sc[2][NSC], zw[2];  // the stage's scale dwords and zero-point word per n tile
+  u4 wv[2][NI];           // packed words of the two 64-k halves: [half][n tile], word = step % 4
+  h8 av[2][NI];           // expanded W operands of the step in hand and of the next
+  uint32_t sc[NI][NSC], zw[NI];  // the stage's scale dwords and zero-point word per n tile
   // what expansion needs, per [half][n tile]: -(1024 + z), -(64 + z) and the scale in
   // both halves of a register (MXFP4: the scale as a float)
-  h2 cneg[2][2], s2v[2][2];
-  float sf[2][2];
+  h2 cneg[2][NI], s2v[2][NI];
+  float sf[2][NI];
   // Where this lane reads inside a stage buffer, worked out once: the X piece of
   // step u in m tile 0 (tile j is 8 KB further), its four words of half s2 in n tile
   // 0 (tile 1 is 2 KB further), its scale dword.  A read is then one add of the
@@ -220,12 +227,12 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   auto read_w = [&](u4* dst, uint32_t buf, int s2) {
     const uint8_t* p = td_lds + (buf + woff[s2]);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) dst[i] = *(const u4*)(p + i * 2048);
+    for (int i = 0; i < NI; ++i) dst[i] = *(const u4*)(p + i * 2048);
   };
   auto read_sc = [&](uint32_t buf) {
     const uint8_t* p = td_lds + (buf + scoff);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NI; ++i) {
 #pragma unroll
       for (int k = 0; k < NSC; ++k) sc[i][k] = *(const uint32_t*)(p + k * (TD_TN * 4) + i * 128);
       if (ASYM) zw[i] = *(const uint32_t*)(p + 2 * (TD_TN * 4) + i * 128);
@@ -235,7 +242,7 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
 #pragma unroll
     for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < NI; ++i) {
         if constexpr (MX) {  // block 4 d + 2 s2 + h of the row
           sf[s2][i] = mx_scale((sc[i][0] >> (8 * (2 * s2 + h))) & 0xFFu);
         } else {
@@ -258,7 +265,7 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   };
   auto expand = [&](h8* dst, int d, int u) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < NI; ++i) {
       if constexpr (MX) {
         h2 n4[4];
         dq_mx(wv[u >> 2][i][u & 3], sf[u >> 2][i], n4);
@@ -272,9 +279,9 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
     }
   };
 
-  f16v acc[2][MJ];
+  f16v acc[NI][MJ];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < NI; ++i)
 #pragma unroll
     for (int j = 0; j < MJ; ++j)
 #pragma unroll
@@ -322,38 +329,35 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
         expand(av[(u + 1) & 1], d, u + 1);
       }
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < NI; ++i)
 #pragma unroll
         for (int j = 0; j < MJ; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
               av[u & 1][i], __builtin_bit_cast(h8, xv[u & 1][j]), acc[i][j], 0, 0, 0);
       // LDS reads first, then the expansion spread evenly under the MFMAs: a wave
       // can issue about six vector instructions in the shadow of one MFMA
-      constexpr int NM = 2 * MJ;  // MFMAs of a step
+      constexpr int NM = NI * MJ;  // MFMAs of a step
+      // vector instructions of a step (16 per word, a few more), shared out over its MFMAs
+      constexpr int VPM = (16 * NI + 8 + NM - 1) / NM, VPM0 = VPM + 2;
+      constexpr int VPM7 = (16 * NI + 16 + NM / 2) / (NM / 2 + 1);
       if (u == 7) {
         // the words to expand have only just been asked for: the first MFMAs cover that
-        __builtin_amdgcn_sched_group_barrier(0x100, 2 + MJ + 2 * NSC + (ASYM ? 2 : 0), 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, NI + MJ + NI * NSC + (ASYM ? NI : 0), 0);
 #pragma unroll
         for (int k = 0; k < NM / 2 - 1; ++k) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
 #pragma unroll
         for (int k = 0; k < NM / 2 + 1; ++k) {
-          if (MJ == 4) __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
-          else __builtin_amdgcn_sched_group_barrier(0x002, 16, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, VPM7, 0);
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         }
       } else {
-        if (u == 0) __builtin_amdgcn_sched_group_barrier(0x100, MJ + 2, 0);
+        if (u == 0) __builtin_amdgcn_sched_group_barrier(0x100, MJ + NI, 0);
         else __builtin_amdgcn_sched_group_barrier(0x100, MJ, 0);
 #pragma unroll
         for (int k = 0; k < NM; ++k) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          if (MJ == 4) {
-            if (u == 0) __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);
-            else __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
-          } else {
-            if (u == 0) __builtin_amdgcn_sched_group_barrier(0x002, 12, 0);
-            else __builtin_amdgcn_sched_group_barrier(0x002, 10, 0);
-          }
+          if (u == 0) __builtin_amdgcn_sched_group_barrier(0x002, VPM0, 0);
+          else __builtin_amdgcn_sched_group_barrier(0x002, VPM, 0);
         }
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -371,13 +375,14 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   // x 64 (n) block out in rows of 144 bytes and reads it back 16 bytes a lane.
   const bool whole = m0 + TD_TM <= M && n0 + TD_TN <= N && (N & 7) == 0 && ((uintptr_t)c & 15) == 0;
   if (whole) {
-    constexpr int PITCH = 144;
+    constexpr int RB = 64 * NI, PITCH = RB + 16;  // bytes of a row of the wave's block, and its LDS pitch
+    constexpr int PP = RB / 16, ROWS = 64 / PP;   // 16-byte pieces per row, rows per store instruction
     __syncthreads();  // no wave reads a stage buffer any more, no load is landing in one
     uint8_t* mine = td_lds + wave * (TD_TM * PITCH);
 #pragma unroll
     for (int j = 0; j < MJ; ++j)
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < NI; ++i)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           h4 out;
@@ -385,10 +390,10 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
           for (int e = 0; e < 4; ++e) out[e] = (_Float16)acc[i][j][4 * q + e];
           *(h4*)(mine + (j * 32 + r) * PITCH + i * 64 + q * 16 + h * 8) = out;
         }
-    w4_half* cw = c + (size_t)m0 * N + n0 + wave * 64;
+    w4_half* cw = c + (size_t)m0 * N + n0 + wave * (32 * NI);
 #pragma unroll
-    for (int it = 0; it < TD_TM / 8; ++it) {
-      const int row = it * 8 + (lane >> 3), piece = lane & 7;
+    for (int it = 0; it < TD_TM / ROWS; ++it) {
+      const int row = it * ROWS + lane / PP, piece = lane % PP;
       const u4 v = *(const u4*)(mine + row * PITCH + piece * 16);
       *(u4*)(cw + (size_t)row * N + piece * 8) = v;
     }
@@ -399,10 +404,10 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
     const int m = m0 + j * 32 + r;
     if (m >= M) continue;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < NI; ++i)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int nn = n0 + wave * 64 + i * 32 + 8 * q + 4 * h;
+        const int nn = n0 + wave * (32 * NI) + i * 32 + 8 * q + 4 * h;
         w4_half* dst = c + (size_t)m * N + nn;
         if (nn + 3 < N && ((uintptr_t)dst & 7) == 0) {
           h4 out;
@@ -420,42 +425,44 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   }
 }
 
-template <int FMT, int GSM, bool HOOK, int TM>
+template <int FMT, int GSM, bool HOOK, int TM, int TN>
 hipError_t launch(const WView& v, const w4_half* x, w4_half* c, w4_half* w_out, int M,
                   hipStream_t s, int tiles_n, int tiles_m) {
-  constexpr int TD_LDS = td_lds_bytes(TM);
+  constexpr int TD_LDS = td_lds_bytes(TM, TN);
   // more than 64 KB of LDS has to be granted per device, once
   static bool granted[64] = {};
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
   if (dev < 0 || dev >= 64 || !granted[dev]) {
-    const hipError_t e = hipFuncSetAttribute((const void*)w4_tile_dma_kernel<FMT, GSM, HOOK, TM>,
+    const hipError_t e = hipFuncSetAttribute((const void*)w4_tile_dma_kernel<FMT, GSM, HOOK, TM, TN>,
                                              hipFuncAttributeMaxDynamicSharedMemorySize, TD_LDS);
     if (e != hipSuccess) return e;
     if (dev >= 0 && dev < 64) granted[dev] = true;
   }
-  w4_tile_dma_kernel<FMT, GSM, HOOK, TM>
+  w4_tile_dma_kernel<FMT, GSM, HOOK, TM, TN>
       <<<dim3((unsigned)(tiles_n * tiles_m)), dim3(TD_THREADS), TD_LDS, s>>>(
           v.q, v.scales, v.zeros, x, c, w_out, v.N, v.K, v.mx ? v.B : v.G, v.gs, M, tiles_n,
           tiles_m);
   return hipGetLastError();
 }
 
-// tm_rows: 128 or 64 rows of X per workgroup (the hooked kernels exist for 128 only)
+// shape: 0 = 128 x 256 (rows of X x rows of W), 1 = 64 x 256, 2 = 64 x 128 (the hooked
+// kernels exist for the first only)
 template <int FMT, int GSM>
 hipError_t launch_hook(const WView& v, const w4_half* x, w4_half* c, w4_half* w_out, int M,
-                       hipStream_t s, int tn, int tm, int tm_rows) {
-  if (w_out) return launch<FMT, GSM, true, 128>(v, x, c, w_out, M, s, tn, tm);
-  return tm_rows == 64 ? launch<FMT, GSM, false, 64>(v, x, c, nullptr, M, s, tn, tm)
-                       : launch<FMT, GSM, false, 128>(v, x, c, nullptr, M, s, tn, tm);
+                       hipStream_t s, int tn, int tm, int shape) {
+  if (w_out) return launch<FMT, GSM, true, 128, 256>(v, x, c, w_out, M, s, tn, tm);
+  if (shape == 2) return launch<FMT, GSM, false, 64, 128>(v, x, c, nullptr, M, s, tn, tm);
+  if (shape == 1) return launch<FMT, GSM, false, 64, 256>(v, x, c, nullptr, M, s, tn, tm);
+  return launch<FMT, GSM, false, 128, 256>(v, x, c, nullptr, M, s, tn, tm);
 }
 
 template <int FMT>
 hipError_t launch_gsm(int gsm, const WView& v, const w4_half* x, w4_half* c, w4_half* w_out,
-                      int M, hipStream_t s, int tn, int tm, int tm_rows) {
-  if (gsm == 0) return launch_hook<FMT, 0>(v, x, c, w_out, M, s, tn, tm, tm_rows);
-  if (gsm == 1) return launch_hook<FMT, 1>(v, x, c, w_out, M, s, tn, tm, tm_rows);
-  return launch_hook<FMT, 2>(v, x, c, w_out, M, s, tn, tm, tm_rows);
+                      int M, hipStream_t s, int tn, int tm, int shape) {
+  if (gsm == 0) return launch_hook<FMT, 0>(v, x, c, w_out, M, s, tn, tm, shape);
+  if (gsm == 1) return launch_hook<FMT, 1>(v, x, c, w_out, M, s, tn, tm, shape);
+  return launch_hook<FMT, 2>(v, x, c, w_out, M, s, tn, tm, shape);
 }
 
 }  // namespace
@@ -474,14 +481,21 @@ bool try_tile_dma(const WView& v, const w4_half* x, w4_half* c, int M, hipStream
     else if (v.gs == 64) gsm = 1;
     else if (v.gs != 32) return false;
   }
-  // 64-row tiles of X when that grid still fits the chip's 256 compute units in one
-  // round: half the walk over K per workgroup (hooked and unhooked calls add in the
-  // same order either way: a wave's sums do not depend on how many rows of X its
-  // workgroup holds)
-  const long long tiles_n = (v.N + TD_TN - 1) / TD_TN;
-  const int tm_rows = (w_out == nullptr && tiles_n * ((M + 63) / 64) <= 256) ? 64 : 128;
-  const long long tiles_m = (M + tm_rows - 1) / tm_rows;
-  if (M < 96 || tiles_n * ((M + 127) / 128) < 8 || tiles_n * tiles_m > 0x7FFFFFFFLL) return false;
+  // The smallest of the three tile shapes whose grid still fits the chip's 256 compute
+  // units in one round (two workgroups of the smallest fit a unit's LDS): a smaller
+  // tile shortens a workgroup's walk over K -- N = K = 4096, M = 512: 45.6 us with
+  // 128 x 256 tiles, 38.1 with 64 x 256, 27.0 with 64 x 128.  (Hooked
+  // and unhooked calls add in the same order whatever the shape: a wave's sums do
+  // not depend on how many rows its workgroup holds.)
+  const long long n256 = (v.N + 255) / 256, n128 = (v.N + 127) / 128;
+  const long long m128 = (M + 127) / 128, m64 = (M + 63) / 64;
+  int shape = 0;
+  if (w_out == nullptr) {
+    if (n128 * m64 <= 512 && !(gsm == 2 && !v.mx && !v.symmetric)) shape = 2;  // (three scale planes: no)
+    else if (n256 * m64 <= 256) shape = 1;
+  }
+  const long long tiles_n = shape == 2 ? n128 : n256, tiles_m = shape == 0 ? m128 : m64;
+  if (M < 96 || n256 * m128 < 8 || tiles_n * tiles_m > 0x7FFFFFFFLL) return false;
   if ((long long)v.N * v.K / 2 >= (1LL << 32) || (long long)M * v.K * 2 >= (1LL << 32)) return false;
   // one FP16 scale per stage: the dword around it must lie inside the array
   if (gsm == 0 && (((long long)v.N * v.G) & 1)) return false;
@@ -489,9 +503,9 @@ bool try_tile_dma(const WView& v, const w4_half* x, w4_half* c, int M, hipStream
   if (!v.mx && !v.symmetric && (v.zeros == nullptr || ((uintptr_t)v.zeros & 3))) return false;
   if (w_out && ((uintptr_t)w_out & 15)) return false;
   const int tn = (int)tiles_n, tm = (int)tiles_m;
-  if (v.mx) *err = launch_hook<2, 2>(v, x, c, w_out, M, s, tn, tm, tm_rows);
-  else if (v.symmetric) *err = launch_gsm<0>(gsm, v, x, c, w_out, M, s, tn, tm, tm_rows);
-  else *err = launch_gsm<1>(gsm, v, x, c, w_out, M, s, tn, tm, tm_rows);
+  if (v.mx) *err = launch_hook<2, 2>(v, x, c, w_out, M, s, tn, tm, shape);
+  else if (v.symmetric) *err = launch_gsm<0>(gsm, v, x, c, w_out, M, s, tn, tm, shape);
+  else *err = launch_gsm<1>(gsm, v, x, c, w_out, M, s, tn, tm, shape);
   return true;
 }
 

@@ -446,12 +446,13 @@ hipError_t launch(const WView& v, const w4_half* x, w4_half* c, w4_half* w_out, 
   return hipGetLastError();
 }
 
-// shape: 0 = 128 x 256 (rows of X x rows of W), 1 = 64 x 256, 2 = 64 x 128 (the hooked
-// kernels exist for the first only)
+// shape: 0 = 128 x 256 (rows of X x rows of W), 1 = 64 x 256, 2 = 64 x 128, 3 = 128 x 128
+// (the hooked kernels exist for the first only)
 template <int FMT, int GSM>
 hipError_t launch_hook(const WView& v, const w4_half* x, w4_half* c, w4_half* w_out, int M,
                        hipStream_t s, int tn, int tm, int shape) {
   if (w_out) return launch<FMT, GSM, true, 128, 256>(v, x, c, w_out, M, s, tn, tm);
+  if (shape == 3) return launch<FMT, GSM, false, 128, 128>(v, x, c, nullptr, M, s, tn, tm);
   if (shape == 2) return launch<FMT, GSM, false, 64, 128>(v, x, c, nullptr, M, s, tn, tm);
   if (shape == 1) return launch<FMT, GSM, false, 64, 256>(v, x, c, nullptr, M, s, tn, tm);
   return launch<FMT, GSM, false, 128, 256>(v, x, c, nullptr, M, s, tn, tm);
@@ -481,20 +482,23 @@ bool try_tile_dma(const WView& v, const w4_half* x, w4_half* c, int M, hipStream
     else if (v.gs == 64) gsm = 1;
     else if (v.gs != 32) return false;
   }
-  // The smallest of the three tile shapes whose grid still fits the chip's 256 compute
-  // units in one round (two workgroups of the smallest fit a unit's LDS): a smaller
-  // tile shortens a workgroup's walk over K -- N = K = 4096, M = 512: 45.6 us with
-  // 128 x 256 tiles, 38.1 with 64 x 256, 27.0 with 64 x 128.  (Hooked
+  // The smallest of the tile shapes whose grid still fits the chip's 256 compute
+  // units in one round: a smaller tile shortens a workgroup's walk over K -- N = K =
+  // 4096, M = 512: 45.6 us with 128 x 256 tiles, 38.1 with 64 x 256, 27.0 with 64 x 128.
+  // (Hooked
   // and unhooked calls add in the same order whatever the shape: a wave's sums do
   // not depend on how many rows its workgroup holds.)
   const long long n256 = (v.N + 255) / 256, n128 = (v.N + 127) / 128;
   const long long m128 = (M + 127) / 128, m64 = (M + 63) / 64;
   int shape = 0;
   if (w_out == nullptr) {
-    if (n128 * m64 <= 512 && !(gsm == 2 && !v.mx && !v.symmetric)) shape = 2;  // (three scale planes: no)
+    const bool planes3 = gsm == 2 && !v.mx && !v.symmetric;  // needs 256 rows of W per workgroup
+    if (!planes3 && n128 * m64 <= 256) shape = 2;
+    else if (!planes3 && n128 * m128 <= 256) shape = 3;
     else if (n256 * m64 <= 256) shape = 1;
   }
-  const long long tiles_n = shape == 2 ? n128 : n256, tiles_m = shape == 0 ? m128 : m64;
+  const long long tiles_n = (shape == 2 || shape == 3) ? n128 : n256;
+  const long long tiles_m = (shape == 0 || shape == 3) ? m128 : m64;
   if (M < 96 || n256 * m128 < 8 || tiles_n * tiles_m > 0x7FFFFFFFLL) return false;
   if ((long long)v.N * v.K / 2 >= (1LL << 32) || (long long)M * v.K * 2 >= (1LL << 32)) return false;
   // one FP16 scale per stage: the dword around it must lie inside the array

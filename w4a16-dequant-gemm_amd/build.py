@@ -23,6 +23,12 @@ FLAGS = [
     "-Wno-inline-asm",
 ]
 
+# Per-file additions.  The flash-decode kernel rescales its accumulators with
+# vector-ALU multiplies between matrix instructions: with the accumulators in
+# the AGPR half of the register file the compiler copies all 36 of them across
+# every loop edge, so keep its MFMA results in ordinary VGPRs.
+EXTRA_FLAGS = {"flash_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
 
 def _stale():
     if not os.path.exists(LIB):
@@ -41,7 +47,7 @@ def build(force=False, verbose=True):
     for src in SOURCES:
         obj = os.path.join(PKG, "lib", "obj", src.replace(".hip", ".o"))
         objs.append(obj)
-        cmd = ["hipcc", *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = ["hipcc", *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
         procs.append((src, subprocess.Popen(cmd, stderr=subprocess.PIPE, text=True)))
     for src, p in procs:
         _, err = p.communicate()

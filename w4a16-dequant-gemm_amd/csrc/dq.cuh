@@ -62,6 +62,14 @@ __device__ __forceinline__ W4Group w4_group(uint16_t scale_bits, int z) {
   return g;
 }
 
+__device__ __forceinline__ W4Group w4_group(_Float16 scale, int z) {
+  W4Group g;
+  g.s = splat(scale);
+  g.zlo = splat_bits(0x6400u | (uint32_t)z);
+  g.zhi = splat_bits(0x5400u | ((uint32_t)z << 4));
+  return g;
+}
+
 // (a & mask) | orv in one VOP3 instruction (the compiler otherwise emits an
 // AND and an OR with literal operands).
 __device__ __forceinline__ uint32_t and_or(uint32_t a, uint32_t mask, uint32_t orv) {

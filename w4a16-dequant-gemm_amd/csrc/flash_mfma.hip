@@ -25,6 +25,8 @@
 // and merge their (m, l, O) through LDS in wave order, so a split yields one
 // partial and every sum has a fixed order: paged and contiguous caches give the
 // same bytes.
+#include <type_traits>
+
 #include "dq.cuh"
 #include "kernels.h"
 
@@ -32,7 +34,7 @@ namespace w4k {
 
 constexpr int FM_TILE = 32;   // positions per wave tile
 constexpr int FM_WAVES = 4;
-constexpr int FM_DEPTH = 2;   // tiles in flight per wave
+constexpr int FM_DEPTH = 3;   // ring slots per wave: one tile computed, two in flight
 constexpr int FM_HEADS = 16;  // query heads per pass
 
 // What one lane fetches for one tile, before expansion.
@@ -42,8 +44,10 @@ struct TileRaw;
 template <int NC>
 struct TileRaw<KIND_W4, NC> {
   uint32_t k[2][NC];
-  uint32_t ks[2], kz[2];
-  uint32_t v[8], vs[8], vz[8];
+  _Float16 ks[2];
+  uint32_t kz[2];
+  uint32_t v[8], vz[8];
+  _Float16 vs[8];
 };
 template <int NC>
 struct TileRaw<KIND_F16, NC> {
@@ -53,9 +57,9 @@ struct TileRaw<KIND_F16, NC> {
 template <int NC>
 struct TileRaw<KIND_F8, NC> {
   u2 k[2][NC];
-  uint32_t ks[2];
+  _Float16 ks[2];
   u2 v[8];
-  uint32_t vs[8];
+  _Float16 vs[8];
 };
 
 // Position of element e (0..7) of an expanded 8-element block: register and half.
@@ -96,6 +100,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
   const int split = blockIdx.y, slab = blockIdx.x, nsplit = gridDim.y;  // slabs on x: no 65535 bound
   const int nh = min(FM_HEADS, a.group - qh0);
   const float inv_sqrt_d = 1.0f / sqrtf((float)FM_D);
+  const float exp_scale = inv_sqrt_d * 1.44269504088896340736f;  // exp(x / sqrt(D)) = exp2(x * exp_scale)
   const int G = a.G, wg = words(a.G);
   const int vb = c16 & (NB - 1);                               // this lane's V element block
   const int gk = KIND == KIND_F16 ? 0 : (8 * NC * q4) / a.gs;  // group of this lane's K elements
@@ -109,8 +114,18 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
   } else {
     rows0 = (long long)slab * a.S;
   }
-  uint32_t slab_sk = 0, slab_sv = 0;
-  if (KIND == KIND_F8 && a.scale_mode == 1) slab_sk = a.s_k[slab], slab_sv = a.s_v[slab];
+  // Scales stay 16-bit values from the load to the packed operand: widened to 32
+  // bits they would be masked right behind the load, which makes the wave wait
+  // for a prefetch it has just issued.
+  auto as_half = [](uint16_t b) { return __builtin_bit_cast(_Float16, b); };
+  // Used where a prefetched scale is consumed: the empty statement keeps the
+  // compiler from packing the scales of the next tile right behind their loads.
+  auto at_use = [](_Float16 x) {
+    asm("" : "+v"(x));
+    return x;
+  };
+  _Float16 slab_sk = 0, slab_sv = 0;
+  if (KIND == KIND_F8 && a.scale_mode == 1) slab_sk = as_half(a.s_k[slab]), slab_sv = as_half(a.s_v[slab]);
 
   const int s0 = split * split_len;
   const int s1 = min(a.S, s0 + split_len);
@@ -143,6 +158,91 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     return rows0 + (long long)bt[pg] * a.page + (t - pg * a.page);
   };
 
+  // ---- whole tiles (all 32 positions below s1; with pages, each half of 16 in
+  // one page): buffer loads whose wave-uniform part (slab base in the
+  // descriptor, tile row in the scalar offset) never touches the vector ALU.
+  // A lane adds only the constant byte offsets below.
+  constexpr int ROWB = KIND == KIND_W4 ? DH / 2 : KIND == KIND_F8 ? DH : 2 * DH;  // bytes per cache row
+  constexpr int VBB = ROWB / NB;                                                  // bytes per V block
+  const long long slab_rows = PAGED ? a.pool_rows : a.S;
+  // offsets are 32-bit: larger slabs take the general fetch for every tile
+  const bool whole_ok = PAGED != 2 && slab_rows * ROWB < (1ll << 31) && slab_rows * G * 2 < (1ll << 31);
+  auto rsrc = [&](const void* base, long long row_bytes) {
+    const char* p0 = (const char*)base + rows0 * row_bytes;
+    return __builtin_amdgcn_make_buffer_rsrc((void*)p0, 0, whole_ok ? (int)(slab_rows * row_bytes) : 0,
+                                             0x00020000);
+  };
+  const auto rk = rsrc(a.k, ROWB), rv = rsrc(a.v, ROWB);
+  const auto rsk = rsrc(a.s_k, 2 * G), rsv = rsrc(a.s_v, 2 * G);
+  const auto rzk = rsrc(a.z_k, 4 * wg), rzv = rsrc(a.z_v, 4 * wg);
+  const int kq_off = c16 * ROWB + q4 * (ROWB / 4);  // the lane's quarter of K row c16
+  const int ks_off = 2 * (c16 * G + gk);
+  const int kz_off = 4 * (c16 * wg + (gk >> 3));
+  const int vq_off = 4 * q4 * ROWB + vb * VBB;      // block vb of the first of the lane's 4 V rows
+  const int vs_off = 2 * (4 * q4 * G + gv);
+  const int vz_off = 4 * (4 * q4 * wg + (gv >> 3));
+  const bool row_scales = KIND == KIND_W4 || (KIND == KIND_F8 && a.scale_mode == 0);
+
+  // Row, in the slab (in the head's pool when paged), of position t, a multiple
+  // of 16 that starts a half tile.  Positions past the last whole half are
+  // clamped: the look-ahead below asks for them and drops the answer.
+  auto slab_row = [&](int t) -> int {
+    if (PAGED == 0) return t;
+    const int tc = min(t, max(a.S - 16, 0));
+    const int pg = tc / a.page;
+    return bt[pg] * a.page + (tc - pg * a.page);
+  };
+
+  // rb[j]: slab_row(first position of half j)
+  auto fetch_whole = [&](TileRaw<KIND, NC>& raw, const int rbs[2]) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int rb = rbs[j];
+      constexpr int KQ = ROWB / 64;  // 16-byte pieces of a lane's K quarter (0: 8 bytes)
+      u4 kraw[KQ ? KQ : 1];
+      if constexpr (KQ == 0) {
+        const u2 t2 = __builtin_amdgcn_raw_buffer_load_b64(rk, kq_off, rb * ROWB, 2);
+        kraw[0] = u4{t2[0], t2[1], 0u, 0u};
+      } else {
+#pragma unroll
+        for (int i = 0; i < KQ; ++i)
+          kraw[i] = __builtin_amdgcn_raw_buffer_load_b128(rk, kq_off + 16 * i, rb * ROWB, 2);
+      }
+      if constexpr (KIND == KIND_W4) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) raw.k[j][c] = kraw[0][c];
+      } else if constexpr (KIND == KIND_F16) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) raw.k[j][c] = kraw[c];
+      } else {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) raw.k[j][c] = u2{kraw[c >> 1][2 * (c & 1)], kraw[c >> 1][2 * (c & 1) + 1]};
+      }
+      if constexpr (KIND != KIND_F16) {
+        if (row_scales) raw.ks[j] = as_half(__builtin_amdgcn_raw_buffer_load_b16(rsk, ks_off, rb * 2 * G, 0));
+        else raw.ks[j] = slab_sk;
+      }
+      if constexpr (KIND == KIND_W4)
+        if (ASYM) raw.kz[j] = __builtin_amdgcn_raw_buffer_load_b32(rzk, kz_off, rb * 4 * wg, 0);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int k = 4 * j + r;
+        if constexpr (KIND == KIND_W4) {
+          raw.v[k] = __builtin_amdgcn_raw_buffer_load_b32(rv, vq_off, (rb + r) * ROWB, 2);
+          if (ASYM) raw.vz[k] = __builtin_amdgcn_raw_buffer_load_b32(rzv, vz_off, (rb + r) * 4 * wg, 0);
+        } else if constexpr (KIND == KIND_F16) {
+          raw.v[k] = __builtin_amdgcn_raw_buffer_load_b128(rv, vq_off, (rb + r) * ROWB, 2);
+        } else {
+          raw.v[k] = __builtin_amdgcn_raw_buffer_load_b64(rv, vq_off, (rb + r) * ROWB, 2);
+        }
+        if constexpr (KIND != KIND_F16) {
+          if (row_scales) raw.vs[k] = as_half(__builtin_amdgcn_raw_buffer_load_b16(rsv, vs_off, (rb + r) * 2 * G, 0));
+          else raw.vs[k] = slab_sv;
+        }
+      }
+    }
+  };
+
   auto fetch = [&](TileRaw<KIND, NC>& raw, int t0) {
     int pg_lo = 0, pg_hi = 0;
     long long base_lo = 0, base_hi = 0;
@@ -167,7 +267,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
           raw.k[j][0] = t2[0];
           raw.k[j][1] = t2[1];
         }
-        raw.ks[j] = a.s_k[row * G + gk];
+        raw.ks[j] = as_half(a.s_k[row * G + gk]);
         if (ASYM) raw.kz[j] = a.z_k[row * wg + (gk >> 3)];
       } else if constexpr (KIND == KIND_F16) {
 #pragma unroll
@@ -188,7 +288,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
           raw.k[j][0] = u2{t4[0], t4[1]};
           raw.k[j][1] = u2{t4[2], t4[3]};
         }
-        raw.ks[j] = a.scale_mode == 0 ? (uint32_t)a.s_k[row * G + gk] : slab_sk;
+        raw.ks[j] = a.scale_mode == 0 ? as_half(a.s_k[row * G + gk]) : slab_sk;
       }
     }
 #pragma unroll
@@ -197,13 +297,13 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
       const long long row = phys(t, pg_lo, base_lo, pg_hi, base_hi, k >= 4);
       if constexpr (KIND == KIND_W4) {
         raw.v[k] = __builtin_nontemporal_load((const uint32_t*)a.v + row * WD + vb);
-        raw.vs[k] = a.s_v[row * G + gv];
+        raw.vs[k] = as_half(a.s_v[row * G + gv]);
         if (ASYM) raw.vz[k] = a.z_v[row * wg + (gv >> 3)];
       } else if constexpr (KIND == KIND_F16) {
         raw.v[k] = __builtin_nontemporal_load((const u4*)((const uint16_t*)a.v + row * FM_D + 8 * vb));
       } else {
         raw.v[k] = __builtin_nontemporal_load((const u2*)((const uint8_t*)a.v + row * FM_D + 8 * vb));
-        raw.vs[k] = a.scale_mode == 0 ? (uint32_t)a.s_v[row * G + gv] : slab_sv;
+        raw.vs[k] = a.scale_mode == 0 ? as_half(a.s_v[row * G + gv]) : slab_sv;
       }
     }
   };
@@ -218,7 +318,9 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     *(u4*)dst = u4{as_u32(nat[0]), as_u32(nat[1]), as_u32(nat[2]), as_u32(nat[3])};
   };
 
-  auto compute = [&](const TileRaw<KIND, NC>& raw, int t0) {
+  // whole: every position of the tile is below s1 (no masking)
+  auto compute = [&](const TileRaw<KIND, NC>& raw, int t0, auto whole) {
+    constexpr bool WHOLE = decltype(whole)::value;
     // ---- scores
     f4 sc[2];
 #pragma unroll
@@ -227,12 +329,14 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
       const int t = t0 + 16 * j + c16;
       uint16_t* kdst = HOOK ? a.k_out + (hook_base + t) * FM_D + 8 * NC * q4 : nullptr;
       const bool kst = hook_k && t < s1;
+      _Float16 ksc = 0;
+      if constexpr (KIND != KIND_F16) ksc = at_use(raw.ks[j]);
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
         h2 d[4];
         if constexpr (KIND == KIND_W4) {
           const int z = ASYM ? (int)((raw.kz[j] >> (4 * (gk & 7))) & 0xFu) : 8;
-          dq_w4(raw.k[j][c], w4_group((uint16_t)raw.ks[j], z), d);
+          dq_w4(raw.k[j][c], w4_group(ksc, z), d);
           if (kst) {
             h2 nat[4];
             to_natural(d, nat);
@@ -243,7 +347,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
           for (int p = 0; p < 4; ++p) d[p] = as_h2(raw.k[j][c][p]);
           if (kst) store16(kdst + 8 * c, d);
         } else {
-          const h2 s = splat_bits(raw.ks[j]);
+          const h2 s = splat(ksc);
           dq_f8(raw.k[j][c][0], s, d);
           dq_f8(raw.k[j][c][1], s, d + 2);
           if (kst) {
@@ -256,13 +360,15 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
         sc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pack8(d), qop[c], sc[j], 0, 0, 0);
       }
     }
-    // ---- online softmax for head c16 over this lane's 8 positions
+    // ---- online softmax for head c16 over this lane's 8 positions.  The running
+    // maximum is kept on the raw dot products (the scale is positive, so the order
+    // is the same); exp((x - m) / sqrt(D)) is one FMA and one v_exp_f32.
     float x[8];
     float tmax = -INFINITY;
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       const int t = t0 + 16 * (k >> 2) + 4 * q4 + (k & 3);
-      x[k] = t < s1 ? sc[k >> 2][k & 3] * inv_sqrt_d : -INFINITY;
+      x[k] = WHOLE || t < s1 ? sc[k >> 2][k & 3] : -INFINITY;
       tmax = fmaxf(tmax, x[k]);
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
@@ -270,74 +376,150 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     const float m_new = fmaxf(m_run, tmax);
     const float m_use = m_new == -INFINITY ? 0.0f : m_new;
     if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {  // wave-uniform
-      const float alpha = __expf(m_run - m_use);
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * exp_scale);
 #pragma unroll
       for (int e = 0; e < 8; ++e) o[e] *= alpha;
       lsum *= alpha;
     }
     m_run = m_new;
+    const float m_sub = -m_use * exp_scale;
     h2 pr[4];
 #pragma unroll
     for (int k = 0; k < 4; ++k)
-      pr[k] = h2{(_Float16)__expf(x[2 * k] - m_use), (_Float16)__expf(x[2 * k + 1] - m_use)};
+      pr[k] = h2{(_Float16)__builtin_amdgcn_exp2f(__builtin_fmaf(x[2 * k], exp_scale, m_sub)),
+                 (_Float16)__builtin_amdgcn_exp2f(__builtin_fmaf(x[2 * k + 1], exp_scale, m_sub))};
     const h8 pop = pack8(pr);
     lsum = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pop, lsum, 0, 0, 0);
-    // ---- V: expand the 8 positions x 8 elements of this lane, regroup, accumulate
-    h2 vt[8][4];
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
+    // ---- V: expand the 8 positions x 8 elements of this lane so that MFMA e takes
+    // element e of every position, accumulate
+    auto hook_store_v = [&](int k, const h2 nat[4]) {
       const int t = t0 + 16 * (k >> 2) + 4 * q4 + (k & 3);
-      const bool vst = hook_v && t < s1 && c16 < NB;
-      uint16_t* vdst = HOOK ? a.v_out + (hook_base + t) * FM_D + 8 * vb : nullptr;
-      if constexpr (KIND == KIND_W4) {
-        const int z = ASYM ? (int)((raw.vz[k] >> (4 * (gv & 7))) & 0xFu) : 8;
-        dq_w4(raw.v[k], w4_group((uint16_t)raw.vs[k], z), vt[k]);
-        if (vst) {
-          h2 nat[4];
-          to_natural(vt[k], nat);
-          store16(vdst, nat);
-        }
-      } else if constexpr (KIND == KIND_F16) {
+      if (hook_v && t < s1 && c16 < NB) store16(a.v_out + (hook_base + t) * FM_D + 8 * vb, nat);
+    };
+    if constexpr (KIND == KIND_W4) {
+      // Two positions at a time: v_perm puts byte b of both words into the two
+      // halves of a register, so each expanded register already is the pair
+      // (position 2 kk, position 2 kk + 1) of one element -- the MFMA operand
+      // layout -- and the two scales ride in one packed multiply.  Per element the
+      // arithmetic is that of dq_w4: (1024 + n) - (1024 + z) or (64 + n) - (64 + z),
+      // exact, then one rounding in the multiply by the scale.
+      h2 pe[4][8];
+      uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u;
+      asm("" : "+v"(magic_lo));
+      asm("" : "+v"(magic_hi));
 #pragma unroll
-        for (int p = 0; p < 4; ++p) vt[k][p] = as_h2(raw.v[k][p]);
-        if (vst) store16(vdst, vt[k]);
-      } else {
-        const h2 s = splat_bits(raw.vs[k]);
-        dq_f8(raw.v[k][0], s, vt[k]);
-        dq_f8(raw.v[k][1], s, vt[k] + 2);
-        if (vst) {
-          h2 nat[4];
-          to_natural_f8(vt[k], nat);
-          to_natural_f8(vt[k] + 2, nat + 2);
-          store16(vdst, nat);
+      for (int kk = 0; kk < 4; ++kk) {
+        const uint32_t w0 = raw.v[2 * kk], w1 = raw.v[2 * kk + 1];
+        const h2 s2 = h2{at_use(raw.vs[2 * kk]), at_use(raw.vs[2 * kk + 1])};
+        uint32_t zz = 0x00080008u;  // zero points of the two positions, one per half
+        if (ASYM) {
+          const int sh = 4 * (gv & 7);
+          zz = ((raw.vz[2 * kk] >> sh) & 0xFu) | (((raw.vz[2 * kk + 1] >> sh) & 0xFu) << 16);
+        }
+        const h2 clo = as_h2(0xE400E400u | zz);         // -(1024 + z), ulp 1
+        const h2 chi = as_h2(0xD400D400u | (zz << 4));  // -(64 + z), ulp 1/16
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          const uint32_t p = __builtin_amdgcn_perm(w1, w0, 0x0c000c00u | ((4u + b) << 16) | b);
+          pe[kk][2 * b] = (as_h2(and_or(p, 0x000F000Fu, magic_lo)) + clo) * s2;
+          pe[kk][2 * b + 1] = (as_h2(and_or(p, 0x00F000F0u, magic_hi)) + chi) * s2;
+        }
+        if constexpr (HOOK) {
+          h2 n0[4], n1[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            n0[i] = as_h2(__builtin_amdgcn_perm(as_u32(pe[kk][2 * i + 1]), as_u32(pe[kk][2 * i]), 0x05040100u));
+            n1[i] = as_h2(__builtin_amdgcn_perm(as_u32(pe[kk][2 * i + 1]), as_u32(pe[kk][2 * i]), 0x07060302u));
+          }
+          hook_store_v(2 * kk, n0);
+          hook_store_v(2 * kk + 1, n1);
         }
       }
-    }
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      constexpr uint32_t LO = 0x05040100u, HI = 0x07060302u;
-      const int rg = reg_of<KIND>(e);
-      const uint32_t sel = half_of<KIND>(e) ? HI : LO;
-      h2 at[4];
+      for (int e = 0; e < 8; ++e) {
+        const h2 at[4] = {pe[0][e], pe[1][e], pe[2][e], pe[3][e]};
+        o[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pack8(at), pop, o[e], 0, 0, 0);
+      }
+    } else {
+      h2 vt[8][4];
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk)
-        at[kk] = as_h2(__builtin_amdgcn_perm(as_u32(vt[2 * kk + 1][rg]), as_u32(vt[2 * kk][rg]), sel));
-      o[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pack8(at), pop, o[e], 0, 0, 0);
+      for (int k = 0; k < 8; ++k) {
+        if constexpr (KIND == KIND_F16) {
+#pragma unroll
+          for (int p = 0; p < 4; ++p) vt[k][p] = as_h2(raw.v[k][p]);
+          if constexpr (HOOK) hook_store_v(k, vt[k]);
+        } else {
+          const h2 s = splat(at_use(raw.vs[k]));
+          dq_f8(raw.v[k][0], s, vt[k]);
+          dq_f8(raw.v[k][1], s, vt[k] + 2);
+          if constexpr (HOOK) {
+            h2 nat[4];
+            to_natural_f8(vt[k], nat);
+            to_natural_f8(vt[k] + 2, nat + 2);
+            hook_store_v(k, nat);
+          }
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        constexpr uint32_t LO = 0x05040100u, HI = 0x07060302u;
+        const int rg = reg_of<KIND>(e);
+        const uint32_t sel = half_of<KIND>(e) ? HI : LO;
+        h2 at[4];
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+          at[kk] = as_h2(__builtin_amdgcn_perm(as_u32(vt[2 * kk + 1][rg]), as_u32(vt[2 * kk][rg]), sel));
+        o[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pack8(at), pop, o[e], 0, 0, 0);
+      }
     }
   };
 
   // tiles of this wave: s0 + 32 * (wave + 4 * it)
   const int nit = (s1 - s0 + FM_WAVES * FM_TILE - 1) / (FM_WAVES * FM_TILE);
   auto tile_start = [&](int it) { return s0 + FM_TILE * (wave + FM_WAVES * it); };
+  // the first nwhole tiles of this wave lie wholly below s1
+  const int room = s1 - s0 - FM_TILE * (wave + 1);
+  const int nwhole = whole_ok && room >= 0 ? room / (FM_WAVES * FM_TILE) + 1 : 0;
+  // Tile number `it` of this wave into `raw`: buffer loads when it is whole, the
+  // general fetch when it is cut by s1, nothing when it lies past the split.
+  auto fetch_any = [&](TileRaw<KIND, NC>& raw, int it) {
+    if (it < nwhole) {
+      const int rb[2] = {slab_row(tile_start(it)), slab_row(tile_start(it) + 16)};
+      fetch_whole(raw, rb);
+    } else if (it < nit) {
+      fetch(raw, tile_start(it));
+    }
+  };
+  // A ring slot is refilled right after the tile in it has been consumed, into
+  // the same registers: the loop carries no copies, and FM_DEPTH - 1 tiles are in
+  // flight while one is computed.
   TileRaw<KIND, NC> ring[FM_DEPTH];
 #pragma unroll
-  for (int d = 0; d < FM_DEPTH; ++d) fetch(ring[d], tile_start(d));
-  for (int it0 = 0; it0 < nit; it0 += FM_DEPTH) {
+  for (int d = 0; d < FM_DEPTH; ++d) fetch_any(ring[d], d);
+  int it0 = 0;
+  // Page-table lookups run one tile ahead of the loads that need them, so the
+  // scalar load's latency is off the path to the vector loads.
+  int rb_next[2] = {slab_row(tile_start(FM_DEPTH)), slab_row(tile_start(FM_DEPTH) + 16)};
+  for (; it0 + 2 * FM_DEPTH <= nwhole; it0 += FM_DEPTH) {  // computes and fetches whole tiles only
 #pragma unroll
     for (int d = 0; d < FM_DEPTH; ++d) {
-      const TileRaw<KIND, NC> raw = ring[d];
-      fetch(ring[d], tile_start(it0 + d + FM_DEPTH));
-      compute(raw, tile_start(it0 + d));
+      compute(ring[d], tile_start(it0 + d), std::true_type{});
+      __builtin_amdgcn_sched_barrier(0);
+      const int rb[2] = {rb_next[0], rb_next[1]};
+      const int t_after = tile_start(it0 + d + FM_DEPTH + 1);
+      rb_next[0] = slab_row(t_after);
+      rb_next[1] = slab_row(t_after + 16);
+      fetch_whole(ring[d], rb);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  for (; it0 < nit; it0 += FM_DEPTH) {
+#pragma unroll
+    for (int d = 0; d < FM_DEPTH; ++d) {
+      if (it0 + d < nit) compute(ring[d], tile_start(it0 + d), std::false_type{});
+      __builtin_amdgcn_sched_barrier(0);
+      fetch_any(ring[d], it0 + d + FM_DEPTH);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 
@@ -351,7 +533,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
       if (4 * q4 + r < NB) mine[32 * q4 + 8 * r + e] = o[e][r];
   if (q4 == 0) {
     mine[FM_D] = lsum[0];
-    mine[FM_D + 1] = m_run;
+    mine[FM_D + 1] = m_run * inv_sqrt_d;  // the maximum of the scaled scores
   }
   __syncthreads();
   for (int i = threadIdx.x; i < nh * (FM_D + 1); i += FM_WAVES * 64) {

@@ -25,6 +25,8 @@ ATT = [(1, 1, 64, 32), (2, 7, 64, 8), (4, 128, 128, 128), (2, 300, 96, 32), (3, 
        # head dimension 64 on the matrix-core kernel (gs a multiple of 16)
        (2, 100, 64, 16), (1, 1, 64, 64), (3, 257, 64, 32)]
 BIG = [(2, 5000, 64, 32), (1, 9000, 128, 64)]
+# more slabs than workgroups wanted: one split per slab, 9 to 11 tiles per wave
+LONG_SPLITS = [(520, 1300, 128, 32), (600, 1100, 64, 32)]
 
 
 def _w4_case(H, S, D, gs, sym, seed, group=1):
@@ -110,12 +112,24 @@ F8 = [(1, 1, 64, 32), (2, 7, 64, 8), (4, 128, 128, 128), (2, 300, 96, 32), (3, 6
 
 @pytest.mark.parametrize("i", range(len(F8)))
 def test_f8_flash(i):
-    c = w4amd.capi()
     H, S, D, gs = F8[i]
     seed = 0xF80A ^ (i * 977)
     k = orc.normal_weights(H * S * D, seed)
     v = orc.normal_weights(H * S * D, seed + 1)
     q = orc.normal_activations(H * D, seed + 2)
+    _check_f8(H, S, D, gs, k, v, q)
+
+
+def test_f8_flash_long_splits():
+    """Splits of 6 and more tiles per wave: the loop that only sees whole tiles."""
+    H, S, D, gs = LONG_SPLITS[0]
+    rng = np.random.default_rng(0xF81B)
+    k, v = rng.standard_normal(H * S * D), rng.standard_normal(H * S * D)
+    _check_f8(H, S, D, gs, k, v, orc.normal_activations(H * D, 0xF81C))
+
+
+def _check_f8(H, S, D, gs, k, v, q):
+    c = w4amd.capi()
     c8 = orc.quantize_cache_f8(k, v, H, S, D, gs)
     kd, vd = orc.dequant_cache_f8(c8, False), orc.dequant_cache_f8(c8, True)
     ref = orc.attention_f16(q, kd, vd, H, 1, S, D)
@@ -234,6 +248,30 @@ def test_paged_equals_contiguous(i, sym):
     c.attention_w4_flash_paged(view, ptr(bt_d), page, npages, ptr(q_d), ptr(out), 0, ptr(ko), ptr(vo))
     assert np.array_equal(bits(out), o_w4), "paged output == contiguous output, bytewise"
     assert np.array_equal(bits(ko), kd.ravel()) and np.array_equal(bits(vo), vd.ravel())
+
+
+@pytest.mark.parametrize("sym", [True, False], ids=["sym", "asym"])
+@pytest.mark.parametrize("i", range(len(LONG_SPLITS)))
+def test_w4_flash_long_splits(i, sym):
+    """So many slabs that each gets one or two splits: a wave walks 6 and more tiles,
+    which takes the loop that only sees whole tiles (its look-ahead of the page
+    table included), then the loop for the cut tiles at the end."""
+    c = w4amd.capi()
+    H, S, D, gs = LONG_SPLITS[i]
+    seed = 0x10E6 ^ (i * 977 + (0 if sym else 1))
+    rng = np.random.default_rng(seed)
+    k, v = rng.standard_normal(H * S * D), rng.standard_normal(H * S * D)
+    c4 = orc.quantize_cache(k, v, H, S, D, gs, sym)
+    q = orc.normal_activations(H * D, seed + 2)
+    o_w4, dk, q_d, kd, vd, ref = _check_w4(c4, q)
+    for page in (16, 48):
+        npages = (S + page - 1) // page
+        bt = np.random.default_rng(seed ^ page).permutation(npages).astype(np.int32)
+        keep, view = _paged_pool(c4, page, bt)
+        bt_d = to_dev(bt)
+        out = halves(H * D, 0x7E00)
+        c.attention_w4_flash_paged(view, ptr(bt_d), page, npages, ptr(q_d), ptr(out))
+        assert np.array_equal(bits(out), o_w4), "paged output == contiguous output, bytewise"
 
 
 @pytest.mark.parametrize("D", [64, 128])

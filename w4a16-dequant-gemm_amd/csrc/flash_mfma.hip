@@ -104,6 +104,12 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
   const int G = a.G, wg = words(a.G);
   const int vb = c16 & (NB - 1);                               // this lane's V element block
   const int gk = KIND == KIND_F16 ? 0 : (8 * NC * q4) / a.gs;  // group of this lane's K elements
+  // First of the 8 row elements that score MFMA c contracts in this lane.  The
+  // quantized kinds take a contiguous quarter of the row per lane (one load, one
+  // scale).  FP16 needs a 16-byte load per MFMA either way, so there the four
+  // k-blocks of an MFMA are neighbours: a load instruction reads 64 contiguous
+  // bytes of each row instead of 16 bytes out of every 64.
+  auto kcol = [&](int c) { return KIND == KIND_F16 ? 32 * c + 8 * q4 : 8 * NC * q4 + 8 * c; };
   const int gv = KIND == KIND_F16 ? 0 : (8 * vb) / a.gs;       // ... and of its V elements
 
   const int* bt = nullptr;
@@ -133,17 +139,17 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
   const bool hook_k = HOOK && a.k_out && qh0 == 0, hook_v = HOOK && a.v_out && qh0 == 0;
 
   // Query operands: lane (head c16, k-block q4) of MFMA c holds
-  // q[head][8 NC q4 + 8 c + elem_of(p, hf)].
+  // q[head][kcol(c) + elem_of(p, hf)].
   h8 qop[NC];
   {
     const uint16_t* qp =
-        a.q + ((long long)slab * a.group + qh0 + min(c16, nh - 1)) * FM_D + 8 * NC * q4;
+        a.q + ((long long)slab * a.group + qh0 + min(c16, nh - 1)) * FM_D;
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       h2 t[4];
 #pragma unroll
       for (int p = 0; p < 4; ++p) {
-        const uint32_t lo = qp[8 * c + elem_of<KIND>(p, 0)], hi = qp[8 * c + elem_of<KIND>(p, 1)];
+        const uint32_t lo = qp[kcol(c) + elem_of<KIND>(p, 0)], hi = qp[kcol(c) + elem_of<KIND>(p, 1)];
         t[p] = as_h2(c16 < nh ? (lo | (hi << 16)) : 0u);
       }
       qop[c] = pack8(t);
@@ -206,7 +212,8 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
       } else {
 #pragma unroll
         for (int i = 0; i < KQ; ++i)
-          kraw[i] = __builtin_amdgcn_raw_buffer_load_b128(rk, kq_off + 16 * i, rb * ROWB, 2);
+          kraw[i] = __builtin_amdgcn_raw_buffer_load_b128(
+              rk, KIND == KIND_F16 ? c16 * ROWB + 2 * kcol(i) : kq_off + 16 * i, rb * ROWB, 2);
       }
       if constexpr (KIND == KIND_W4) {
 #pragma unroll
@@ -273,7 +280,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
 #pragma unroll
         for (int c = 0; c < NC; ++c)
           raw.k[j][c] = __builtin_nontemporal_load(
-              (const u4*)((const uint16_t*)a.k + row * FM_D + 8 * NC * q4 + 8 * c));
+              (const u4*)((const uint16_t*)a.k + row * FM_D + kcol(c)));
       } else {
         const uint8_t* src = (const uint8_t*)a.k + row * FM_D + 8 * NC * q4;
         if constexpr (NC == 4) {
@@ -327,7 +334,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     for (int j = 0; j < 2; ++j) {
       sc[j] = f4{0.f, 0.f, 0.f, 0.f};
       const int t = t0 + 16 * j + c16;
-      uint16_t* kdst = HOOK ? a.k_out + (hook_base + t) * FM_D + 8 * NC * q4 : nullptr;
+      uint16_t* kdst = HOOK ? a.k_out + (hook_base + t) * FM_D : nullptr;
       const bool kst = hook_k && t < s1;
       _Float16 ksc = 0;
       if constexpr (KIND != KIND_F16) ksc = at_use(raw.ks[j]);
@@ -340,12 +347,12 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
           if (kst) {
             h2 nat[4];
             to_natural(d, nat);
-            store16(kdst + 8 * c, nat);
+            store16(kdst + kcol(c), nat);
           }
         } else if constexpr (KIND == KIND_F16) {
 #pragma unroll
           for (int p = 0; p < 4; ++p) d[p] = as_h2(raw.k[j][c][p]);
-          if (kst) store16(kdst + 8 * c, d);
+          if (kst) store16(kdst + kcol(c), d);
         } else {
           const h2 s = splat(ksc);
           dq_f8(raw.k[j][c][0], s, d);
@@ -354,7 +361,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
             h2 nat[4];
             to_natural_f8(d, nat);
             to_natural_f8(d + 2, nat + 2);
-            store16(kdst + 8 * c, nat);
+            store16(kdst + kcol(c), nat);
           }
         }
         sc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pack8(d), qop[c], sc[j], 0, 0, 0);

@@ -509,6 +509,9 @@ def probe(b, which):
         views = b.rand_w4(N, K, 128, True, 18)
         for M, fn in ((1, "w4_gemm_fused"), (8, "w4_gemm_mma"), (16, "w4_gemm_mma")):
             out["%s_M%d_us" % (fn, M)] = b.gemm_us(fn, views, M, N, K)
+    elif which == "attention":  # C5 flash decode over FP16 / W4 / paged W4 / FP8 caches
+        b.steps = 200
+        out.update(extras_attention(b, False))
     elif which == "quantize":  # the device-side quantizers, 20 calls of each workload
         b.steps, b.warmup = 200, 2
         out.update(extras_quantize(b, False))
@@ -539,7 +542,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--extras", choices=["none", "quick", "full"], default="quick")
-    ap.add_argument("--probe", choices=["decode", "prefill", "quantize", "w4a4"], default=None,
+    ap.add_argument("--probe", choices=["decode", "prefill", "quantize", "w4a4", "attention"], default=None,
                     help="run only a short fixed workload (for counter collection) and exit")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -22,7 +22,6 @@ namespace w4k {
 
 constexpr int FL_TILE = 256;   // positions per tile
 constexpr int FL_WAVES = 4;
-constexpr int FL_MAXGQ = 4;    // query heads handled per pass
 
 
 // Offset within a lane's E-element chunk of register pair p, half hf.

@@ -315,9 +315,17 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     }
   };
 
-  f4 o[8], lsum = f4{0.f, 0.f, 0.f, 0.f};
+  // W4 at D = 64: a row has only 8 element blocks for the 16 operand rows of the
+  // PV MFMA, so lanes i and i + 8 share block i % 8 and split its elements (0..3
+  // and 4..7): 4 MFMAs whose row i is d = 8 (i % 8) + 4 (i / 8) + e, and half of
+  // the expansion per lane.  (FP16 / FP8 at D = 64 repeat the blocks instead and
+  // drop the upper rows.)
+  constexpr bool SPLITV = KIND == KIND_W4 && DH == 64;
+  constexpr int NE = SPLITV ? 4 : 8;  // PV MFMAs per tile = elements a lane expands per position
+  const int hi8 = SPLITV ? c16 >> 3 : 0;
+  f4 o[NE], lsum = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int e = 0; e < 8; ++e) o[e] = f4{0.f, 0.f, 0.f, 0.f};
+  for (int e = 0; e < NE; ++e) o[e] = f4{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY;
   const h8 ones = h8{1, 1, 1, 1, 1, 1, 1, 1};
 
@@ -385,7 +393,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {  // wave-uniform
       const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * exp_scale);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) o[e] *= alpha;
+      for (int e = 0; e < NE; ++e) o[e] *= alpha;
       lsum *= alpha;
     }
     m_run = m_new;
@@ -403,6 +411,12 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
       const int t = t0 + 16 * (k >> 2) + 4 * q4 + (k & 3);
       if (hook_v && t < s1 && c16 < NB) store16(a.v_out + (hook_base + t) * FM_D + 8 * vb, nat);
     };
+    // the 4 elements of a lane of the split layout
+    auto hook_store_v4 = [&](int k, const h2 nat[2]) {
+      const int t = t0 + 16 * (k >> 2) + 4 * q4 + (k & 3);
+      if (hook_v && t < s1)
+        *(u2*)(a.v_out + (hook_base + t) * FM_D + 8 * vb + 4 * hi8) = u2{as_u32(nat[0]), as_u32(nat[1])};
+    };
     if constexpr (KIND == KIND_W4) {
       // Two positions at a time: v_perm puts byte b of both words into the two
       // halves of a register, so each expanded register already is the pair
@@ -410,10 +424,12 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
       // layout -- and the two scales ride in one packed multiply.  Per element the
       // arithmetic is that of dq_w4: (1024 + n) - (1024 + z) or (64 + n) - (64 + z),
       // exact, then one rounding in the multiply by the scale.
-      h2 pe[4][8];
+      h2 pe[4][NE];
       uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u;
       asm("" : "+v"(magic_lo));
       asm("" : "+v"(magic_hi));
+      // byte b of a lane's share of the word is byte b + 2 hi8 of the word
+      const uint32_t byte0 = 2u * (uint32_t)hi8;
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
         const uint32_t w0 = raw.v[2 * kk], w1 = raw.v[2 * kk + 1];
@@ -426,24 +442,29 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
         const h2 clo = as_h2(0xE400E400u | zz);         // -(1024 + z), ulp 1
         const h2 chi = as_h2(0xD400D400u | (zz << 4));  // -(64 + z), ulp 1/16
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-          const uint32_t p = __builtin_amdgcn_perm(w1, w0, 0x0c000c00u | ((4u + b) << 16) | b);
+        for (int b = 0; b < NE / 2; ++b) {
+          const uint32_t p = __builtin_amdgcn_perm(w1, w0, 0x0c000c00u | ((4u + b + byte0) << 16) | (b + byte0));
           pe[kk][2 * b] = (as_h2(and_or(p, 0x000F000Fu, magic_lo)) + clo) * s2;
           pe[kk][2 * b + 1] = (as_h2(and_or(p, 0x00F000F0u, magic_hi)) + chi) * s2;
         }
         if constexpr (HOOK) {
           h2 n0[4], n1[4];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
+          for (int i = 0; i < NE / 2; ++i) {
             n0[i] = as_h2(__builtin_amdgcn_perm(as_u32(pe[kk][2 * i + 1]), as_u32(pe[kk][2 * i]), 0x05040100u));
             n1[i] = as_h2(__builtin_amdgcn_perm(as_u32(pe[kk][2 * i + 1]), as_u32(pe[kk][2 * i]), 0x07060302u));
           }
-          hook_store_v(2 * kk, n0);
-          hook_store_v(2 * kk + 1, n1);
+          if constexpr (SPLITV) {
+            hook_store_v4(2 * kk, n0);
+            hook_store_v4(2 * kk + 1, n1);
+          } else {
+            hook_store_v(2 * kk, n0);
+            hook_store_v(2 * kk + 1, n1);
+          }
         }
       }
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
+      for (int e = 0; e < NE; ++e) {
         const h2 at[4] = {pe[0][e], pe[1][e], pe[2][e], pe[3][e]};
         o[e] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pack8(at), pop, o[e], 0, 0, 0);
       }
@@ -534,10 +555,13 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
   // O[head][32 q4 + 8 r + e] in o[e][r] (output rows past D / 8 are repeats: dropped)
   float* mine = wo[wave] + c16 * LDW;
 #pragma unroll
-  for (int e = 0; e < 8; ++e)
+  for (int e = 0; e < NE; ++e)
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-      if (4 * q4 + r < NB) mine[32 * q4 + 8 * r + e] = o[e][r];
+    for (int r = 0; r < 4; ++r) {
+      const int i = 4 * q4 + r;  // operand row of the PV MFMA
+      if constexpr (SPLITV) mine[8 * (i & 7) + 4 * (i >> 3) + e] = o[e][r];
+      else if (i < NB) mine[8 * i + e] = o[e][r];
+    }
   if (q4 == 0) {
     mine[FM_D] = lsum[0];
     mine[FM_D + 1] = m_run * inv_sqrt_d;  // the maximum of the scaled scores

@@ -14,11 +14,16 @@
 //            the 32 positions, B = the probabilities straight from the score
 //            registers (FP16), A = V transposed: lane (i = l%16, r = l/16) loads
 //            the 8 cache elements d = 8i..8i+7 of its 8 positions (one packed
-//            word, 8 bytes, or 16 bytes each), expands them and regroups the
-//            8x8 block with v_perm so that MFMA e takes element e of every
-//            position.  A ninth MFMA with A = 1 accumulates the denominators.
-//            (D = 64 has only 8 element blocks: lanes i >= 8 repeat blocks 0..7
-//            and their output rows are dropped.)
+//            word, 8 bytes, or 16 bytes each) and expands them so that MFMA e
+//            takes element e of every position: W4 expands two positions at a
+//            time straight into that layout, FP16 / FP8 regroup the 8x8 block
+//            with v_perm.  A ninth MFMA with A = 1 accumulates the denominators.
+//            (D = 64 has only 8 element blocks for 16 operand rows: W4 lets lanes
+//            i and i + 8 split the elements of block i % 8 -- 4 MFMAs --, FP16 /
+//            FP8 repeat blocks 0..7 and drop the upper output rows.)
+// Whole tiles are fetched with buffer loads whose wave-uniform part lives in the
+// descriptor and the scalar offset; a ring of three raw tiles is refilled in
+// place, two tiles in flight while one is computed.
 // Dequantisation is the bit-exact register step of dq.cuh (the k_out / v_out
 // hooks store those values); only the order of the FP32 sums differs from the
 // vector kernel.  The four waves of a workgroup interleave tiles of one split

@@ -185,6 +185,36 @@ def test_f8_every_code_and_slab_scale():
     assert orc.rel_l2(f64(out), ref) <= TOL
 
 
+@pytest.mark.parametrize("nan_codes", ["none", "first_tile", "all"])
+def test_f8_every_code_matrix_core_kernel(nan_codes):
+    """Every byte code under odd scales through the D = 128 matrix-core kernel, hooks
+    bit-exact.  The closed-form decode reads the NaN codes 0x7F / 0xFF as +-480
+    (kvfp8.hpp:41-50); none / some / all of the tiles hold such a code, so a decode
+    that treats those tiles differently is covered on both sides."""
+    c = w4amd.capi()
+    H, S, D, gs = 2, 160, 128, 32
+    G = D // gs
+    c8 = orc.KVCacheF8()
+    c8.H, c8.S, c8.D, c8.gs, c8.G = H, S, D, gs, G
+    codes = (np.arange(H * S * D) % 256).astype(np.uint8)
+    pos = (np.arange(H * S * D) // D) % S
+    special = (codes & 0x7F) == 0x7F
+    if nan_codes == "none":
+        codes[special] -= 1
+    elif nan_codes == "first_tile":
+        codes[special & (pos >= 32)] -= 1
+    c8.q_k, c8.q_v = codes, codes[::-1].copy()
+    sc = np.array([0x3C00, 0x0001, 0x03FF, 0x5BFF, 0x7BFF, 0x2E66, 0x8400, 0x1400, 0x3555], np.uint16)
+    c8.s_k = np.resize(sc, H * S * G)
+    c8.s_v = np.resize(sc[::-1], H * S * G)
+    kd, vd = orc.dequant_cache_f8(c8, False), orc.dequant_cache_f8(c8, True)
+    d8 = DevKVF8(c8)
+    q_d = to_dev(np.zeros(H * D, np.uint16))
+    out, ko, vo = halves(H * D), halves(H * S * D, 0x7E00), halves(H * S * D, 0x7E00)
+    c.attention_f8_flash(d8.view, ptr(q_d), ptr(out), 0, ptr(ko), ptr(vo))
+    assert np.array_equal(bits(ko), kd.ravel()) and np.array_equal(bits(vo), vd.ravel())
+
+
 def test_f8_slab_scale_head_dim_128():
     c = w4amd.capi()
     H, S, D, gs, group = 2, 500, 128, 128, 4

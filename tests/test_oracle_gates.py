@@ -41,6 +41,30 @@ def test_w4_per_element_bounds(i, sym):
         assert q.min() >= 1  # symmetric codes live in [1, 15]
 
 
+def test_w4_rounding_ties_go_away_from_zero():
+    """pack.hpp:113-121 rounds the zero-point and every code with std::lround, which
+    sends halves away from zero.  Codes derived by hand on groups whose stored scale
+    is exactly 1.0, so every quotient is the value itself; round-half-to-even would
+    give 8, 8, 10, 6, 10, 6, 14 on the symmetric ties and zero-point 2 below."""
+    # symmetric: amax = 7 -> scale 7/7 = 1.0, code = lround(w) + 8
+    w = np.array([7.0, 0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 6.5])
+    p = orc.quantize(w, 1, 8, 8, True)
+    assert p.scales[0] == 0x3C00
+    assert nibbles(p.q, 1, 8)[0].tolist() == [15, 9, 7, 10, 6, 11, 5, 15]
+    # asymmetric: lo = -2.5, hi = 12.5 -> scale 15/15 = 1.0, z = lround(2.5) = 3,
+    # code = clamp(lround(w) + 3): -2.5 -> -3 + 3 = 0, 12.5 -> 13 + 3 = 16 -> 15
+    w = np.array([-2.5, 12.5, 0.5, -0.5, 1.5, 3.5, -1.5, 4.5])
+    p = orc.quantize(w, 1, 8, 8, False)
+    assert p.scales[0] == 0x3C00 and int(p.zeros[0] & 0xF) == 3
+    assert nibbles(p.q, 1, 8)[0].tolist() == [0, 15, 4, 2, 5, 7, 1, 8]
+    # a one-sided group: the range is widened to bracket zero (lo = 0, hi = 7.5 ->
+    # scale 0.5, z = 0), codes lround(w / 0.5): 0.25 -> lround(0.5) = 1, 1.25 -> 3
+    w = np.array([7.5, 0.25, 1.25, 2.0, 0.75, 3.25, 0.0, 5.0])
+    p = orc.quantize(w, 1, 8, 8, False)
+    assert p.scales[0] == 0x3800 and int(p.zeros[0] & 0xF) == 0
+    assert nibbles(p.q, 1, 8)[0].tolist() == [15, 1, 3, 4, 2, 7, 0, 10]
+
+
 def test_gemm_oracle_hand_pin():
     # test_oracle.cpp:63-78
     x = np.array([1, 2], np.float16).view(np.uint16)

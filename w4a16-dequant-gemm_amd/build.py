@@ -44,9 +44,14 @@ def build(force=False, verbose=True):
     os.makedirs(os.path.dirname(LIB), exist_ok=True)
     objs, procs = [], []
     os.makedirs(os.path.join(PKG, "lib", "obj"), exist_ok=True)
+    hdr_t = max(os.path.getmtime(os.path.join(CSRC, h)) for h in HEADERS if not h.endswith(".hip"))
+    hdr_t = max(hdr_t, os.path.getmtime(os.path.abspath(__file__)))
     for src in SOURCES:
         obj = os.path.join(PKG, "lib", "obj", src.replace(".hip", ".o"))
         objs.append(obj)
+        if (not force and os.path.exists(obj)
+                and os.path.getmtime(obj) > max(hdr_t, os.path.getmtime(os.path.join(CSRC, src)))):
+            continue  # this object is newer than its source and every shared header
         cmd = ["hipcc", *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
         procs.append((src, subprocess.Popen(cmd, stderr=subprocess.PIPE, text=True)))
     for src, p in procs:

@@ -36,13 +36,16 @@ __host__ __device__ __forceinline__ int words(int n) { return (n + 7) >> 3; }
 // Group index of each of the four 8-k words of a lane's 32-k slice that starts
 // at k0 (gs: a multiple of 8).  One division (a shift when gs is a power of two:
 // gs_shift >= 0), then compares: 32 k span at most four groups.
-__device__ __forceinline__ void groups_of_slice(int k0, int gs, int gs_shift, int g[4]) {
+// A slice that runs past K (K % 32 != 0) names groups past the last one; they are
+// clamped to g_last so that no scale or zero-point is read beyond its row.
+__device__ __forceinline__ void groups_of_slice(int k0, int gs, int gs_shift, int g_last,
+                                                int g[4]) {
   const int g0 = gs_shift >= 0 ? (k0 >> gs_shift) : k0 / gs;
   const int rem = k0 - g0 * gs;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int o = rem + 8 * j;
-    g[j] = g0 + (o >= gs) + (o >= 2 * gs) + (o >= 3 * gs);
+    g[j] = min(g0 + (o >= gs) + (o >= 2 * gs) + (o >= 3 * gs), g_last);
   }
 }
 

@@ -219,7 +219,7 @@ __global__ __launch_bounds__(DEC_WAVES * 64) void mfma_decode_kernel(
     for (int i = 0; i < CH; ++i) {
       int g4[4];
       if (NS == 1) g4[0] = MX ? (kl[i] >> 5) : gs_shift >= 0 ? (kl[i] >> gs_shift) : kl[i] / p.gs;
-      else groups_of_slice(kl[i], p.gs, gs_shift, g4);
+      else groups_of_slice(kl[i], p.gs, gs_shift, p.G - 1, g4);
 #pragma unroll
       for (int e = 0; e < NS; ++e) {
         const int g = g4[e];
@@ -431,7 +431,7 @@ __global__ __launch_bounds__(64 * NW * KW) void mfma_stream_kernel(
       const int kc = (LEAN || (s < cpk && k < p.K)) ? k : 0;
       int g[4];
       if (NS == 1) g[0] = group_of(kc);
-      else groups_of_slice(kc, p.gs, gs_shift, g);
+      else groups_of_slice(kc, p.gs, gs_shift, p.G - 1, g);
 #pragma unroll
       for (int e = 0; e < NS; ++e) {
         if (MX) {

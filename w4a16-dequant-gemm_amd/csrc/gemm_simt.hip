@@ -353,7 +353,7 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_unrolled_kernel(
     const int k0 = s * 2048 + lane * 32;
     int g[4];
     if (NS == 1) g[0] = MX ? (k0 >> 5) : POW2 ? (k0 >> gs_shift) : k0 / p.gs;
-    else groups_of_slice(k0, p.gs, gs_shift, g);
+    else groups_of_slice(k0, p.gs, gs_shift, p.G - 1, g);
 #pragma unroll
     for (int e = 0; e < NS; ++e) zsh[s][e] = 4u * (uint32_t)(g[e] & 7);
 #pragma unroll
@@ -506,7 +506,7 @@ __global__ __launch_bounds__(W * 64) void simt_ksplit_kernel(
   for (int s = 0; s < STEPS; ++s) {
     int g[4];
     if (NS == 1) g[0] = MX ? (k0[s] >> 5) : gs_shift >= 0 ? (k0[s] >> gs_shift) : k0[s] / p.gs;
-    else groups_of_slice(k0[s], p.gs, gs_shift, g);
+    else groups_of_slice(k0[s], p.gs, gs_shift, p.G - 1, g);
 #pragma unroll
     for (int e = 0; e < NS; ++e) {
       zsh[s][e] = 4u * (uint32_t)(g[e] & 7);

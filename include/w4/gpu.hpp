@@ -243,6 +243,18 @@ inline void attention_w4_flash_gqa(const DeviceKVW4& p, int group, const __half*
                                           detail::h(k_out), detail::h(v_out)));
 }
 
+// The same call with the split-S partials in the library's built-in device array:
+// no device allocation (for callers under graph capture or in loops that must not
+// hipMalloc); throws std::invalid_argument when the partials exceed
+// W4_NOALLOC_SCRATCH_BYTES.  Calls on one GPU share the array and must not overlap.
+inline void attention_w4_flash_noalloc(const DeviceKVW4& p, int group, const __half* q,
+                                       __half* out, hipStream_t stream = 0,
+                                       __half* k_out = nullptr, __half* v_out = nullptr) {
+  const auto v = detail::abi(p);
+  detail::raise(w4_attention_w4_flash_gqa_noalloc(&v, group, detail::h(q), detail::h(out), stream,
+                                                  detail::h(k_out), detail::h(v_out)));
+}
+
 inline void attention_fp16_flash_gqa(const __half* q, const __half* k16, const __half* v16,
                                      __half* out, int H, int group, int S, int D,
                                      hipStream_t stream = 0) {

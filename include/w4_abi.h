@@ -154,6 +154,21 @@ int w4_attention_w4_flash_paged_batched(const w4_kv_view* p, const int* bt,
                                         const w4_half* q, w4_half* out,
                                         w4_stream stream);
 
+/* No counterpart in the reference: w4_attention_w4_flash_gqa for callers that
+ * cannot allocate device memory (HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  Same arguments, kernels and output bytes;
+ * the split-S partials live in a W4_NOALLOC_SCRATCH_BYTES array built into the
+ * library (one copy per GPU, held until the process ends) instead of the
+ * library's grow-only buffer, and the call makes no hipMalloc / hipFree.  Calls
+ * whose partials (slabs * group * splits * (D + 2) floats, splits chosen so that
+ * about 512 workgroups run) do not fit are rejected with W4_EINVAL.  Every call
+ * on one GPU shares that GPU's array: calls that overlap on one GPU race. */
+#define W4_NOALLOC_SCRATCH_BYTES (4u << 20)
+int w4_attention_w4_flash_gqa_noalloc(const w4_kv_view* p, int group,
+                                      const w4_half* q, w4_half* out,
+                                      w4_stream stream, w4_half* k_out,
+                                      w4_half* v_out);
+
 /* ---- device-side quantizers: the host quantizers as kernels, same bytes -----
  * The view's arrays are the OUTPUTS (device memory of the sizes the view
  * implies; no need to clear them).  Sources are row-major FP64, as the host

@@ -1,0 +1,63 @@
+"""GPU gate for the entry point that allocates nothing
+(w4_attention_w4_flash_gqa_noalloc): through the C ABI, its output equals the
+output of w4_attention_w4_flash_gqa byte for byte (same kernels, same split
+plan, only the home of the split-S partials differs) and is within rel L2 1e-3
+of the FP64 softmax(QK^T/sqrt(D))V over the dequantized cache, on two calls in a
+row, the second on a smaller input, so stale partials of the first call would
+show.  Partials that do not fit the built-in array are rejected, not truncated.
+"""
+import numpy as np
+import pytest
+import torch
+
+import orc
+import w4amd
+from devutil import DevKV, bits, halves, ptr, to_dev
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+# (slabs, positions, head dim, gs, query heads per slab, symmetric); the second of
+# each pair is the smaller call that follows the first
+PAIRS = [((4, 3000, 128, 32, 4, True), (2, 700, 128, 32, 2, True)),      # matrix-core kernel
+         ((3, 1500, 96, 32, 2, False), (1, 65, 40, 8, 1, False))]        # vector kernel, zero-points
+
+
+def _one(c, H, S, D, gs, group, sym, seed, hooks):
+    k = orc.normal_weights(H * S * D, seed)
+    v = orc.normal_weights(H * S * D, seed + 1)
+    q = orc.normal_activations(H * group * D, seed + 2)
+    c4 = orc.quantize_cache(k, v, H, S, D, gs, sym)
+    kd, vd = orc.dequant_cache(c4, False), orc.dequant_cache(c4, True)
+    ref = orc.attention_f16(q, kd, vd, H, group, S, D)
+    dk, q_d = DevKV(c4), to_dev(q)
+    want = halves(H * group * D, 0x7E00)
+    c.attention_w4_flash(dk.view, ptr(q_d), ptr(want), group=group)
+    want = bits(want).copy()
+    got = halves(H * group * D, 0x7E00)
+    ko = halves(H * S * D, 0x7E00) if hooks else None
+    vo = halves(H * S * D, 0x7E00) if hooks else None
+    print(f"noalloc case H={H} S={S} D={D} gs={gs} group={group} sym={sym} hooks={hooks}", flush=True)
+    c.attention_w4_flash_noalloc(dk.view, ptr(q_d), ptr(got), 0, ptr(ko), ptr(vo), group=group)
+    got = bits(got).copy()
+    assert np.array_equal(got, want), "noalloc output differs from w4_attention_w4_flash_gqa"
+    assert orc.rel_l2(got.view(np.float16), ref) <= TOL
+    if hooks:
+        assert np.array_equal(bits(ko), kd.ravel()) and np.array_equal(bits(vo), vd.ravel())
+
+
+@pytest.mark.parametrize("i", range(len(PAIRS)))
+def test_noalloc_equals_allocating_entry_twice_in_a_row(i):
+    c = w4amd.capi()
+    first, second = PAIRS[i]
+    _one(c, *first, seed=0xA110C ^ (i * 977), hooks=False)
+    _one(c, *second, seed=0xA110D ^ (i * 977), hooks=True)
+
+
+def test_noalloc_rejects_partials_beyond_the_builtin_scratch():
+    c = w4amd.capi()
+    # 1 slab, 64 query heads, S = 2^19: 512 splits * 64 heads * 130 floats = 17 MB of partials
+    one = 256  # non-null, never dereferenced: the size check comes before any device work
+    view = c.kv_view(1, 1 << 19, 128, 32, 4, 1, one, one, 0, one, one, 0)
+    with pytest.raises(ValueError, match="exceed the built-in scratch"):
+        c.attention_w4_flash_noalloc(view, one, one, group=64)

@@ -57,6 +57,7 @@ SIGNATURES = {
     "w4_attention_w4_flash_paged": ([C.POINTER(KVView), vp, C.c_int, C.c_int, vp, vp, vp, vp, vp], C.c_int),
     "w4_dequant_f8": ([vp, vp, vp, C.c_int, C.c_int, C.c_int, vp], C.c_int),
     "w4_attention_w4_flash_gqa": ([C.POINTER(KVView), C.c_int, vp, vp, vp, vp, vp], C.c_int),
+    "w4_attention_w4_flash_gqa_noalloc": ([C.POINTER(KVView), C.c_int, vp, vp, vp, vp, vp], C.c_int),
     "w4_attention_fp16_flash_gqa": ([vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, vp], C.c_int),
     "w4_attention_f8_flash_gqa": ([C.POINTER(KVF8View), C.c_int, C.c_int, vp, vp, vp, vp, vp], C.c_int),
     "w4_attention_w4_flash_paged_batched": ([C.POINTER(KVView), vp, C.c_int, C.c_int, C.c_int, C.c_int,
@@ -157,6 +158,13 @@ def gemm_fp16(w, x, c, M, N, K, stream=0):
 def attention_w4_flash(view, q, out, stream=0, k_out=0, v_out=0, group=1):
     check(load().w4_attention_w4_flash_gqa(C.byref(view), group, _n(q), _n(out), _n(stream),
                                            _n(k_out), _n(v_out)))
+
+
+def attention_w4_flash_noalloc(view, q, out, stream=0, k_out=0, v_out=0, group=1):
+    """attention_w4_flash with the split-S partials in the library's built-in device
+    array: no device allocation; rejects calls whose partials do not fit."""
+    check(load().w4_attention_w4_flash_gqa_noalloc(C.byref(view), group, _n(q), _n(out),
+                                                   _n(stream), _n(k_out), _n(v_out)))
 
 
 def attention_fp16_flash(q, k16, v16, out, H, S, D, stream=0, group=1):

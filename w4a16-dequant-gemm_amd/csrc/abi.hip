@@ -114,11 +114,42 @@ int check_kv_common(int H, int S, int D, int gs, int G, const char* who) {
   return W4_OK;
 }
 
+// ---- the entry point that allocates nothing --------------------------------------
+// Split-S partials of w4_attention_w4_flash_gqa_noalloc live in this file-scope
+// device array instead of the grow-only buffer above.  Every GPU the library runs
+// on holds its own copy until the process ends; its address on a device is looked
+// up once, with that device current, and only that address is ever handed to
+// kernels (the array's name is a host-side handle, not a device address).
+constexpr size_t NOALLOC_SCRATCH_FLOATS = (size_t)W4_NOALLOC_SCRATCH_BYTES / sizeof(float);
+__device__ __align__(256) float scratch[NOALLOC_SCRATCH_FLOATS];
+
+constexpr int NOALLOC_MAX_DEVICES = 64;
+std::mutex g_noalloc_mu;
+float* g_noalloc_ptr[NOALLOC_MAX_DEVICES] = {};
+
+// Device address of `scratch` on the current device (looked up on first use).
+hipError_t noalloc_scratch(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lk(g_noalloc_mu);
+  if (!g_noalloc_ptr[dev]) {
+    float* ptr = nullptr;
+    e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!ptr) return hipErrorInvalidSymbol;
+    g_noalloc_ptr[dev] = ptr;
+  }
+  *out = g_noalloc_ptr[dev];
+  return hipSuccess;
+}
+
 int run_flash(w4k::FlashArgs& a, w4_stream stream, const char* what) {
-  float* scratch = nullptr;
-  hipError_t e = scratch_floats(w4k::flash_scratch_floats(a), &scratch);
+  float* part = nullptr;
+  hipError_t e = scratch_floats(w4k::flash_scratch_floats(a), &part);
   if (e != hipSuccess) return runtime("flash scratch", e);
-  return done(what, w4k::launch_flash(a, scratch, (hipStream_t)stream));
+  return done(what, w4k::launch_flash(a, part, (hipStream_t)stream));
 }
 
 }  // namespace
@@ -232,6 +263,27 @@ int w4_attention_w4_flash_gqa(const w4_kv_view* p, int group, const w4_half* q, 
   fill_w4(a, p, group);
   a.q = q; a.out = out; a.k_out = k_out; a.v_out = v_out;
   return run_flash(a, stream, "flash_w4");
+}
+
+int w4_attention_w4_flash_gqa_noalloc(const w4_kv_view* p, int group, const w4_half* q,
+                                      w4_half* out, w4_stream stream, w4_half* k_out,
+                                      w4_half* v_out) {
+  if (int rc = check_kv_w4(p, "kv flash")) return rc;
+  REQUIRE(q && out, "kv flash w4: null pointer");
+  REQUIRE(group >= 1 && group <= 64, "kv flash w4: bad query group");
+  w4k::FlashArgs a;
+  fill_w4(a, p, group);
+  a.q = q; a.out = out; a.k_out = k_out; a.v_out = v_out;
+  // Same kernels and the same split plan as w4_attention_w4_flash_gqa: only where
+  // the partials live differs, so the two give the same output bytes.  Phase 1
+  // writes every partial phase 2 reads, so nothing needs clearing between calls.
+  REQUIRE(w4k::flash_scratch_floats(a) <= NOALLOC_SCRATCH_FLOATS,
+          "kv flash w4 noalloc: split-S partials exceed the built-in scratch "
+          "(heads * group * splits * (D + 2) floats must fit W4_NOALLOC_SCRATCH_BYTES)");
+  float* part = nullptr;
+  hipError_t e = noalloc_scratch(&part);
+  if (e != hipSuccess) return runtime("flash noalloc scratch", e);
+  return done("flash_w4", w4k::launch_flash(a, part, (hipStream_t)stream));
 }
 
 int w4_attention_w4_flash(const w4_kv_view* p, const w4_half* q, w4_half* out,

@@ -88,3 +88,19 @@ def test_quantize_contracts():
         c.gemm_mx_w4a8(w, c.act_mx8_view(2, 64, 3, 16, one), one)
     with pytest.raises(ValueError, match="null pointer"):
         c.quantize_mx8_f16(x8, 0, one)
+
+
+def test_noalloc_entry_contracts_without_a_device():
+    """The entry point that allocates nothing validates like w4_attention_w4_flash_gqa
+    and rejects partials beyond its built-in array before any device call."""
+    c = w4amd.capi()
+    one = 256
+    with pytest.raises(ValueError, match="null pointer"):
+        c.attention_w4_flash_noalloc(c.kv_view(1, 64, 128, 32, 4, 1, one, one, 0, one, one, 0), 0, one)
+    with pytest.raises(ValueError, match="G inconsistent"):
+        c.attention_w4_flash_noalloc(c.kv_view(1, 64, 128, 32, 3, 1, one, one, 0, one, one, 0), one, one)
+    with pytest.raises(ValueError, match="bad query group"):
+        c.attention_w4_flash_noalloc(c.kv_view(1, 64, 128, 32, 4, 1, one, one, 0, one, one, 0), one, one, group=65)
+    # 512 splits x 64 query heads x 130 floats = 17 MB of partials
+    with pytest.raises(ValueError, match="exceed the built-in scratch"):
+        c.attention_w4_flash_noalloc(c.kv_view(1, 1 << 19, 128, 32, 4, 1, one, one, 0, one, one, 0), one, one, group=64)

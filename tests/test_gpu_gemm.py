@@ -62,7 +62,11 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         # long K (8, 11 and 14 chunks of 128 per wave; the last waves own fewer when K / 128 is no
         # multiple of 8: 86 chunks at K = 11008, 57 at K = 7296, 81 at K = 10368)
         (16, 256, 11008, 128), (64, 512, 14336, 64), (5, 128, 8192, 32), (33, 96, 7296, 128),
-        (100, 64, 10368, 96)]
+        (100, 64, 10368, 96),
+        # four rows per wave (N % 16 == 0, K = 2048 / 4096 / 8192, gs 32 ... 256): one to four
+        # activation rows, one to eight scale loads per lane
+        (3, 32, 4096, 32), (4, 48, 2048, 64), (2, 32, 8192, 32), (1, 16, 4096, 256), (4, 16, 4096, 128),
+        (1, 4096, 4096, 128), (2, 11008, 4096, 128), (1, 64, 2048, 32)]
 TOL, CROSS = 1e-3, 2e-3  # rel L2 vs the FP64 oracle; between two gated paths
 
 

@@ -13,7 +13,7 @@ LIB = os.path.join(PKG, "lib", "libw4amd.so")
 BENCH_LIB = os.path.join(PKG, "lib", "libw4bench.so")
 SOURCES = ["abi.hip", "dequant.hip", "gemm_simt.hip", "gemm_mfma.hip", "flash.hip", "flash_mfma.hip", "quantize.hip", "gemm_mxnative.hip", "gemm_tile_dma.hip", "gemm_decode_resident.hip",
            "baseline.hip"]
-HEADERS = ["dq.cuh", "kernels.h", "bench_kernels.hip", os.path.join("..", "..", "include", "w4_abi.h")]
+HEADERS = ["dq.cuh", "kernels.h", "simt_rows4.cuh", "bench_kernels.hip", os.path.join("..", "..", "include", "w4_abi.h")]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed-FP32 VALU forms stay off for every kernel in this library
@@ -67,9 +67,11 @@ def build(force=False, verbose=True):
     subprocess.check_call(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs,
                            "-lhipblaslt"])
     # bandwidth yardsticks used only by bench.py
-    subprocess.check_call(["hipcc", *[f for f in FLAGS if not f.startswith("-W")], "-shared",
-                           os.path.join(CSRC, "bench_kernels.hip"), "-o", BENCH_LIB],
-                          stderr=subprocess.DEVNULL)
+    bench_src = os.path.join(CSRC, "bench_kernels.hip")
+    if (force or not os.path.exists(BENCH_LIB)
+            or os.path.getmtime(BENCH_LIB) < max(hdr_t, os.path.getmtime(bench_src))):
+        subprocess.check_call(["hipcc", *[f for f in FLAGS if not f.startswith("-W")], "-shared",
+                               bench_src, "-o", BENCH_LIB], stderr=subprocess.DEVNULL)
     return LIB
 
 

@@ -1,45 +1,128 @@
-// Bandwidth yardsticks for the benchmark (not part of the C ABI the tests
-// bind): a streaming read that folds every dwordx4 into a register, and a
-// dwordx4 copy.  The measured rates are the denominators the fused kernels'
-// achieved GB/s are compared with, next to the 8 TB/s HBM3E figure.
+// Kernels of the benchmark only (libw4bench.so; not part of the C ABI the tests
+// bind): the bandwidth yardsticks, the launch-floor probes and the time-stamped
+// form of the decode-shape vector kernel.
+//
+// Yardsticks: a streaming read that folds every dwordx4 into a register, and a
+// dwordx4 copy.  Each workgroup owns one contiguous chunk and walks it in 4 KiB
+// blocks with eight loads in flight per lane; a grid-stride walk of the same
+// buffer measures 0.8 of these rates.  They are the denominators the fused
+// kernels' achieved GB/s are compared with, next to the 8 TB/s HBM3E figure.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "simt_rows4.cuh"
+
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 
-__global__ __launch_bounds__(256) void stream_read(const u4* __restrict__ src, size_t n16,
+constexpr int YARD_U = 8;  // loads in flight per lane
+
+__global__ __launch_bounds__(256) void stream_read(const u4* __restrict__ src, size_t per,
                                                    uint32_t* __restrict__ sink) {
-  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  const size_t stride = (size_t)gridDim.x * 256;
+  const u4* p = src + (size_t)blockIdx.x * per + threadIdx.x;
   u4 acc = {0u, 0u, 0u, 0u};
-  for (; i + 3 * stride < n16; i += 4 * stride) {
-    const u4 a = __builtin_nontemporal_load(src + i);
-    const u4 b = __builtin_nontemporal_load(src + i + stride);
-    const u4 c = __builtin_nontemporal_load(src + i + 2 * stride);
-    const u4 d = __builtin_nontemporal_load(src + i + 3 * stride);
-    acc ^= a ^ b ^ c ^ d;
+  for (size_t i = 0; i < per; i += 256 * YARD_U) {
+    u4 v[YARD_U];
+#pragma unroll
+    for (int u = 0; u < YARD_U; ++u) v[u] = __builtin_nontemporal_load(p + i + u * 256);
+#pragma unroll
+    for (int u = 0; u < YARD_U; ++u) acc ^= v[u];
   }
-  for (; i < n16; i += stride) acc ^= __builtin_nontemporal_load(src + i);
   const uint32_t r = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
   if (r == 0x9E3779B9u) sink[0] = r;  // practically never; keeps the loads alive
 }
 
 __global__ __launch_bounds__(256) void stream_copy(const u4* __restrict__ src,
-                                                   u4* __restrict__ dst, size_t n16) {
-  size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  const size_t stride = (size_t)gridDim.x * 256;
-  for (; i < n16; i += stride) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+                                                   u4* __restrict__ dst, size_t per) {
+  const u4* p = src + (size_t)blockIdx.x * per + threadIdx.x;
+  u4* d = dst + (size_t)blockIdx.x * per + threadIdx.x;
+  for (size_t i = 0; i < per; i += 256 * YARD_U) {
+    u4 v[YARD_U];
+#pragma unroll
+    for (int u = 0; u < YARD_U; ++u) v[u] = __builtin_nontemporal_load(p + i + u * 256);
+#pragma unroll
+    for (int u = 0; u < YARD_U; ++u) __builtin_nontemporal_store(v[u], d + i + u * 256);
+  }
 }
 
+// bytes must be a multiple of blocks * 256 * 16 * YARD_U (the callers use 1 GiB).
 extern "C" int w4bench_read(const void* src, size_t bytes, void* sink, int blocks, void* stream) {
-  stream_read<<<blocks, 256, 0, (hipStream_t)stream>>>((const u4*)src, bytes / 16, (uint32_t*)sink);
+  if (blocks < 1 || bytes % ((size_t)blocks * 256 * 16 * YARD_U)) return (int)hipErrorInvalidValue;
+  stream_read<<<blocks, 256, 0, (hipStream_t)stream>>>((const u4*)src, bytes / 16 / blocks,
+                                                       (uint32_t*)sink);
   return (int)hipGetLastError();
 }
 
 extern "C" int w4bench_copy(const void* src, void* dst, size_t bytes, int blocks, void* stream) {
-  stream_copy<<<blocks, 256, 0, (hipStream_t)stream>>>((const u4*)src, (u4*)dst, bytes / 16);
+  if (blocks < 1 || bytes % ((size_t)blocks * 256 * 16 * YARD_U)) return (int)hipErrorInvalidValue;
+  stream_copy<<<blocks, 256, 0, (hipStream_t)stream>>>((const u4*)src, (u4*)dst, bytes / 16 / blocks);
   return (int)hipGetLastError();
 }
+
+// ---- launch-floor probes ----------------------------------------------------------
+// What a launch costs before it does any arithmetic: a kernel that does nothing,
+// and a kernel that only reads a weight matrix with the grid and the access
+// pattern of the decode-shape vector kernel (every lane `per` dwordx4 loads, all
+// requested before the first is consumed, folded with one XOR each).
+__global__ __launch_bounds__(256) void probe_empty(uint32_t* sink) {
+  if (sink == (uint32_t*)1) sink[0] = 1u;
+}
+
+template <int PER>
+__global__ __launch_bounds__(256) void probe_read(const u4* __restrict__ src,
+                                                  uint32_t* __restrict__ sink) {
+  // workgroup b reads the contiguous run [b * 256 * PER, (b + 1) * 256 * PER) of dwordx4
+  const u4* p = src + (size_t)blockIdx.x * 256 * PER + threadIdx.x;
+  u4 v[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) v[i] = __builtin_nontemporal_load(p + i * 256);
+  u4 a = v[0];
+#pragma unroll
+  for (int i = 1; i < PER; ++i) a ^= v[i];
+  if ((a[0] ^ a[1] ^ a[2] ^ a[3]) == 0x9E3779B9u) sink[0] = 1u;
+}
+
+extern "C" int w4bench_probe_empty(int blocks, void* sink, void* stream) {
+  probe_empty<<<blocks, 256, 0, (hipStream_t)stream>>>((uint32_t*)sink);
+  return (int)hipGetLastError();
+}
+
+// Reads `bytes` (a multiple of 32 KiB) with bytes / 32768 workgroups of 256 lanes,
+// eight dwordx4 per lane: the grid of the decode-shape kernel on the same matrix
+// (16 rows of K = 4096 per workgroup).
+extern "C" int w4bench_probe_read(const void* src, size_t bytes, void* sink, void* stream) {
+  if (bytes % 32768) return (int)hipErrorInvalidValue;
+  probe_read<8><<<(unsigned)(bytes / 32768), 256, 0, (hipStream_t)stream>>>((const u4*)src,
+                                                                            (uint32_t*)sink);
+  return (int)hipGetLastError();
+}
+
+// `steps` back-to-back launches of one probe, rotating through `nsrc` matrices
+// (kind 0: probe_empty with `blocks` workgroups, 1: probe_read of `bytes` each).
+extern "C" int w4bench_probe_loop(int kind, const void* const* srcs, int nsrc, size_t bytes,
+                                  int blocks, void* sink, int steps, void* stream) {
+  for (int i = 0; i < steps; ++i) {
+    const int rc = kind == 0 ? w4bench_probe_empty(blocks, sink, stream)
+                             : w4bench_probe_read(srcs[i % nsrc], bytes, sink, stream);
+    if (rc) return rc;
+  }
+  return 0;
+}
+
+// The decode-shape vector kernel on W4 symmetric gs = 128, K = 4096, M = 1, with
+// time stamps: stamps receives N / 4 waves x ROWS4_STAMPS uint64 (10 ns ticks):
+// [0] wave start, [1] all requests issued, [2] activations landed, [3] group
+// parameters read back, [4 + i] run i landed (i < 8), [12] arithmetic done,
+// [13] reduced; [23] compute die of the wave.
+extern "C" int w4bench_c1_timeline(const void* q, const void* scales, const void* x, void* c,
+                                   int N, void* stamps, void* stream) {
+  if (N < 16 || N % 16) return (int)hipErrorInvalidValue;
+  w4k::simt_rows4_kernel<0, 1, 2, false, 7, true>
+      <<<N / 16, w4k::SIMT_WAVES * 64, 0, (hipStream_t)stream>>>(
+          (const uint32_t*)q, scales, nullptr, (const w4_half*)x, (w4_half*)c, N, 1,
+          (uint64_t*)stamps);
+  return (int)hipGetLastError();
+}
+extern "C" int w4bench_c1_timeline_slots(void) { return w4k::ROWS4_STAMPS; }
 
 // Host-side launch loop: `steps` back-to-back calls of one GEMM entry point,
 // rotating through `nviews` weight views, without returning to the caller's

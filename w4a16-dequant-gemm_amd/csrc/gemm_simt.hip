@@ -24,10 +24,10 @@
 
 #include "dq.cuh"
 #include "kernels.h"
+#include "simt_rows4.cuh"
 
 namespace w4k {
 
-constexpr int SIMT_WAVES = 4;           // waves per workgroup
 constexpr int SIMT_R = 2;               // weight rows per wave
 constexpr int SIMT_LDS_HALVES = 16384;  // activations resident in LDS at once (32 KiB)
 
@@ -464,195 +464,13 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_unrolled_kernel(
   }
 }
 
-// ---- decode shapes, four rows per wave -----------------------------------------------
-// K = STEPS * 2048, N a multiple of 16, one group per 32-k lane slice with a
-// power-of-two group size (or MXFP4), no hook.  What a launch of this size spends
-// its time on, measured with time stamps inside the waves (N = K = 4096): 0.25 us
-// until the first request leaves a wave (argument fetch, address arithmetic), 0.4 us
-// until the first weights arrive, then 17 vector instructions per packed word on one
-// wave per SIMD -- as long as the stream itself -- and a reduce-and-store tail.
-// Hence:
-//  * every argument is a scalar or a pointer, so they arrive in SGPRs with the wave
-//    (the build preloads the kernarg segment) instead of through a scalar load;
-//  * 256 workgroups of 4 waves x 4 rows: one wave per SIMD, half the waves to
-//    launch, and the activations cross L2 -> CU once per 16 rows (through LDS, two
-//    16-byte loads per lane and one barrier, both under the latency of the weights);
-//  * the scales (and zero-point words) of a wave's four rows are one contiguous run:
-//    one load per lane into the wave's own LDS region instead of 4 * STEPS gathers,
-//    each with its own address arithmetic, in front of the weight requests;
-//  * requests go out in the order activations, scales, weights (memory returns them
-//    in that order) and every 1 KiB of a row is expanded as soon as it has landed
-//    (hand-placed vmcnt waits), so arithmetic overlaps the rest of the stream.
-// The order of additions is that of simt_fast_kernel / simt_unrolled_kernel (one
-// chain per lane over steps, words and pairs, then the DPP wave sum): same bytes.
-#define W4_GLOAD16_NT(dst, ptr) asm volatile("global_load_dwordx4 %0, %1, off nt" : "=v"(dst) : "v"(ptr) : "memory")
-#define W4_GLOAD16(dst, ptr) asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(ptr) : "memory")
-#define W4_GLOAD4(dst, ptr) asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(ptr) : "memory")
-
-template <int CNT>
-__device__ __forceinline__ void vm_wait() {
-  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(CNT) : "memory");
-}
-// The register was written by an asm load; from here on the compiler may read it.
-template <class T>
-__device__ __forceinline__ void landed(T& v) {
-  asm volatile("" : "+v"(v)::"memory");
-}
-
-constexpr int ROWS4_R = 4;
-
-template <int MX, int MT, int STEPS, bool ASYM, int GSH>
-__global__ __launch_bounds__(SIMT_WAVES * 64) void simt_rows4_kernel(
-    const uint32_t* __restrict__ q, const void* __restrict__ scales,
-    const uint32_t* __restrict__ zeros, const w4_half* __restrict__ x, w4_half* __restrict__ c,
-    const int N, const int M) {
-  constexpr int R = ROWS4_R, K = STEPS * 2048, WPR = K / 8, NQ = R * STEPS;
-  constexpr int G = MX ? K / 32 : (K >> GSH);             // groups (blocks) per row
-  constexpr int SB = MX ? R * G : R * G * 2;              // scale bytes of a wave's rows
-  constexpr int SD = SB / 4;                              // ... as dwords
-  constexpr int NSL = (SD + 63) / 64;                     // scale loads per lane
-  constexpr int WG = (G + 7) / 8;                         // zero-point words per row
-  constexpr int NZL = ASYM ? (R * WG + 63) / 64 : 0;      // zero-point loads per lane
-  constexpr int XL = MT * STEPS;                          // activation loads per thread
-  __shared__ u4 xs[MT * STEPS * 256];
-  __shared__ uint32_t ss[SIMT_WAVES][NSL * 64];
-  __shared__ uint32_t zs[SIMT_WAVES][ASYM ? NZL * 64 : 1];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n0 = (blockIdx.x * SIMT_WAVES + wave) * R;
-  const int m0 = blockIdx.y * MT;
-
-  u4 xv[XL], qw[NQ];
-  uint32_t sw[NSL], zw[ASYM ? NZL : 1];
-#pragma unroll
-  for (int t = 0; t < XL; ++t) {
-    const int i = t * SIMT_WAVES * 64 + threadIdx.x;
-    const int m = min(i / (STEPS * 256), M - 1 - m0), g8 = i % (STEPS * 256);
-    W4_GLOAD16(xv[t], x + (size_t)(m0 + m) * K + g8 * 8);  // rows past M: a valid row, never stored
-  }
-  const uint32_t* srun = (const uint32_t*)((const uint8_t*)scales + (size_t)n0 * (SB / R));
-#pragma unroll
-  for (int t = 0; t < NSL; ++t) {
-    const int i = min(t * 64 + lane, SD - 1);
-    W4_GLOAD4(sw[t], srun + i);
-  }
-#pragma unroll
-  for (int t = 0; t < NZL; ++t) {
-    const int i = min(t * 64 + lane, R * WG - 1);
-    W4_GLOAD4(zw[t], zeros + (size_t)n0 * WG + i);
-  }
-#pragma unroll
-  for (int i = 0; i < NQ; ++i) {  // block-major: the four rows of a 2048-k block share its activations
-    const int st = i / R, r = i % R;
-    W4_GLOAD16_NT(qw[i], q + (size_t)(n0 + r) * WPR + st * 256 + lane * 4);
-  }
-
-  vm_wait<NQ + NZL + NSL>();  // activations
-#pragma unroll
-  for (int t = 0; t < XL; ++t) {
-    landed(xv[t]);
-    const int i = t * SIMT_WAVES * 64 + threadIdx.x;
-    const int m = i / (STEPS * 256), g8 = i % (STEPS * 256);
-    const int slot = (g8 & ~255) + (g8 & 3) * 64 + ((g8 & 255) >> 2);
-    xs[m * STEPS * 256 + slot] = MX ? xv[t] : pair_strided(xv[t]);
-  }
-  vm_wait<NQ>();  // scales and zero-points: into this wave's own LDS region
-#pragma unroll
-  for (int t = 0; t < NSL; ++t) {
-    landed(sw[t]);
-    ss[wave][t * 64 + lane] = sw[t];
-  }
-#pragma unroll
-  for (int t = 0; t < NZL; ++t) {
-    landed(zw[t]);
-    zs[wave][t * 64 + lane] = zw[t];
-  }
-  __syncthreads();
-
-  // group parameters of this lane's slices, read back from LDS
-  uint32_t sc[NQ];
-  int zp[NQ];
-#pragma unroll
-  for (int i = 0; i < NQ; ++i) {
-    const int st = i / R, r = i % R;
-    const int g = MX ? st * 64 + lane : (st * 2048 + lane * 32) >> GSH;
-    if (MX) sc[i] = ((const uint8_t*)ss[wave])[r * G + g];
-    else sc[i] = ((const uint16_t*)ss[wave])[r * G + g];
-    zp[i] = ASYM ? (int)((zs[wave][r * WG + (g >> 3)] >> (4 * (g & 7))) & 0xFu) : 8;
-  }
-
-  float acc[R][MT];
-#pragma unroll
-  for (int r = 0; r < R; ++r)
-#pragma unroll
-    for (int m = 0; m < MT; ++m) acc[r][m] = 0.0f;
-
-  // step i expands the 1 KiB run (2048-k block i / R, row i % R); the runs were
-  // requested in this order, so run i has landed when at most NQ - 1 - i are outstanding
-  u4 xr[MT][4];
-  auto step = [&](auto ic) {
-    constexpr int i = decltype(ic)::value;
-    constexpr int st = i / R, r = i % R;
-    __builtin_amdgcn_sched_barrier(0);
-    if (r == 0) {
-#pragma unroll
-      for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) xr[m][j] = xs[m * STEPS * 256 + st * 256 + j * 64 + lane];
-    }
-    vm_wait<(NQ - 1 - i > 0 ? NQ - 1 - i : 0)>();
-    landed(qw[i]);
-    const float mxs = mx_scale(sc[i]);
-    const W4Group grp = w4_group((uint16_t)sc[i], zp[i]);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      h2 d[4];
-      if (MX) dq_mx(qw[i][j], mxs, d);
-      else dq_w4(qw[i][j], grp, d);
-#pragma unroll
-      for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[r][m] = dot2(d[e], as_h2(xr[m][j][e]), acc[r][m]);
-    }
-  };
-  // (a row's chain still runs over its blocks in ascending k, as in the other kernels)
-#define W4_STEP(I) \
-  if constexpr (I < NQ) step(std::integral_constant<int, I>{});
-  W4_STEP(0) W4_STEP(1) W4_STEP(2) W4_STEP(3) W4_STEP(4) W4_STEP(5) W4_STEP(6) W4_STEP(7)
-  W4_STEP(8) W4_STEP(9) W4_STEP(10) W4_STEP(11) W4_STEP(12) W4_STEP(13) W4_STEP(14) W4_STEP(15)
-#undef W4_STEP
-  static_assert(NQ <= 16, "steps are spelled out up to 16");
-
-#pragma unroll
-  for (int r = 0; r < R; ++r)
-#pragma unroll
-    for (int m = 0; m < MT; ++m) acc[r][m] = wave_sum_to_lane63(acc[r][m]);
-  if (lane == 63) {
-#pragma unroll
-    for (int m = 0; m < MT; ++m) {
-      if (m0 + m >= M) continue;
-      uint16_t h[R];
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        const _Float16 v = (_Float16)acc[r][m];
-        h[r] = __builtin_bit_cast(uint16_t, v);
-      }
-      // N is a multiple of 16 and c is 8-byte aligned: the four rows leave as one store
-      *(u2*)(c + (size_t)(m0 + m) * N + n0) =
-          u2{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16)};
-    }
-  }
-}
-#undef W4_GLOAD16_NT
-#undef W4_GLOAD16
-#undef W4_GLOAD4
-
 template <int MX, int MT, int STEPS>
 static hipError_t launch_rows4(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s) {
   const dim3 grid((unsigned)(v.N / (SIMT_WAVES * ROWS4_R)), (unsigned)((M + MT - 1) / MT));
   const int gsh = MX ? 5 : __builtin_ctz((unsigned)v.gs);
 #define W4_GO(ASYM, GSH)                                                               \
-  simt_rows4_kernel<MX, MT, STEPS, ASYM, GSH><<<grid, SIMT_WAVES * 64, 0, s>>>(        \
-      v.q, v.scales, v.zeros, x, c, v.N, M)
+  simt_rows4_kernel<MX, MT, STEPS, ASYM, GSH, false><<<grid, SIMT_WAVES * 64, 0, s>>>( \
+      v.q, v.scales, v.zeros, x, c, v.N, M, nullptr)
 #define W4_GSH(ASYM)                                          \
   switch (gsh) {                                              \
     case 5: W4_GO(ASYM, 5); break;                            \

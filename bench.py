@@ -291,24 +291,8 @@ def mx_bytes(N, K, M):
     return N * ((K + 7) // 8) * 4 + N * ((K + 31) // 32) + 2 * M * K + 2 * M * N
 
 
-# ---- the configs' data distributions (host, seeded) ---------------------------------
-def weights_c2(np, orc, N, K, gs, seed):
-    """0.02 * N(0,1); one in ten (row, group)s made one-sided (all positive)."""
-    w = (orc.normal_weights(N * K, seed) * 0.02).reshape(N, K)
-    G = (K + gs - 1) // gs
-    one_sided = np.random.default_rng(seed ^ 0x51DE).random((N, G)) < 0.10
-    mask = one_sided[:, np.arange(K) // gs]
-    w[mask] = np.abs(w[mask])
-    return w.ravel()
-
-
-def weights_c3(np, orc, N, K, seed):
-    """0.02 * N(0,1); one element in a hundred replaced by an outlier of +-20 sigma."""
-    w = orc.normal_weights(N * K, seed) * 0.02
-    rng = np.random.default_rng(seed ^ 0x0071)
-    idx = rng.random(N * K) < 0.01
-    w[idx] = np.where(rng.random(int(idx.sum())) < 0.5, -1.0, 1.0) * (20 * 0.02)
-    return w
+# The configs' data distributions (10 % one-sided groups; 1 % outliers at 20 sigma) are
+# orc.one_sided_group_weights and orc.outlier_weights, shared with the test suite.
 
 
 def quant_rel_l2(np, w, w16):
@@ -448,7 +432,7 @@ def extras_gemm(b, full):
     rows, gates = [], []
     shapes = [(11008, 4096, 128), (11008, 4096, 32), (11008, 4096, 48), (11008, 4104, 8)]
     for si, (N, K, gs) in enumerate(shapes):
-        w = weights_c2(np, orc, N, K, gs, 0xC2C2 + si)
+        w = orc.one_sided_group_weights(N, K, gs, 0xC2C2 + si)
         p = orc.quantize(w, N, K, gs, False)
         w_ref = orc.dequant_all(p)
         qerr = quant_rel_l2(np, w, w_ref)
@@ -481,7 +465,7 @@ def extras_gemm(b, full):
     # C3: MXFP4 N=14336 K=4096, 1 % outliers; format error against W4 gs=128 on the same W
     rows = []
     N, K = 14336, 4096
-    w = weights_c3(np, orc, N, K, 0xE40F)
+    w = orc.outlier_weights(N, K, 0xE40F)
     t0 = time.perf_counter()
     p = orc.quantize_mx(w, N, K)
     t_qmx = time.perf_counter() - t0

@@ -105,6 +105,26 @@ def uniform_int_stream(seed, rng, n):
     return out
 
 
+# ---- the benchmark configs' weight distributions ----------------------------
+def one_sided_group_weights(N, K, gs, seed, sigma=0.02, fraction=0.10):
+    """sigma * N(0,1); `fraction` of the (row, group)s made one-sided (all positive)."""
+    w = (normal_weights(N * K, seed) * sigma).reshape(N, K)
+    G = (K + gs - 1) // gs
+    one_sided = np.random.default_rng(seed ^ 0x51DE).random((N, G)) < fraction
+    mask = one_sided[:, np.arange(K) // gs]
+    w[mask] = np.abs(w[mask])
+    return w.ravel()
+
+
+def outlier_weights(N, K, seed, sigma=0.02, fraction=0.01, at=20.0):
+    """sigma * N(0,1); `fraction` of the elements replaced by an outlier of +-`at` sigma."""
+    w = normal_weights(N * K, seed) * sigma
+    rng = np.random.default_rng(seed ^ 0x0071)
+    idx = rng.random(N * K) < fraction
+    w[idx] = np.where(rng.random(int(idx.sum())) < 0.5, -1.0, 1.0) * (at * sigma)
+    return w
+
+
 # ---- W4 --------------------------------------------------------------------
 class PackedW:
     def __init__(self, N, K, gs, symmetric, q, scales, zeros):

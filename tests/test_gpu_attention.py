@@ -362,3 +362,40 @@ def test_paged_batched_prefix_sharing(D):
         o = halves(Hkv * group * D, 0x7E00)
         c.attention_w4_flash(dk.view, ptr(to_dev(qs[s])), ptr(o), group=group)
         assert np.array_equal(bits(o), got[s]), "paged batch == contiguous, bytewise"
+
+
+@pytest.mark.parametrize("sym", [True, False], ids=["sym", "asym"])
+def test_w4_flash_batch_plan_of_64_slabs_by_32768_positions(sym):
+    """The split plan of the batch-8, 8-kv-head decode step: 64 slabs of 32768 positions give
+    8 splits per slab and 32 tiles of 32 positions per wave, with 4 query heads per slab.
+    The 64 slabs are 4 oracle-quantized sample slabs repeated (slab i holds sample i % 4), so
+    hooks and outputs are checked against four slabs' worth of oracle work; everything is
+    compared on the device."""
+    c = w4amd.capi()
+    H, NS, S, D, gs, group = 64, 4, 32768, 128, 32, 4
+    seed = 0xB8B8 + (0 if sym else 1)
+    c4 = orc.quantize_cache(orc.normal_weights(NS * S * D, seed), orc.normal_weights(NS * S * D, seed + 1),
+                            NS, S, D, gs, sym)
+    kd, vd = orc.dequant_cache(c4, False), orc.dequant_cache(c4, True)
+    q = orc.normal_activations(H * group * D, seed + 2)
+    idx = torch.arange(H, device="cuda") % NS
+
+    def rep(a):
+        return to_dev(np.ascontiguousarray(a).reshape(NS, -1))[idx].contiguous()
+    t = [rep(c4.q_k), rep(c4.s_k), None if sym else rep(c4.z_k), rep(c4.q_v), rep(c4.s_v),
+         None if sym else rep(c4.z_v)]
+    view = c.kv_view(H, S, D, gs, c4.G, sym, *[ptr(a) for a in t])
+    q_d = to_dev(q)
+    out, out2 = halves(H * group * D, 0x7E00), halves(H * group * D, 0x7E00)
+    ko, vo = halves(H * S * D, 0x7E00), halves(H * S * D, 0x7E00)
+    c.attention_w4_flash(view, ptr(q_d), ptr(out), 0, ptr(ko), ptr(vo), group=group)
+    assert torch.equal(ko.view(H, -1), to_dev(kd).view(NS, -1)[idx]), "k_out bitwise"
+    assert torch.equal(vo.view(H, -1), to_dev(vd).view(NS, -1)[idx]), "v_out bitwise"
+    del ko, vo
+    c.attention_w4_flash(view, ptr(q_d), ptr(out2), group=group)
+    assert torch.equal(out, out2), "hooked and unhooked bytes differ"
+    got = bits(out2).view(np.float16).reshape(H, group, D)
+    for i in (0, 9, 18, 27, 63):  # slabs of five different sequences, all four samples
+        ref = orc.attention_f16(q.reshape(H, group * D)[i], kd[i % NS:i % NS + 1], vd[i % NS:i % NS + 1],
+                                1, group, S, D)
+        assert orc.rel_l2(got[i], ref) <= TOL

@@ -142,6 +142,73 @@ def test_mx_gemm_gates(i):
     assert np.array_equal(cd, want) and np.array_equal(wd, w_ref)
 
 
+# The benchmark configs' own data and shapes at a reduced N: asymmetric weights with one
+# (row, group) in ten one-sided, K = 4096 with gs 32 / 48 / 128 and K = 4104 with gs 8,
+# M swept over the crossover; MXFP4 with one element in a hundred at 20 sigma, K = 4096
+# and the ragged K = 72 / 100, M = 1 / 16 / 128.
+C2_SHAPES = [(4096, 32), (4096, 48), (4096, 128), (4104, 8)]
+
+
+@pytest.mark.parametrize("M", [1, 2, 4, 8, 9, 16, 64])
+@pytest.mark.parametrize("ks", range(len(C2_SHAPES)))
+def test_w4_asym_one_sided_groups_crossover_sweep(ks, M):
+    c = w4amd.capi()
+    K, gs = C2_SHAPES[ks]
+    N = 352  # 11008 / 32 rounded to whole 16-row tiles
+    seed = 0xC2C2 + ks
+    w = orc.one_sided_group_weights(N, K, gs, seed)
+    p = orc.quantize(w, N, K, gs, False)
+    assert p.zeros is not None and (orc_nibbles(p.zeros, N, p.G) == 0).any(), "no one-sided group"
+    w_ref = orc.dequant_all(p)
+    x = orc.normal_activations(M * K, seed + 100 + M)
+    ref = orc.gemm_oracle(x, M, K, w_ref, N)
+    dp, x_d = DevPacked(p), to_dev(x)
+    for fn in (c.gemm_fused, c.gemm_mma, c.gemm):
+        cf, wf = _run(fn, dp.view, x_d, M, N, K)
+        assert np.array_equal(wf, w_ref), "w_out bitwise"
+        assert orc.rel_l2(cf.view(np.float16), ref) <= TOL
+        cf2, _ = _run(fn, dp.view, x_d, M, N, K, hook=False)
+        assert np.array_equal(cf, cf2), "hooked and unhooked bytes differ"
+
+
+def orc_nibbles(words_, rows, n):
+    w = words_.reshape(rows, -1)
+    sh = (4 * np.arange(8, dtype=np.uint32))[None, None, :]
+    return ((w[:, :, None] >> sh) & 0xF).reshape(rows, -1)[:, :n]
+
+
+@pytest.mark.parametrize("M", [1, 16, 128])
+@pytest.mark.parametrize("K", [4096, 72, 100])
+def test_mx_outlier_weights(K, M):
+    c = w4amd.capi()
+    N = 448  # 14336 / 32
+    seed = 0xE40F + K
+    w = orc.outlier_weights(N, K, seed)
+    p = orc.quantize_mx(w, N, K)
+    w_ref = orc.dequant_all_mx(p)
+    # the no-saturation scale rule holds with the outliers in: no element clips at 6 * 2^e
+    err = np.abs(w_ref.view(np.float16).astype(np.float64) - w)
+    assert err.max() <= 0.5 * 20 * 0.02, "an outlier was clipped"
+    x = orc.normal_activations(M * K, seed + M)
+    ref = orc.gemm_oracle(x, M, K, w_ref, N)
+    dp, x_d = DevPackedMx(p), to_dev(x)
+    w_d = halves(N * K, 0x7E00)
+    c.dequant_mx(dp.view, ptr(w_d))
+    assert np.array_equal(bits(w_d), w_ref), "mx dequant bitwise"
+    for fn in ((c.gemm_fused_mx, c.gemm_mma_mx, c.gemm_mx) if M <= 16 else (c.gemm_mma_mx, c.gemm_mx)):
+        cf, wf = _run(fn, dp.view, x_d, M, N, K)
+        assert np.array_equal(wf, w_ref), "w_out bitwise"
+        assert orc.rel_l2(cf.view(np.float16), ref) <= TOL
+        cf2, _ = _run(fn, dp.view, x_d, M, N, K, hook=False)
+        assert np.array_equal(cf, cf2)
+    # format error against W4 gs = 128 on the same matrix (needs K a multiple of 8 only)
+    if K == 4096:
+        w4 = orc.dequant_all(orc.quantize(w, N, K, 128, True))
+        e_mx = np.sqrt(np.sum((w_ref.view(np.float16).astype(np.float64) - w) ** 2) / np.sum(w * w))
+        e_w4 = np.sqrt(np.sum((w4.view(np.float16).astype(np.float64) - w) ** 2) / np.sum(w * w))
+        assert e_mx < e_w4, "per-32 block scales should beat per-128 group scales on outliers"
+
+
 def test_w4_dequant_exhaustive_scales():
     """Every FP16 scale x every code x every zero-point: the device dequant step
     equals RNE_half(float(s) * (q - z)) bit for bit (NaN scales excluded)."""

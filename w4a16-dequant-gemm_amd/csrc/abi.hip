@@ -76,24 +76,33 @@ int check_mx(const w4_packed_mx_view* p) {
   return W4_OK;
 }
 
-// Grow-only device scratch for the split-S partials, shared by all calls (calls
-// on different streams must not overlap, as with the reference's
-// kv_part_scratch, kvflash.cuh:56-69).
+// Grow-only device scratch for the split-S partials, one per device, shared by all
+// calls on that device (calls on different streams must not overlap, as with the
+// reference's kv_part_scratch, kvflash.cuh:56-69).
+constexpr int MAX_DEVICES = 64;
 std::mutex g_scratch_mu;
-float* g_scratch = nullptr;
-size_t g_scratch_cap = 0;
+float* g_scratch[MAX_DEVICES] = {};
+size_t g_scratch_cap[MAX_DEVICES] = {};
 
 hipError_t scratch_floats(size_t n, float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
   std::lock_guard<std::mutex> lk(g_scratch_mu);
-  if (n > g_scratch_cap) {
+  if (n > g_scratch_cap[dev]) {
     float* nb = nullptr;
-    hipError_t e = hipMalloc((void**)&nb, n * sizeof(float));
+    e = hipMalloc((void**)&nb, n * sizeof(float));
     if (e != hipSuccess) return e;
-    if (g_scratch) (void)hipFree(g_scratch);
-    g_scratch = nb;
-    g_scratch_cap = n;
+    // a call still in flight may be using the old buffer: let the device drain first
+    if (g_scratch[dev]) {
+      (void)hipDeviceSynchronize();
+      (void)hipFree(g_scratch[dev]);
+    }
+    g_scratch[dev] = nb;
+    g_scratch_cap[dev] = n;
   }
-  *out = g_scratch;
+  *out = g_scratch[dev];
   return hipSuccess;
 }
 
@@ -123,7 +132,7 @@ int check_kv_common(int H, int S, int D, int gs, int G, const char* who) {
 constexpr size_t NOALLOC_SCRATCH_FLOATS = (size_t)W4_NOALLOC_SCRATCH_BYTES / sizeof(float);
 __device__ __align__(256) float scratch[NOALLOC_SCRATCH_FLOATS];
 
-constexpr int NOALLOC_MAX_DEVICES = 64;
+constexpr int NOALLOC_MAX_DEVICES = MAX_DEVICES;
 std::mutex g_noalloc_mu;
 float* g_noalloc_ptr[NOALLOC_MAX_DEVICES] = {};
 

@@ -340,10 +340,15 @@ static hipError_t launch_decode_mt(const WView& v, const w4_half* x, w4_half* c,
 }
 
 // Hooked calls of the shapes the resident-activation kernel takes with 17 <= M <= 64
-// (gs % 32 == 0, 16-byte aligned rows): same K split, same order of additions.
+// (gs % 32 == 0, 16-byte aligned rows): same K split, same order of additions.  Only
+// that instantiation exists for more than 16 activation rows, so anything else is
+// rejected here rather than run on loads and group lookups it does not fit.
 template <int FMT, int MT>
 static hipError_t launch_decode_hooked_mt(const WView& v, const w4_half* x, w4_half* c, int M,
-                                          hipStream_t s, w4_half* w_out) {
+                                          hipStream_t s, w4_half* w_out, bool wvec) {
+  const bool gs32 = v.mx || v.gs % 32 == 0;
+  if (!w_out || !wvec || !gs32 || (((uintptr_t)w_out | (uintptr_t)x) & 15))
+    return hipErrorInvalidValue;
   int gs_shift = -1;
   if (!v.mx && (v.gs & (v.gs - 1)) == 0) gs_shift = __builtin_ctz((unsigned)v.gs);
   const dim3 grid((unsigned)((v.N + 15) / 16), (unsigned)((M + 16 * MT - 1) / (16 * MT)));
@@ -356,8 +361,8 @@ template <int FMT>
 static hipError_t launch_decode(const WView& v, const w4_half* x, w4_half* c, int M,
                                 hipStream_t s, w4_half* w_out, bool wvec) {
   if (M <= 16) return launch_decode_mt<FMT, 1>(v, x, c, M, s, w_out, wvec);
-  if (M <= 32) return launch_decode_hooked_mt<FMT, 2>(v, x, c, M, s, w_out);
-  return launch_decode_hooked_mt<FMT, 4>(v, x, c, M, s, w_out);
+  if (M <= 32) return launch_decode_hooked_mt<FMT, 2>(v, x, c, M, s, w_out, wvec);
+  return launch_decode_hooked_mt<FMT, 4>(v, x, c, M, s, w_out, wvec);  // grid.y walks 64 rows at a time
 }
 
 // ---- streaming decode-batch kernel --------------------------------------------------

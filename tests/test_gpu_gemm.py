@@ -66,7 +66,11 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         # four rows per wave (N % 16 == 0, K = 2048 / 4096 / 8192, gs 32 ... 256): one to four
         # activation rows, one to eight scale loads per lane
         (3, 32, 4096, 32), (4, 48, 2048, 64), (2, 32, 8192, 32), (1, 16, 4096, 256), (4, 16, 4096, 128),
-        (1, 4096, 4096, 128), (2, 11008, 4096, 128), (1, 64, 2048, 32)]
+        (1, 4096, 4096, 128), (2, 11008, 4096, 128), (1, 64, 2048, 32),
+        # M <= 64 with group parameters through LDS: odd group sizes, ragged K, one and two
+        # tiles per workgroup, one / two / four activation row tiles, 2 .. 5 chunks per wave
+        (9, 4128, 4096, 48), (50, 4128, 4104, 8), (16, 8208, 2048, 24), (64, 4112, 3072, 48),
+        (30, 64, 5000, 40), (8, 32, 1160, 8), (33, 48, 2568, 16)]
 TOL, CROSS = 1e-3, 2e-3  # rel L2 vs the FP64 oracle; between two gated paths
 
 

@@ -1,0 +1,379 @@
+// Decode-batch W4A16 GEMM (M <= 64) for the shapes the resident-activation kernel of
+// gemm_decode_resident.hip does not take: group sizes that are no multiple of 32 (a
+// lane's 32-k slice then spans several groups) and K that is no multiple of 128
+// (K % 8 == 0: whole packed words; rows of words are then only 4-byte aligned).
+// mma.cuh:63-230 is the reference's kernel for this path: any gs % 8 == 0, any K,
+// zero-padded edges.
+//
+// Same structure as the resident-activation kernel -- 8 waves split K by 128-k
+// chunks, a workgroup takes T 16-row tiles and brings its activations in once
+// (global_load_lds_dwordx4 into each wave's own LDS region, XOR-swizzled), partial
+// sums meet in LDS in wave order -- and the same order of additions as
+// mfma_decode_kernel, which serves the hooked calls of these shapes.  What differs:
+//  * group parameters come through LDS.  The scales of a tile's 16 rows are one
+//    contiguous 32-byte-aligned run of 32 G bytes (the zero-point words one of
+//    64 words(G) bytes): the workgroup copies the runs of its T tiles with 16-byte
+//    loads, and every lane then reads the scale and the zero-point word of each of
+//    its packed words from LDS (one group lookup per word, computed once per kernel).
+//    Gathering them from memory costs a separate request per (row, group) touched:
+//    at gs = 48, N = 11008 that was as much as the shared activations saved.
+//  * rows of packed words are read with 16-byte loads at 4-byte aligned addresses
+//    (the memory path takes them at 0.95 of the aligned rate); a slice that runs past
+//    the end of its row is read word by word with the index clamped to the row.
+//  * the last chunk of a row may be partial: its activations beyond K are fetched
+//    from a clamped address and zeroed on the way to the MFMA operands.
+#include "dq.cuh"
+#include "kernels.h"
+
+namespace w4k {
+namespace {
+
+typedef __attribute__((address_space(3))) void* lds_ptr;
+constexpr int DG_WAVES = 8, DG_THREADS = 64 * DG_WAVES;
+constexpr int dg_waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
+extern __shared__ __attribute__((aligned(16))) uint8_t dg_lds[];
+
+// Eight codes of a packed word -> eight FP16 weights in k order (as in the
+// resident-activation kernel): cneg = packed {-(1024 + z), -(64 + z)}, s2 = the scale
+// in both halves, mask / magic = 0x00F0000F / 0x54006400 held in registers.
+__device__ __forceinline__ h8 dg_expand_word(uint32_t w, h2 cneg, h2 s2, uint32_t mask, uint32_t magic) {
+  u4 out;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t p = __builtin_amdgcn_perm(0u, w, 0x0c000c00u | (uint32_t)(i << 16) | (uint32_t)i);
+    const uint32_t v = (p & mask) | magic;
+    out[i] = as_u32((as_h2(v) + cneg) * s2);
+  }
+  return __builtin_bit_cast(h8, out);
+}
+
+// ASYM: zero-points.  CH = ceil(ceil(K / 128) / 8) chunks per wave.  T tiles of 16 rows
+// per workgroup (tile blockIdx.x + gridDim.x t), MT tiles of 16 activation rows
+// (blockIdx.y walks M in steps of 16 MT).  A tile's scales are copied with PS = 3 16-byte
+// loads per thread (2 G <= 1536 of them; indices past the run repeat its last piece and
+// are not written).  Arguments are scalars and pointers so that they arrive preloaded
+// in SGPRs.
+template <bool ASYM, int CH, int T, int MT>
+__global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
+    const uint32_t* __restrict__ q, const w4_half* __restrict__ scales,
+    const uint32_t* __restrict__ zeros, const w4_half* __restrict__ x, w4_half* __restrict__ c,
+    const int N, const int K, const int gs, const int gs_shift, const int G, const int M,
+    const int tiles) {
+  constexpr int PS = 3;
+  const int WPR = K >> 3, nchunks = (K + 127) >> 7, WG = (G + 7) >> 3;
+  constexpr int CP = (4 / MT) < CH ? (4 / MT) : CH;  // chunks per phase
+  constexpr int PH = (CH + CP - 1) / CP;              // phases (the last may be partial)
+  constexpr int XBYTES = MT * CP * 4096;              // the wave's LDS region
+  const int SB = 32 * G, ZB = ASYM ? 64 * WG : 0;     // a tile's scale / zero-point bytes
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int r = lane & 15, b = lane >> 4;
+  const int m0 = (int)blockIdx.y * (16 * MT);
+  // chunk i of this wave (clamped to the row's last chunk) and this lane's first k in it
+  auto chunk_of = [&](int i) { return min(wave * CH + i, nchunks - 1); };
+  auto lane_k = [&](int i) { return chunk_of(i) * 128 + 32 * b; };
+
+  int tile_of[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) tile_of[t] = min((int)blockIdx.x + (int)gridDim.x * t, tiles - 1);
+
+  // ---- requests: activations of phase 0, codes of tile 0, group parameters, other codes ----
+  const uint32_t region = (uint32_t)(uintptr_t)(lds_ptr)dg_lds + (uint32_t)wave * XBYTES;
+  const char* xb = (const char*)x;
+  auto request_x = [&](int ph) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int cc = 0; cc < CP; ++cc)
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq) {
+          if (ph * CP + cc >= CH) continue;
+          const int r16 = 4 * rq + (lane >> 4), row = m0 + 16 * mt + r16;
+          const int cidx = chunk_of(ph * CP + cc);
+          // 16-byte piece (lane % 16) ^ r16 of the chunk's 256 bytes; pieces past K repeat piece 0
+          int piece = (lane & 15) ^ r16;
+          if (cidx * 128 + piece * 8 >= K) piece = 0;
+          const uint32_t off = (uint32_t)min(row, M - 1) * (uint32_t)(K * 2) + (uint32_t)cidx * 256u +
+                               (uint32_t)(piece * 16);
+          const uint32_t dst = region + (uint32_t)((mt * CP + cc) * 4 + rq) * 1024u;
+          asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                       :
+                       : "v"(off), "s"(xb), "s"(dst)
+                       : "memory", "m0");
+        }
+  };
+  u4 qw[T][CH];
+  auto load_tile = [&](int t) {
+    const uint32_t* qr = q + (size_t)(tile_of[t] * 16 + r) * WPR;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const int w0 = lane_k(i) >> 3;
+      if (w0 + 4 <= WPR) {
+        qw[t][i] = __builtin_nontemporal_load((const u4*)(qr + w0));
+      } else {  // the slice runs past the row: word by word, clamped (those words meet zero activations)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) qw[t][i][j] = __builtin_nontemporal_load(qr + min(w0 + j, WPR - 1));
+      }
+    }
+  };
+  request_x(0);
+  load_tile(0);
+  u4 sv[T][PS], zv[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    const u4* sp = (const u4*)((const uint8_t*)scales + (size_t)tile_of[t] * SB);
+#pragma unroll
+    for (int ps = 0; ps < PS; ++ps) {
+      const int i = min(ps * DG_THREADS + (int)threadIdx.x, SB / 16 - 1);
+      sv[t][ps] = sp[i];
+    }
+    if (ASYM) {
+      const u4* zp = (const u4*)((const uint8_t*)zeros + (size_t)tile_of[t] * ZB);
+      zv[t] = zp[min((int)threadIdx.x, ZB / 16 - 1)];
+    }
+  }
+#pragma unroll
+  for (int t = 1; t < T; ++t) load_tile(t);
+  __builtin_amdgcn_sched_barrier(0);  // every request above is issued before the wait below
+
+  // Group of each packed word of this lane (the same for every tile), as byte offsets
+  // into a tile's parameter block: scale at 2 (r G + g), zero-point word at
+  // SB + 4 (r WG + g / 8), nibble g % 8.
+  uint32_t soff[CH][4], zoff[CH][4], zsh[CH][4];
+#pragma unroll
+  for (int i = 0; i < CH; ++i) {
+    int g4[4];
+    groups_of_slice(lane_k(i), gs, gs_shift, G - 1, g4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      soff[i][j] = (uint32_t)(r * G + g4[j]) * 2u;
+      zoff[i][j] = (uint32_t)SB + (uint32_t)(r * WG + (g4[j] >> 3)) * 4u;
+      zsh[i][j] = 4u * (uint32_t)(g4[j] & 7);
+    }
+  }
+
+  // At most the codes of tiles 1 .. T - 1 may still be outstanding (CH vector loads
+  // each; a wave that also issued word-by-word loads waits for more than it must):
+  // phase 0 of x, the codes of tile 0 and the parameter loads have landed.
+  static_assert(CH * (T - 1) < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(dg_waitcnt_vm(CH * (T - 1)));
+  const int PB = SB + ZB;  // parameter block of one tile, behind the x regions
+  uint8_t* params = dg_lds + DG_WAVES * XBYTES;
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+#pragma unroll
+    for (int ps = 0; ps < PS; ++ps) {
+      const int i = ps * DG_THREADS + (int)threadIdx.x;
+      if (i < SB / 16) *(u4*)(params + t * PB + i * 16) = sv[t][ps];
+    }
+    if (ASYM && (int)threadIdx.x < ZB / 16) *(u4*)(params + t * PB + SB + threadIdx.x * 16) = zv[t];
+  }
+  __syncthreads();
+
+  uint32_t mask = 0x00F0000Fu, magic = 0x54006400u;
+  asm volatile("" : "+s"(mask));   // opaque: as literals they cost two instructions
+  asm volatile("" : "+v"(magic));  // instead of one and-or
+  f4 acc[T][MT];
+#pragma unroll
+  for (int t = 0; t < T; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = f4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+  for (int ph = 0; ph < PH; ++ph) {
+    if (ph > 0) __builtin_amdgcn_s_waitcnt(dg_waitcnt_vm(0));  // later phases are the youngest requests
+    // B operands: MFMA j of chunk i contracts k = lane_k(i) + 8 j .. + 7 = piece 4 b + j
+    u4 xv[MT][CP][4];
+    {
+      const uint8_t* mine = dg_lds + wave * XBYTES;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int cc = 0; cc < CP; ++cc)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int i = ph * CP + cc;
+            if (i >= CH) continue;
+            xv[mt][cc][j] = *(const u4*)(mine + ((mt * CP + cc) * 4 + (r >> 2)) * 1024 +
+                                         ((r & 3) * 16 + ((4 * b + j) ^ r)) * 16);
+            // chunks past the row's last one, and k past K inside it, contribute nothing
+            if (wave * CH + i >= nchunks || lane_k(i) + 8 * j >= K) xv[mt][cc][j] = u4{0u, 0u, 0u, 0u};
+          }
+    }
+    if (ph + 1 < PH) {
+      // the region is free once these reads have returned: ask for the next phase now
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+      __builtin_amdgcn_sched_barrier(0);
+      request_x(ph + 1);
+    }
+#pragma unroll
+    for (int t = 0; t < T; ++t)
+#pragma unroll
+      for (int cc = 0; cc < CP; ++cc) {
+        const int i = ph * CP + cc;
+        if (i >= CH) continue;
+        const uint8_t* pt = params + t * PB;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t sbits = *(const uint16_t*)(pt + soff[i][j]);
+          uint32_t z = 8u;
+          if (ASYM) z = (*(const uint32_t*)(pt + zoff[i][j]) >> zsh[i][j]) & 0xFu;
+          const h2 cneg = as_h2(0xD400E400u | (z << 20) | z);
+          const h8 a = dg_expand_word(qw[t][i][j], cneg, splat_bits(sbits), mask, magic);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+            acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(h8, xv[mt][cc][j]),
+                                                                acc[t][mt], 0, 0, 0);
+        }
+      }
+  }
+
+  // Fixed-order combine of the 8 K slices (the x regions are free once every wave is
+  // here): entry (t, mt) of wave w goes to red[w][t MT + mt]; wave w sums the entries
+  // e = w, w + 8, ... in wave order and stores them.
+  constexpr int E = T * MT;
+  static_assert(DG_WAVES * E * 1024 <= DG_WAVES * XBYTES, "reduction buffer fits the x regions");
+  __syncthreads();
+  f4* red = (f4*)dg_lds;  // [DG_WAVES][E][64]
+#pragma unroll
+  for (int t = 0; t < T; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) red[(wave * E + t * MT + mt) * 64 + lane] = acc[t][mt];
+  __syncthreads();
+  for (int e = wave; e < E; e += DG_WAVES) {
+    const int t = e / MT, mt = e % MT;
+    const int tile = (int)blockIdx.x + (int)gridDim.x * t;
+    if (tile >= tiles) continue;
+    f4 s = red[e * 64 + lane];
+#pragma unroll
+    for (int w = 1; w < DG_WAVES; ++w) s += red[(w * E + e) * 64 + lane];
+    const int m = m0 + 16 * mt + r;
+    if (m < M) {  // lane: activation row m, weight rows 16 tile + 4 b .. + 3
+      uint16_t hv[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const _Float16 hh = (_Float16)s[k];
+        hv[k] = __builtin_bit_cast(uint16_t, hh);
+      }
+      *(u2*)(c + (size_t)m * N + tile * 16 + 4 * b) =
+          u2{hv[0] | ((uint32_t)hv[1] << 16), hv[2] | ((uint32_t)hv[3] << 16)};
+    }
+  }
+}
+
+struct GeneralPlan {
+  int ch, t, lds;
+};
+
+// LDS the device grants a workgroup (per-device cache); 0 on error.
+int max_lds_bytes() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < 64 && cached[dev]) return cached[dev];
+  int n = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < 64) cached[dev] = n;
+  return n;
+}
+
+int cu_count() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < 64 && cached[dev]) return cached[dev];
+  int n = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < 64) cached[dev] = n;
+  return n;
+}
+
+// Whether, and how, the kernel takes these arguments: W4 only, whole 16-row tiles,
+// whole packed words, 1024 < K <= 5120 (two to five chunks per wave), M <= 64, aligned
+// activations / outputs / parameter arrays, and LDS for the activations of a
+// workgroup plus the parameter blocks of at least one tile.
+bool general_plan(const WView& v, const w4_half* x, const w4_half* c, int M, GeneralPlan* out) {
+  if (v.mx || M < 1 || M > 64 || v.N % 16 || v.K % 8 || v.gs % 8 || v.gs < 8) return false;
+  const int nchunks = (v.K + 127) / 128, ch = (nchunks + DG_WAVES - 1) / DG_WAVES;
+  if (ch < 2 || ch > 5) return false;
+  if (((uintptr_t)x & 15) || ((uintptr_t)c & 7) || ((uintptr_t)v.q & 3)) return false;
+  if (((uintptr_t)v.scales & 15) || (!v.symmetric && ((uintptr_t)v.zeros & 15))) return false;
+  const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+  const int cp = (4 / mt) < ch ? (4 / mt) : ch;
+  const int xbytes = DG_WAVES * mt * cp * 4096;
+  const int pb = 32 * v.G + (v.symmetric ? 0 : 64 * ((v.G + 7) / 8));
+  const int ps = (2 * v.G + DG_THREADS - 1) / DG_THREADS;
+  if (ps > 3 || (!v.symmetric && 4 * ((v.G + 7) / 8) > DG_THREADS)) return false;
+  const int lds_max = max_lds_bytes(), cus = cu_count();
+  if (lds_max < 1 || cus < 1) return false;
+  int t = (v.N / 16 + cus - 1) / cus;  // one workgroup per compute unit covers N, at most two tiles
+  if (t > 2) t = 2;
+  while (t > 0 && xbytes + t * pb > lds_max) --t;
+  if (t < 1) return false;
+  *out = GeneralPlan{ch, t, xbytes + t * pb};
+  return true;
+}
+
+template <bool ASYM, int CH, int T, int MT>
+hipError_t general_go(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
+                      const GeneralPlan& pl) {
+  // more than 64 KB of LDS has to be granted per device, once per instantiation
+  static bool granted[64] = {};
+  static int granted_bytes[64] = {};
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+  if (dev < 0 || dev >= 64 || !granted[dev] || granted_bytes[dev] < pl.lds) {
+    const hipError_t e =
+        hipFuncSetAttribute((const void*)mfma_decode_general_kernel<ASYM, CH, T, MT>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, pl.lds);
+    if (e != hipSuccess) return e;
+    if (dev >= 0 && dev < 64) granted[dev] = true, granted_bytes[dev] = pl.lds;
+  }
+  const int tiles = v.N / 16;
+  const int sh = (v.gs & (v.gs - 1)) == 0 ? __builtin_ctz((unsigned)v.gs) : -1;
+  const dim3 grid((unsigned)((tiles + T - 1) / T), (unsigned)((M + 16 * MT - 1) / (16 * MT)));
+  mfma_decode_general_kernel<ASYM, CH, T, MT><<<grid, DG_THREADS, pl.lds, s>>>(
+      v.q, (const w4_half*)v.scales, v.zeros, x, c, v.N, v.K, v.gs, sh, v.G, M, tiles);
+  return hipGetLastError();
+}
+
+template <bool ASYM, int CH, int T>
+hipError_t general_mt(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
+                      const GeneralPlan& pl) {
+  if (M <= 16) return general_go<ASYM, CH, T, 1>(v, x, c, M, s, pl);
+  if (M <= 32) return general_go<ASYM, CH, T, 2>(v, x, c, M, s, pl);
+  return general_go<ASYM, CH, T, 4>(v, x, c, M, s, pl);
+}
+
+template <bool ASYM, int CH>
+hipError_t general_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
+                     const GeneralPlan& pl) {
+  return pl.t == 1 ? general_mt<ASYM, CH, 1>(v, x, c, M, s, pl) : general_mt<ASYM, CH, 2>(v, x, c, M, s, pl);
+}
+
+template <bool ASYM>
+hipError_t general_ch(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
+                      const GeneralPlan& pl) {
+  switch (pl.ch) {
+    case 2: return general_t<ASYM, 2>(v, x, c, M, s, pl);
+    case 3: return general_t<ASYM, 3>(v, x, c, M, s, pl);
+    case 4: return general_t<ASYM, 4>(v, x, c, M, s, pl);
+    default: return general_t<ASYM, 5>(v, x, c, M, s, pl);
+  }
+}
+
+}  // namespace
+
+bool decode_general_applies(const WView& v, const w4_half* x, const w4_half* c, int M) {
+  GeneralPlan pl;
+  return general_plan(v, x, c, M, &pl);
+}
+
+// Precondition: decode_general_applies(v, x, c, M); no hook.
+hipError_t launch_decode_general(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s) {
+  GeneralPlan pl;
+  if (!general_plan(v, x, c, M, &pl)) return hipErrorInvalidValue;
+  return v.symmetric ? general_ch<false>(v, x, c, M, s, pl) : general_ch<true>(v, x, c, M, s, pl);
+}
+
+}  // namespace w4k

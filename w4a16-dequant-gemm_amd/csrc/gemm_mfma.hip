@@ -339,21 +339,25 @@ static hipError_t launch_decode_mt(const WView& v, const w4_half* x, w4_half* c,
   return hipGetLastError();
 }
 
-// Hooked calls of the shapes the resident-activation kernel takes with 17 <= M <= 64
-// (gs % 32 == 0, 16-byte aligned rows): same K split, same order of additions.  Only
-// that instantiation exists for more than 16 activation rows, so anything else is
-// rejected here rather than run on loads and group lookups it does not fit.
+// Hooked calls of the shapes the resident-activation kernels take with 17 <= M <= 64:
+// same K split, same order of additions.  Group lookups (one per slice or one per
+// word) and row loads (16-byte or word by word) follow the arguments.
 template <int FMT, int MT>
 static hipError_t launch_decode_hooked_mt(const WView& v, const w4_half* x, w4_half* c, int M,
                                           hipStream_t s, w4_half* w_out, bool wvec) {
   const bool gs32 = v.mx || v.gs % 32 == 0;
-  if (!w_out || !wvec || !gs32 || (((uintptr_t)w_out | (uintptr_t)x) & 15))
-    return hipErrorInvalidValue;
+  if (!w_out || v.K % 8 || (((uintptr_t)w_out | (uintptr_t)x) & 15)) return hipErrorInvalidValue;
   int gs_shift = -1;
   if (!v.mx && (v.gs & (v.gs - 1)) == 0) gs_shift = __builtin_ctz((unsigned)v.gs);
   const dim3 grid((unsigned)((v.N + 15) / 16), (unsigned)((M + 16 * MT - 1) / (16 * MT)));
-  mfma_decode_kernel<FMT, MT, 1, 1, true, true, true>
-      <<<grid, DEC_WAVES * 64, 0, s>>>(v, x, c, M, w_out, gs_shift);
+#define W4_GO(GS, WV) \
+  mfma_decode_kernel<FMT, MT, 1, 1, true, GS, WV><<<grid, DEC_WAVES * 64, 0, s>>>(v, x, c, M, w_out, gs_shift)
+  if (gs32) {
+    if (wvec) W4_GO(true, true); else W4_GO(true, false);
+  } else {
+    if (wvec) W4_GO(false, true); else W4_GO(false, false);
+  }
+#undef W4_GO
   return hipGetLastError();
 }
 
@@ -895,7 +899,11 @@ static hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M
   const bool resident = wvec && decode_resident_applies(v, x, c, M) &&
                         (w_out == nullptr || ((uintptr_t)w_out & 15) == 0);
   if (resident && w_out == nullptr) return launch_decode_resident(v, x, c, M, s);
-  if (!resident) {
+  // ... and of its sibling for odd group sizes and ragged K (M <= 64, W4 only)
+  const bool general = !resident && !MX && decode_general_applies(v, x, c, M) &&
+                       (w_out == nullptr || ((uintptr_t)w_out & 15) == 0);
+  if (general && w_out == nullptr) return launch_decode_general(v, x, c, M, s);
+  if (!resident && !general) {
     if (try_tile_dma(v, x, c, M, s, w_out, &terr)) return terr;
     if (try_tile<MX>(v, x, c, M, s, w_out, &terr)) return terr;
   }
@@ -906,7 +914,7 @@ static hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M
   if (aligned) {
     // Measured on N = 4096 .. 14336, K = 4096 .. 11008: the K-split kernel wins for
     // M <= 16 unless N is large enough to give the streaming kernel a full grid.
-    const bool ksplit = M <= 8 || (M <= 16 && v.N < 8192) || resident;
+    const bool ksplit = M <= 8 || (M <= 16 && v.N < 8192) || resident || general;
     if (ksplit) {
       if (MX) return launch_decode<2>(v, x, c, M, s, w_out, wvec);
       return v.symmetric ? launch_decode<0>(v, x, c, M, s, w_out, wvec)

@@ -51,6 +51,13 @@ bool decode_resident_applies(const WView& v, const w4_half* x, const w4_half* c,
 hipError_t launch_decode_resident(const WView& v, const w4_half* x, w4_half* c, int M,
                                   hipStream_t s);
 
+// gemm_decode_general.hip: M <= 64 for any group size (multiple of 8) and any K % 8 == 0
+// with 1024 < K <= 5120, group parameters through LDS; same order of additions as the
+// K-split decode kernels of gemm_mfma.hip.
+bool decode_general_applies(const WView& v, const w4_half* x, const w4_half* c, int M);
+hipError_t launch_decode_general(const WView& v, const w4_half* x, w4_half* c, int M,
+                                 hipStream_t s);
+
 // flash.hip -- one description for the four cache kinds
 struct FlashArgs {
   int kind;  // 0 FP16, 1 W4, 2 FP8

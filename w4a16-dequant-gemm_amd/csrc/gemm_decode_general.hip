@@ -49,11 +49,11 @@ __device__ __forceinline__ h8 dg_expand_word(uint32_t w, h2 cneg, h2 s2, uint32_
 
 // ASYM: zero-points.  CH = ceil(ceil(K / 128) / 8) chunks per wave.  T tiles of 16 rows
 // per workgroup (tile blockIdx.x + gridDim.x t), MT tiles of 16 activation rows
-// (blockIdx.y walks M in steps of 16 MT).  A tile's scales are copied with PS = 3 16-byte
+// (blockIdx.y walks M in steps of 16 MT); CPX, if not 0, chunks of x per phase.  A tile's scales are copied with PS = 3 16-byte
 // loads per thread (2 G <= 1536 of them; indices past the run repeat its last piece and
 // are not written).  Arguments are scalars and pointers so that they arrive preloaded
 // in SGPRs.
-template <bool ASYM, int CH, int T, int MT>
+template <bool ASYM, int CH, int T, int MT, int CPX>
 __global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
     const uint32_t* __restrict__ q, const w4_half* __restrict__ scales,
     const uint32_t* __restrict__ zeros, const w4_half* __restrict__ x, w4_half* __restrict__ c,
@@ -61,7 +61,10 @@ __global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
     const int tiles) {
   constexpr int PS = 3;
   const int WPR = K >> 3, nchunks = (K + 127) >> 7, WG = (G + 7) >> 3;
-  constexpr int CP = (4 / MT) < CH ? (4 / MT) : CH;  // chunks per phase
+  // chunks per phase: as many as 16 KB per wave hold (4 / MT), or CPX if given (fewer
+  // chunks per phase leave LDS for the parameter blocks of more tiles)
+  constexpr int CPD = CPX > 0 ? CPX : 4 / MT;
+  constexpr int CP = CPD < CH ? CPD : CH;
   constexpr int PH = (CH + CP - 1) / CP;              // phases (the last may be partial)
   constexpr int XBYTES = MT * CP * 4096;              // the wave's LDS region
   const int SB = 32 * G, ZB = ASYM ? 64 * WG : 0;     // a tile's scale / zero-point bytes
@@ -262,7 +265,7 @@ __global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
 }
 
 struct GeneralPlan {
-  int ch, t, lds;
+  int ch, t, cpx, lds;
 };
 
 // LDS the device grants a workgroup (per-device cache); 0 on error.
@@ -299,22 +302,37 @@ bool general_plan(const WView& v, const w4_half* x, const w4_half* c, int M, Gen
   if (((uintptr_t)x & 15) || ((uintptr_t)c & 7) || ((uintptr_t)v.q & 3)) return false;
   if (((uintptr_t)v.scales & 15) || (!v.symmetric && ((uintptr_t)v.zeros & 15))) return false;
   const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
-  const int cp = (4 / mt) < ch ? (4 / mt) : ch;
-  const int xbytes = DG_WAVES * mt * cp * 4096;
   const int pb = 32 * v.G + (v.symmetric ? 0 : 64 * ((v.G + 7) / 8));
   const int ps = (2 * v.G + DG_THREADS - 1) / DG_THREADS;
   if (ps > 3 || (!v.symmetric && 4 * ((v.G + 7) / 8) > DG_THREADS)) return false;
   const int lds_max = max_lds_bytes(), cus = cu_count();
   if (lds_max < 1 || cus < 1) return false;
-  int t = (v.N / 16 + cus - 1) / cus;  // one workgroup per compute unit covers N, at most two tiles
-  if (t > 2) t = 2;
-  while (t > 0 && xbytes + t * pb > lds_max) --t;
+  // tiles per workgroup: enough that one workgroup per compute unit covers N, at most
+  // four; with one activation row tile the x regions may shrink to two chunks per
+  // phase to make room for the parameter blocks
+  int want = (v.N / 16 + cus - 1) / cus;
+  if (want > 4) want = 4;
+  auto fit = [&](int cpd, int* lds) {
+    const int cp = cpd < ch ? cpd : ch;
+    const int xbytes = DG_WAVES * mt * cp * 4096;
+    int t = want;
+    while (t > 0 && xbytes + t * pb > lds_max) --t;
+    *lds = xbytes + t * pb;
+    return t;
+  };
+  int lds = 0, cpx = 0;
+  int t = fit(4 / mt, &lds);
+  if (t < want && mt == 1 && ch > 2) {
+    int lds2 = 0;
+    const int t2 = fit(2, &lds2);
+    if (t2 > t) t = t2, lds = lds2, cpx = 2;
+  }
   if (t < 1) return false;
-  *out = GeneralPlan{ch, t, xbytes + t * pb};
+  *out = GeneralPlan{ch, t, cpx, lds};
   return true;
 }
 
-template <bool ASYM, int CH, int T, int MT>
+template <bool ASYM, int CH, int T, int MT, int CPX>
 hipError_t general_go(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                       const GeneralPlan& pl) {
   // more than 64 KB of LDS has to be granted per device, once per instantiation
@@ -324,7 +342,7 @@ hipError_t general_go(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
   if (dev < 0 || dev >= 64 || !granted[dev] || granted_bytes[dev] < pl.lds) {
     const hipError_t e =
-        hipFuncSetAttribute((const void*)mfma_decode_general_kernel<ASYM, CH, T, MT>,
+        hipFuncSetAttribute((const void*)mfma_decode_general_kernel<ASYM, CH, T, MT, CPX>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, pl.lds);
     if (e != hipSuccess) return e;
     if (dev >= 0 && dev < 64) granted[dev] = true, granted_bytes[dev] = pl.lds;
@@ -332,7 +350,7 @@ hipError_t general_go(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
   const int tiles = v.N / 16;
   const int sh = (v.gs & (v.gs - 1)) == 0 ? __builtin_ctz((unsigned)v.gs) : -1;
   const dim3 grid((unsigned)((tiles + T - 1) / T), (unsigned)((M + 16 * MT - 1) / (16 * MT)));
-  mfma_decode_general_kernel<ASYM, CH, T, MT><<<grid, DG_THREADS, pl.lds, s>>>(
+  mfma_decode_general_kernel<ASYM, CH, T, MT, CPX><<<grid, DG_THREADS, pl.lds, s>>>(
       v.q, (const w4_half*)v.scales, v.zeros, x, c, v.N, v.K, v.gs, sh, v.G, M, tiles);
   return hipGetLastError();
 }
@@ -340,15 +358,25 @@ hipError_t general_go(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
 template <bool ASYM, int CH, int T>
 hipError_t general_mt(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                       const GeneralPlan& pl) {
-  if (M <= 16) return general_go<ASYM, CH, T, 1>(v, x, c, M, s, pl);
-  if (M <= 32) return general_go<ASYM, CH, T, 2>(v, x, c, M, s, pl);
-  return general_go<ASYM, CH, T, 4>(v, x, c, M, s, pl);
+  if (M <= 16) {
+    if constexpr (CH > 2) {
+      if (pl.cpx == 2) return general_go<ASYM, CH, T, 1, 2>(v, x, c, M, s, pl);
+    }
+    return general_go<ASYM, CH, T, 1, 0>(v, x, c, M, s, pl);
+  }
+  if (M <= 32) return general_go<ASYM, CH, T, 2, 0>(v, x, c, M, s, pl);
+  return general_go<ASYM, CH, T, 4, 0>(v, x, c, M, s, pl);
 }
 
 template <bool ASYM, int CH>
 hipError_t general_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                      const GeneralPlan& pl) {
-  return pl.t == 1 ? general_mt<ASYM, CH, 1>(v, x, c, M, s, pl) : general_mt<ASYM, CH, 2>(v, x, c, M, s, pl);
+  switch (pl.t) {
+    case 1: return general_mt<ASYM, CH, 1>(v, x, c, M, s, pl);
+    case 2: return general_mt<ASYM, CH, 2>(v, x, c, M, s, pl);
+    case 3: return general_mt<ASYM, CH, 3>(v, x, c, M, s, pl);
+    default: return general_mt<ASYM, CH, 4>(v, x, c, M, s, pl);
+  }
 }
 
 template <bool ASYM>

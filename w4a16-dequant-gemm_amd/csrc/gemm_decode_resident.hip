@@ -439,7 +439,13 @@ int decode_resident_tiles(const WView& v, const w4_half* x, const w4_half* c, in
     // measured at K = 4096: a pass here 8.6 / 13.7 / 16.5 us at N = 4096 / 11008 / 14336, the
     // large-M kernel on its thinnest grids 25 / 37 / 41 us; both grow with K alike, the
     // fixed part of a pass weighs more at K = 2048
-    const double passes = (M + 63) / 64, pass_us = 5.0 + v.N / 1235.0, tile_us = 18.0 + v.N / 590.0;
+    const double passes = (M + 63) / 64, pass_us = 5.0 + v.N / 1235.0;
+    double tile_us = 18.0 + v.N / 590.0;
+    // up to 128 rows the large-M kernel has 64 x 128 tiles, which fill the chip from
+    // N = 8192 on: 20 - 23 us (MXFP4) and 24 - 25 us (W4) for 65 <= M <= 128 at N = 11008
+    // and 14336, where two passes here take 26 and 30 us
+    const bool tile_gs = v.mx || v.gs == 32 || v.gs == 64 || v.gs % 128 == 0;  // what that kernel takes
+    if (M <= 128 && v.N >= 4096 && v.K == 4096 && tile_gs) tile_us = v.mx ? 21.0 : 24.5;
     if (passes * pass_us >= tile_us * (v.K == 2048 ? 0.8 : 1.0)) return 0;
   }
   const int cus = device_cus();

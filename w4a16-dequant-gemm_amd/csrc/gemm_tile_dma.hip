@@ -469,7 +469,7 @@ hipError_t launch_gsm(int gsm, const WView& v, const w4_half* x, w4_half* c, w4_
 }  // namespace
 
 // Takes MXFP4 weights and W4 weights whose groups tile a 128-k stage (gs 32, 64 or a
-// multiple of 128), K a multiple of 128, operands under 4 GiB (32-bit offsets),
+// multiple of 128), M >= 65, K a multiple of 128, operands under 4 GiB (32-bit offsets),
 // 16-byte aligned rows, scales that can be fetched as aligned dwords, and at least
 // eight tiles (measured at N = K = 4096: M = 128, 16 tiles, 44 us against 56 us for
 // the register-staged kernel).  Returns false, launching nothing, otherwise.
@@ -499,7 +499,7 @@ bool try_tile_dma(const WView& v, const w4_half* x, w4_half* c, int M, hipStream
   }
   const long long tiles_n = (shape == 2 || shape == 3) ? n128 : n256;
   const long long tiles_m = (shape == 0 || shape == 3) ? m128 : m64;
-  if (M < 96 || n256 * m128 < 8 || tiles_n * tiles_m > 0x7FFFFFFFLL) return false;
+  if (M < 65 || n256 * m128 < 8 || tiles_n * tiles_m > 0x7FFFFFFFLL) return false;
   if ((long long)v.N * v.K / 2 >= (1LL << 32) || (long long)M * v.K * 2 >= (1LL << 32)) return false;
   // one FP16 scale per stage: the dword around it must lie inside the array
   if (gsm == 0 && (((long long)v.N * v.G) & 1)) return false;

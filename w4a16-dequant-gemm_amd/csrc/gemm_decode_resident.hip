@@ -102,11 +102,50 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
     const int k = chunk_k(i);
     gidx[i] = MX ? (k >> 5) : GSV ? (k >> (8 - GSV)) : POW2 ? (k >> gs_shift) : k / p.gs;
   }
+  // Codes.  The operand layout wants lane (r, b) to hold row r, 32 k of chunk i: fetched
+  // as such, a load instruction takes 64 bytes of each of 16 rows, half of every
+  // 128-byte line it touches, and the memory path moves those at 0.8 of the rate of
+  // whole lines (measured with loads alone on this grid).  So with an even number of
+  // chunks (and rows that are whole lines) the two loads of chunks 2P, 2P + 1 take whole
+  // lines instead: load 2P rows 0..7 of the tile, load 2P + 1 rows 8..15; lane (r, b)
+  // fetches piece b + 4 (r / 8) of its line in the first and piece b + 4 (1 - r / 8) in
+  // the second.  A lane then holds its own row's piece of chunk 2P in one register set
+  // and, in the other, the piece of chunk 2P + 1 that lane r ^ 8 wants: pair_fix()
+  // selects and rotates the rows of 16 lanes by 8, which restores the layout above.
+  constexpr bool PAIRC = CH % 2 == 0;
+  const bool paired = PAIRC && (EXACT || (K & 255) == 0);
   u4 qw[T][CH];
   auto load_tile = [&](int t) {
-    const uint32_t* qr = p.q + nrow[t] * WPR;
+    if (paired) {
+      const uint32_t* qa = p.q + (nrow[t] - (size_t)(r & 8)) * WPR;  // row r % 8 of the tile
+      const uint32_t* qb = qa + (size_t)8 * WPR;                     // row 8 + r % 8
+      const int pa = 4 * (b + 4 * (r >> 3)), pb = 4 * (b + 4 * ((r >> 3) ^ 1));  // piece, in words
 #pragma unroll
-    for (int i = 0; i < CH; ++i) qw[t][i] = __builtin_nontemporal_load((const u4*)(qr + (chunk_k(i) >> 3)));
+      for (int i = 0; i + 1 < CH; i += 2) {
+        const int cidx = wave * CH + i;
+        const int w0 = 16 * ((EXACT || cidx < nchunks) ? cidx : nchunks - 2);
+        qw[t][i] = __builtin_nontemporal_load((const u4*)(qa + w0 + pa));
+        qw[t][i + 1] = __builtin_nontemporal_load((const u4*)(qb + w0 + pb));
+      }
+    } else {
+      const uint32_t* qr = p.q + nrow[t] * WPR;
+#pragma unroll
+      for (int i = 0; i < CH; ++i)
+        qw[t][i] = __builtin_nontemporal_load((const u4*)(qr + (chunk_k(i) >> 3)));
+    }
+  };
+  auto pair_fix = [&](int t) {
+    if (!paired) return;
+    const bool lo = r < 8;
+#pragma unroll
+    for (int i = 0; i + 1 < CH; i += 2)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t a = qw[t][i][e], bb = qw[t][i + 1][e];
+        qw[t][i][e] = lo ? a : bb;
+        // row_ror:8 -- lane r of each row of 16 takes the value of lane r ^ 8
+        qw[t][i + 1][e] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(lo ? bb : a), 0x128, 0xF, 0xF, true);
+      }
   };
   auto load_scales = [&](int t) {
     if constexpr (MX && !EXACT) {
@@ -178,11 +217,7 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
       }
     }
   };
-  // vector loads the scales of all tiles take (between the first x request and the wait)
-  constexpr int SVEC = MX ? 1 : (PER * CH / 2 + 3) / 4;  // vector loads of a tile's scales
   static_assert(EXACT || GSV == 0, "vector scale loads assume K = 1024 CH");
-  constexpr int SLOADS = T * (VEC ? SVEC + ((FMT == 1) ? 1 : 0) : ((FMT == 1) ? 2 * CH : CH));
-  load_tile(0);
 
   // Phase ph of this wave's slice of x -> its LDS region: block (mt, cc, rq) = rows
   // 16 mt + 4 rq .. + 3 of the 128-k chunk CP ph + cc; lane l fetches row l/16 of the
@@ -210,11 +245,27 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
                        : "memory", "m0");
         }
   };
+  // Requests, in the order the memory path will serve them.  The codes of tile t + 1
+  // are requested just before tile t is multiplied, not all up front: a compute
+  // unit's eight waves ask for more than its memory path holds, a wave stands still
+  // at a load until the path takes it, and a wave that had to place every tile's
+  // loads first would start its arithmetic only when most of the stream has gone by
+  // (measured: half of the waves after 3.5 of 7.3 us, the last one with all T tiles
+  // still to expand).  With several tiles the activations go first and a barrier
+  // keeps any wave's codes from overtaking another wave's activations, so that every
+  // wave can start on tile 0 early; with one tile there is nothing to overlap and the
+  // codes, which come from HBM, go first.
+  if (T == 1) load_tile(0);
   request_x(0);
+  if (T > 1) {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    load_tile(0);
+  }
 #pragma unroll
   for (int t = 0; t < T; ++t) load_scales(t);
-#pragma unroll
-  for (int t = 1; t < T; ++t) load_tile(t);
+  if (T > 1) load_tile(1);
   __builtin_amdgcn_sched_barrier(0);  // every request above is issued before the wait below
 
   uint32_t mask = 0x00F0000Fu, magic = 0x54006400u;
@@ -230,8 +281,7 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
   for (int ph = 0; ph < PH; ++ph) {
     // Phase 0 has landed once at most the loads issued after it are outstanding;
     // later phases are the youngest requests of the wave.
-    static_assert(SLOADS + CH * (T - 1) < 64, "vmcnt is a 6-bit counter");
-    if (ph == 0) __builtin_amdgcn_s_waitcnt(waitcnt_vm(SLOADS + CH * (T - 1)));
+    if (ph == 0) __builtin_amdgcn_s_waitcnt(waitcnt_vm(T > 1 ? CH : 0));
     else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     // B operands: MFMA j of chunk i contracts k = kw + 128 i + 8 j .. + 7 = piece 4 b + j
     u4 xv[MT][CP][4];
@@ -256,11 +306,24 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
       request_x(ph + 1);
     }
 #pragma unroll
-    for (int t = 0; t < T; ++t)
+    for (int t = 0; t < T; ++t) {
+      if (ph == 0 && t >= 1) {
+        // request tile t + 1, then wait for tile t: what was requested after it may
+        // still be out (after tile 1: the second phase of x, and tile 2)
+        constexpr int NX1 = PH > 1 ? MT * (CP < CH - CP ? CP : CH - CP) * 4 : 0;
+        static_assert(NX1 + CH < 64, "vmcnt is a 6-bit counter");
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + 1 < T) load_tile(t + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (t == 1) __builtin_amdgcn_s_waitcnt(waitcnt_vm(NX1 + (T > 2 ? CH : 0)));
+        else if (t + 1 < T) __builtin_amdgcn_s_waitcnt(waitcnt_vm(CH));
+        else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+      }
 #pragma unroll
       for (int cc = 0; cc < CP; ++cc) {
         const int i = ph * CP + cc;
         if (i >= CH) continue;
+        if (ph == 0 && cc == 0) pair_fix(t);
         h2 cneg, s2;
         float sf = 0.f;
         if (MX) {
@@ -286,6 +349,7 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
                                                                 acc[t][mt], 0, 0, 0);
         }
       }
+    }
   }
 
   // Fixed-order combine of the 8 K slices.  The x regions are free once every wave

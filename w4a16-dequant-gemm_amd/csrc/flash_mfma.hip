@@ -87,12 +87,14 @@ __device__ __forceinline__ h8 pack8(const h2 v[4]) {
 }
 
 // PAGED: 0 contiguous slabs, 1 pages of a multiple of 16 rows (both halves of a
-// tile lie in one page each), 2 any page size.
-template <int KIND, int DH, bool HOOK, int PAGED, bool ASYM>
+// tile lie in one page each), 2 any page size.  ALT: W4 with zero-points; FP8 with one
+// scale per slab instead of one per row.
+template <int KIND, int DH, bool HOOK, int PAGED, bool ALT>
 __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashArgs a,
                                                                    const int qh0,
                                                                    const int split_len,
                                                                    float* __restrict__ part) {
+  constexpr bool ASYM = KIND == KIND_W4 && ALT, SLAB_SCALE = KIND == KIND_F8 && ALT;
   constexpr int FM_D = DH;       // head dimension
   constexpr int NC = DH / 32;    // MFMAs per score group; a lane's K slice is 8 * NC elements
   constexpr int NB = DH / 8;     // 8-element blocks per row
@@ -102,6 +104,12 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c16 = lane & 15, q4 = lane >> 4;
+  // Row c16 of the score MFMA's A operand holds position kp of the half tile, not
+  // position c16: the result then leaves lane q4 with positions q4, q4 + 4, q4 + 8,
+  // q4 + 12 of each half, so that a V load instruction (the four lanes q4 of an element
+  // block, one position each) takes four neighbouring cache rows -- whole 128-byte
+  // lines -- instead of every fourth row.  The K loads take the same 16 rows either way.
+  const int kp = (c16 >> 2) + 4 * (c16 & 3);
   const int split = blockIdx.y, slab = blockIdx.x, nsplit = gridDim.y;  // slabs on x: no 65535 bound
   const int nh = min(FM_HEADS, a.group - qh0);
   const float inv_sqrt_d = 1.0f / sqrtf((float)FM_D);
@@ -136,7 +144,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     return x;
   };
   _Float16 slab_sk = 0, slab_sv = 0;
-  if (KIND == KIND_F8 && a.scale_mode == 1) slab_sk = as_half(a.s_k[slab]), slab_sv = as_half(a.s_v[slab]);
+  if (SLAB_SCALE) slab_sk = as_half(a.s_k[slab]), slab_sv = as_half(a.s_v[slab]);
 
   const int s0 = split * split_len;
   const int s1 = min(a.S, s0 + split_len);
@@ -186,13 +194,13 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
   const auto rk = rsrc(a.k, ROWB), rv = rsrc(a.v, ROWB);
   const auto rsk = rsrc(a.s_k, 2 * G), rsv = rsrc(a.s_v, 2 * G);
   const auto rzk = rsrc(a.z_k, 4 * wg), rzv = rsrc(a.z_v, 4 * wg);
-  const int kq_off = c16 * ROWB + q4 * (ROWB / 4);  // the lane's quarter of K row c16
-  const int ks_off = 2 * (c16 * G + gk);
-  const int kz_off = 4 * (c16 * wg + (gk >> 3));
-  const int vq_off = 4 * q4 * ROWB + vb * VBB;      // block vb of the first of the lane's 4 V rows
-  const int vs_off = 2 * (4 * q4 * G + gv);
-  const int vz_off = 4 * (4 * q4 * wg + (gv >> 3));
-  const bool row_scales = KIND == KIND_W4 || (KIND == KIND_F8 && a.scale_mode == 0);
+  const int kq_off = kp * ROWB + q4 * (ROWB / 4);  // the lane's quarter of K row kp
+  const int ks_off = 2 * (kp * G + gk);
+  const int kz_off = 4 * (kp * wg + (gk >> 3));
+  const int vq_off = q4 * ROWB + vb * VBB;          // block vb of the first of the lane's 4 V rows
+  const int vs_off = 2 * (q4 * G + gv);
+  const int vz_off = 4 * (q4 * wg + (gv >> 3));
+  constexpr bool row_scales = KIND == KIND_W4 || (KIND == KIND_F8 && !SLAB_SCALE);
 
   // Row, in the slab (in the head's pool when paged), of position t, a multiple
   // of 16 that starts a half tile.  Positions past the last whole half are
@@ -218,7 +226,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
 #pragma unroll
         for (int i = 0; i < KQ; ++i)
           kraw[i] = __builtin_amdgcn_raw_buffer_load_b128(
-              rk, KIND == KIND_F16 ? c16 * ROWB + 2 * kcol(i) : kq_off + 16 * i, rb * ROWB, 2);
+              rk, KIND == KIND_F16 ? kp * ROWB + 2 * kcol(i) : kq_off + 16 * i, rb * ROWB, 2);
       }
       if constexpr (KIND == KIND_W4) {
 #pragma unroll
@@ -240,15 +248,15 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
       for (int r = 0; r < 4; ++r) {
         const int k = 4 * j + r;
         if constexpr (KIND == KIND_W4) {
-          raw.v[k] = __builtin_amdgcn_raw_buffer_load_b32(rv, vq_off, (rb + r) * ROWB, 2);
-          if (ASYM) raw.vz[k] = __builtin_amdgcn_raw_buffer_load_b32(rzv, vz_off, (rb + r) * 4 * wg, 0);
+          raw.v[k] = __builtin_amdgcn_raw_buffer_load_b32(rv, vq_off, (rb + 4 * r) * ROWB, 2);
+          if (ASYM) raw.vz[k] = __builtin_amdgcn_raw_buffer_load_b32(rzv, vz_off, (rb + 4 * r) * 4 * wg, 0);
         } else if constexpr (KIND == KIND_F16) {
-          raw.v[k] = __builtin_amdgcn_raw_buffer_load_b128(rv, vq_off, (rb + r) * ROWB, 2);
+          raw.v[k] = __builtin_amdgcn_raw_buffer_load_b128(rv, vq_off, (rb + 4 * r) * ROWB, 2);
         } else {
-          raw.v[k] = __builtin_amdgcn_raw_buffer_load_b64(rv, vq_off, (rb + r) * ROWB, 2);
+          raw.v[k] = __builtin_amdgcn_raw_buffer_load_b64(rv, vq_off, (rb + 4 * r) * ROWB, 2);
         }
         if constexpr (KIND != KIND_F16) {
-          if (row_scales) raw.vs[k] = as_half(__builtin_amdgcn_raw_buffer_load_b16(rsv, vs_off, (rb + r) * 2 * G, 0));
+          if (row_scales) raw.vs[k] = as_half(__builtin_amdgcn_raw_buffer_load_b16(rsv, vs_off, (rb + 4 * r) * 2 * G, 0));
           else raw.vs[k] = slab_sv;
         }
       }
@@ -266,7 +274,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int t = min(t0 + 16 * j + c16, s1 - 1);
+      const int t = min(t0 + 16 * j + kp, s1 - 1);
       const long long row = phys(t, pg_lo, base_lo, pg_hi, base_hi, j == 1);
       if constexpr (KIND == KIND_W4) {
         const uint32_t* src = (const uint32_t*)a.k + row * WD + NC * q4;
@@ -300,12 +308,12 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
           raw.k[j][0] = u2{t4[0], t4[1]};
           raw.k[j][1] = u2{t4[2], t4[3]};
         }
-        raw.ks[j] = a.scale_mode == 0 ? as_half(a.s_k[row * G + gk]) : slab_sk;
+        raw.ks[j] = SLAB_SCALE ? slab_sk : as_half(a.s_k[row * G + gk]);
       }
     }
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
-      const int t = min(t0 + 16 * (k >> 2) + 4 * q4 + (k & 3), s1 - 1);
+      const int t = min(t0 + 16 * (k >> 2) + q4 + 4 * (k & 3), s1 - 1);
       const long long row = phys(t, pg_lo, base_lo, pg_hi, base_hi, k >= 4);
       if constexpr (KIND == KIND_W4) {
         raw.v[k] = __builtin_nontemporal_load((const uint32_t*)a.v + row * WD + vb);
@@ -315,7 +323,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
         raw.v[k] = __builtin_nontemporal_load((const u4*)((const uint16_t*)a.v + row * FM_D + 8 * vb));
       } else {
         raw.v[k] = __builtin_nontemporal_load((const u2*)((const uint8_t*)a.v + row * FM_D + 8 * vb));
-        raw.vs[k] = a.scale_mode == 0 ? as_half(a.s_v[row * G + gv]) : slab_sv;
+        raw.vs[k] = SLAB_SCALE ? slab_sv : as_half(a.s_v[row * G + gv]);
       }
     }
   };
@@ -346,7 +354,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       sc[j] = f4{0.f, 0.f, 0.f, 0.f};
-      const int t = t0 + 16 * j + c16;
+      const int t = t0 + 16 * j + kp;
       uint16_t* kdst = HOOK ? a.k_out + (hook_base + t) * FM_D : nullptr;
       const bool kst = hook_k && t < s1;
       _Float16 ksc = 0;
@@ -387,7 +395,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     float tmax = -INFINITY;
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
-      const int t = t0 + 16 * (k >> 2) + 4 * q4 + (k & 3);
+      const int t = t0 + 16 * (k >> 2) + q4 + 4 * (k & 3);
       x[k] = WHOLE || t < s1 ? sc[k >> 2][k & 3] : -INFINITY;
       tmax = fmaxf(tmax, x[k]);
     }
@@ -413,12 +421,12 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     // ---- V: expand the 8 positions x 8 elements of this lane so that MFMA e takes
     // element e of every position, accumulate
     auto hook_store_v = [&](int k, const h2 nat[4]) {
-      const int t = t0 + 16 * (k >> 2) + 4 * q4 + (k & 3);
+      const int t = t0 + 16 * (k >> 2) + q4 + 4 * (k & 3);
       if (hook_v && t < s1 && c16 < NB) store16(a.v_out + (hook_base + t) * FM_D + 8 * vb, nat);
     };
     // the 4 elements of a lane of the split layout
     auto hook_store_v4 = [&](int k, const h2 nat[2]) {
-      const int t = t0 + 16 * (k >> 2) + 4 * q4 + (k & 3);
+      const int t = t0 + 16 * (k >> 2) + q4 + 4 * (k & 3);
       if (hook_v && t < s1)
         *(u2*)(a.v_out + (hook_base + t) * FM_D + 8 * vb + 4 * hi8) = u2{as_u32(nat[0]), as_u32(nat[1])};
     };
@@ -524,34 +532,36 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     }
   };
   // A ring slot is refilled right after the tile in it has been consumed, into
-  // the same registers: the loop carries no copies, and FM_DEPTH - 1 tiles are in
+  // the same registers: the loop carries no copies, and DEPTH - 1 tiles are in
   // flight while one is computed.
-  TileRaw<KIND, NC> ring[FM_DEPTH];
+  // (FP8 with row scales: two slots keep two waves per SIMD resident, which pays there)
+  constexpr int DEPTH = KIND == KIND_F8 && !SLAB_SCALE ? 2 : FM_DEPTH;
+  TileRaw<KIND, NC> ring[DEPTH];
 #pragma unroll
-  for (int d = 0; d < FM_DEPTH; ++d) fetch_any(ring[d], d);
+  for (int d = 0; d < DEPTH; ++d) fetch_any(ring[d], d);
   int it0 = 0;
   // Page-table lookups run one tile ahead of the loads that need them, so the
   // scalar load's latency is off the path to the vector loads.
-  int rb_next[2] = {slab_row(tile_start(FM_DEPTH)), slab_row(tile_start(FM_DEPTH) + 16)};
-  for (; it0 + 2 * FM_DEPTH <= nwhole; it0 += FM_DEPTH) {  // computes and fetches whole tiles only
+  int rb_next[2] = {slab_row(tile_start(DEPTH)), slab_row(tile_start(DEPTH) + 16)};
+  for (; it0 + 2 * DEPTH <= nwhole; it0 += DEPTH) {  // computes and fetches whole tiles only
 #pragma unroll
-    for (int d = 0; d < FM_DEPTH; ++d) {
+    for (int d = 0; d < DEPTH; ++d) {
       compute(ring[d], tile_start(it0 + d), std::true_type{});
       __builtin_amdgcn_sched_barrier(0);
       const int rb[2] = {rb_next[0], rb_next[1]};
-      const int t_after = tile_start(it0 + d + FM_DEPTH + 1);
+      const int t_after = tile_start(it0 + d + DEPTH + 1);
       rb_next[0] = slab_row(t_after);
       rb_next[1] = slab_row(t_after + 16);
       fetch_whole(ring[d], rb);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
-  for (; it0 < nit; it0 += FM_DEPTH) {
+  for (; it0 < nit; it0 += DEPTH) {
 #pragma unroll
-    for (int d = 0; d < FM_DEPTH; ++d) {
+    for (int d = 0; d < DEPTH; ++d) {
       if (it0 + d < nit) compute(ring[d], tile_start(it0 + d), std::false_type{});
       __builtin_amdgcn_sched_barrier(0);
-      fetch_any(ring[d], it0 + d + FM_DEPTH);
+      fetch_any(ring[d], it0 + d + DEPTH);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -597,7 +607,7 @@ template <int KIND, bool HOOK, int PAGED>
 static hipError_t go_asym(const FlashArgs& a, int qh0, const FlashPlan& pl, float* part,
                           hipStream_t s) {
   const dim3 grid((unsigned)a.H, (unsigned)pl.nsplit);
-  const bool asym = KIND == KIND_W4 && !a.symmetric;
+  const bool asym = (KIND == KIND_W4 && !a.symmetric) || (KIND == KIND_F8 && a.scale_mode == 1);
 #define W4_GO(DH, ASYM) \
   flash_mfma_phase1<KIND, DH, HOOK, PAGED, ASYM><<<grid, FM_WAVES * 64, 0, s>>>(a, qh0, pl.split_len, part)
   if (a.D == 128) {

@@ -105,8 +105,27 @@ __global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
                        : "memory", "m0");
         }
   };
+  // With an even number of chunks per wave and rows that are whole 128-byte lines the
+  // two loads of chunks 2P, 2P + 1 take whole lines (rows 0..7 of the tile in the
+  // first, 8..15 in the second; lane (r, b) fetches piece b + 4 (r / 8) resp.
+  // b + 4 (1 - r / 8) of its line) and pair_fix() restores the operand layout with a
+  // select and a rotation of the rows of 16 lanes by 8, as in the resident-activation
+  // kernel: loads of 64 bytes out of every line run at 0.8 of the rate.
+  const bool paired = CH % 2 == 0 && (K & 255) == 0;
   u4 qw[T][CH];
   auto load_tile = [&](int t) {
+    if (paired) {
+      const uint32_t* qa = q + (size_t)(tile_of[t] * 16 + (r & 7)) * WPR;
+      const uint32_t* qb = qa + (size_t)8 * WPR;
+      const int pa = 4 * (b + 4 * (r >> 3)), pb = 4 * (b + 4 * ((r >> 3) ^ 1));
+#pragma unroll
+      for (int i = 0; i + 1 < CH; i += 2) {
+        const int w0 = 16 * min(wave * CH + i, nchunks - 2);  // nchunks is even here
+        qw[t][i] = __builtin_nontemporal_load((const u4*)(qa + w0 + pa));
+        qw[t][i + 1] = __builtin_nontemporal_load((const u4*)(qb + w0 + pb));
+      }
+      return;
+    }
     const uint32_t* qr = q + (size_t)(tile_of[t] * 16 + r) * WPR;
 #pragma unroll
     for (int i = 0; i < CH; ++i) {
@@ -118,6 +137,18 @@ __global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
         for (int j = 0; j < 4; ++j) qw[t][i][j] = __builtin_nontemporal_load(qr + min(w0 + j, WPR - 1));
       }
     }
+  };
+  auto pair_fix = [&](int t) {
+    if (!paired) return;
+    const bool lo = r < 8;
+#pragma unroll
+    for (int i = 0; i + 1 < CH; i += 2)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t a = qw[t][i][e], bb = qw[t][i + 1][e];
+        qw[t][i][e] = lo ? a : bb;
+        qw[t][i + 1][e] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(lo ? bb : a), 0x128, 0xF, 0xF, true);
+      }
   };
   request_x(0);
   load_tile(0);
@@ -135,8 +166,10 @@ __global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
       zv[t] = zp[min((int)threadIdx.x, ZB / 16 - 1)];
     }
   }
-#pragma unroll
-  for (int t = 1; t < T; ++t) load_tile(t);
+  // the codes of tile t + 1 are requested just before tile t is multiplied (see the
+  // resident-activation kernel: a wave that has to place every tile's loads first
+  // starts its arithmetic late)
+  if (T > 1) load_tile(1);
   __builtin_amdgcn_sched_barrier(0);  // every request above is issued before the wait below
 
   // Group of each packed word of this lane (the same for every tile), as byte offsets
@@ -155,11 +188,10 @@ __global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
     }
   }
 
-  // At most the codes of tiles 1 .. T - 1 may still be outstanding (CH vector loads
-  // each; a wave that also issued word-by-word loads waits for more than it must):
-  // phase 0 of x, the codes of tile 0 and the parameter loads have landed.
-  static_assert(CH * (T - 1) < 64, "vmcnt is a 6-bit counter");
-  __builtin_amdgcn_s_waitcnt(dg_waitcnt_vm(CH * (T - 1)));
+  // At most the codes of tile 1 may still be outstanding (CH vector loads; a wave that
+  // issued word-by-word loads instead waits for more than it must): phase 0 of x, the
+  // codes of tile 0 and the parameter loads have landed.
+  __builtin_amdgcn_s_waitcnt(dg_waitcnt_vm(T > 1 ? CH : 0));
   const int PB = SB + ZB;  // parameter block of one tile, behind the x regions
   uint8_t* params = dg_lds + DG_WAVES * XBYTES;
 #pragma unroll
@@ -210,11 +242,24 @@ __global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
       request_x(ph + 1);
     }
 #pragma unroll
-    for (int t = 0; t < T; ++t)
+    for (int t = 0; t < T; ++t) {
+      if (ph == 0 && t >= 1) {
+        // request tile t + 1, then wait for tile t: what was requested after it may
+        // still be out (after tile 1: the second phase of x, and tile 2)
+        constexpr int NX1 = PH > 1 ? MT * (CP < CH - CP ? CP : CH - CP) * 4 : 0;
+        static_assert(NX1 + CH < 64, "vmcnt is a 6-bit counter");
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + 1 < T) load_tile(t + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (t == 1) __builtin_amdgcn_s_waitcnt(dg_waitcnt_vm(NX1 + (T > 2 ? CH : 0)));
+        else if (t + 1 < T) __builtin_amdgcn_s_waitcnt(dg_waitcnt_vm(CH));
+        else __builtin_amdgcn_s_waitcnt(dg_waitcnt_vm(0));
+      }
 #pragma unroll
       for (int cc = 0; cc < CP; ++cc) {
         const int i = ph * CP + cc;
         if (i >= CH) continue;
+        if (ph == 0 && cc == 0) pair_fix(t);
         const uint8_t* pt = params + t * PB;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -229,6 +274,7 @@ __global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
                                                                 acc[t][mt], 0, 0, 0);
         }
       }
+    }
   }
 
   // Fixed-order combine of the 8 K slices (the x regions are free once every wave is

@@ -176,6 +176,17 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
       } else if constexpr (DW == 2) {
         const u2 v = *(const u2*)sp;
         w[0] = v[0], w[1] = v[1];
+      } else if constexpr (DW == 8) {
+        // 32 bytes per row: the lower 32 lanes fetch the first 16, the upper 32 the
+        // second 16, and v_permlane32_swap hands each half the other's -- one load
+        // instruction that touches 16 lines instead of two that touch 16 each
+        const u4 v = *(const u4*)(sp + 4 * (lane >> 5));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const auto pr = __builtin_amdgcn_permlane32_swap(v[e], v[e], false, false);
+          w[e] = pr[0];      // lanes 0..31: own, lanes 32..63: that of lane - 32
+          w[4 + e] = pr[1];  // lanes 0..31: that of lane + 32, lanes 32..63: own
+        }
       } else {
 #pragma unroll
         for (int q = 0; q < DW / 4; ++q) {

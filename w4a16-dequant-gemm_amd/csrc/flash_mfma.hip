@@ -104,12 +104,6 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c16 = lane & 15, q4 = lane >> 4;
-  // Row c16 of the score MFMA's A operand holds position kp of the half tile, not
-  // position c16: the result then leaves lane q4 with positions q4, q4 + 4, q4 + 8,
-  // q4 + 12 of each half, so that a V load instruction (the four lanes q4 of an element
-  // block, one position each) takes four neighbouring cache rows -- whole 128-byte
-  // lines -- instead of every fourth row.  The K loads take the same 16 rows either way.
-  const int kp = (c16 >> 2) + 4 * (c16 & 3);
   const int split = blockIdx.y, slab = blockIdx.x, nsplit = gridDim.y;  // slabs on x: no 65535 bound
   const int nh = min(FM_HEADS, a.group - qh0);
   const float inv_sqrt_d = 1.0f / sqrtf((float)FM_D);
@@ -194,12 +188,12 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
   const auto rk = rsrc(a.k, ROWB), rv = rsrc(a.v, ROWB);
   const auto rsk = rsrc(a.s_k, 2 * G), rsv = rsrc(a.s_v, 2 * G);
   const auto rzk = rsrc(a.z_k, 4 * wg), rzv = rsrc(a.z_v, 4 * wg);
-  const int kq_off = kp * ROWB + q4 * (ROWB / 4);  // the lane's quarter of K row kp
-  const int ks_off = 2 * (kp * G + gk);
-  const int kz_off = 4 * (kp * wg + (gk >> 3));
-  const int vq_off = q4 * ROWB + vb * VBB;          // block vb of the first of the lane's 4 V rows
-  const int vs_off = 2 * (q4 * G + gv);
-  const int vz_off = 4 * (q4 * wg + (gv >> 3));
+  const int kq_off = c16 * ROWB + q4 * (ROWB / 4);  // the lane's quarter of K row c16
+  const int ks_off = 2 * (c16 * G + gk);
+  const int kz_off = 4 * (c16 * wg + (gk >> 3));
+  const int vq_off = 4 * q4 * ROWB + vb * VBB;      // block vb of the first of the lane's 4 V rows
+  const int vs_off = 2 * (4 * q4 * G + gv);
+  const int vz_off = 4 * (4 * q4 * wg + (gv >> 3));
   constexpr bool row_scales = KIND == KIND_W4 || (KIND == KIND_F8 && !SLAB_SCALE);
 
   // Row, in the slab (in the head's pool when paged), of position t, a multiple
@@ -226,7 +220,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
 #pragma unroll
         for (int i = 0; i < KQ; ++i)
           kraw[i] = __builtin_amdgcn_raw_buffer_load_b128(
-              rk, KIND == KIND_F16 ? kp * ROWB + 2 * kcol(i) : kq_off + 16 * i, rb * ROWB, 2);
+              rk, KIND == KIND_F16 ? c16 * ROWB + 2 * kcol(i) : kq_off + 16 * i, rb * ROWB, 2);
       }
       if constexpr (KIND == KIND_W4) {
 #pragma unroll
@@ -248,15 +242,15 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
       for (int r = 0; r < 4; ++r) {
         const int k = 4 * j + r;
         if constexpr (KIND == KIND_W4) {
-          raw.v[k] = __builtin_amdgcn_raw_buffer_load_b32(rv, vq_off, (rb + 4 * r) * ROWB, 2);
-          if (ASYM) raw.vz[k] = __builtin_amdgcn_raw_buffer_load_b32(rzv, vz_off, (rb + 4 * r) * 4 * wg, 0);
+          raw.v[k] = __builtin_amdgcn_raw_buffer_load_b32(rv, vq_off, (rb + r) * ROWB, 2);
+          if (ASYM) raw.vz[k] = __builtin_amdgcn_raw_buffer_load_b32(rzv, vz_off, (rb + r) * 4 * wg, 0);
         } else if constexpr (KIND == KIND_F16) {
-          raw.v[k] = __builtin_amdgcn_raw_buffer_load_b128(rv, vq_off, (rb + 4 * r) * ROWB, 2);
+          raw.v[k] = __builtin_amdgcn_raw_buffer_load_b128(rv, vq_off, (rb + r) * ROWB, 2);
         } else {
-          raw.v[k] = __builtin_amdgcn_raw_buffer_load_b64(rv, vq_off, (rb + 4 * r) * ROWB, 2);
+          raw.v[k] = __builtin_amdgcn_raw_buffer_load_b64(rv, vq_off, (rb + r) * ROWB, 2);
         }
         if constexpr (KIND != KIND_F16) {
-          if (row_scales) raw.vs[k] = as_half(__builtin_amdgcn_raw_buffer_load_b16(rsv, vs_off, (rb + 4 * r) * 2 * G, 0));
+          if (row_scales) raw.vs[k] = as_half(__builtin_amdgcn_raw_buffer_load_b16(rsv, vs_off, (rb + r) * 2 * G, 0));
           else raw.vs[k] = slab_sv;
         }
       }
@@ -274,7 +268,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int t = min(t0 + 16 * j + kp, s1 - 1);
+      const int t = min(t0 + 16 * j + c16, s1 - 1);
       const long long row = phys(t, pg_lo, base_lo, pg_hi, base_hi, j == 1);
       if constexpr (KIND == KIND_W4) {
         const uint32_t* src = (const uint32_t*)a.k + row * WD + NC * q4;
@@ -313,7 +307,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     }
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
-      const int t = min(t0 + 16 * (k >> 2) + q4 + 4 * (k & 3), s1 - 1);
+      const int t = min(t0 + 16 * (k >> 2) + 4 * q4 + (k & 3), s1 - 1);
       const long long row = phys(t, pg_lo, base_lo, pg_hi, base_hi, k >= 4);
       if constexpr (KIND == KIND_W4) {
         raw.v[k] = __builtin_nontemporal_load((const uint32_t*)a.v + row * WD + vb);
@@ -354,7 +348,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       sc[j] = f4{0.f, 0.f, 0.f, 0.f};
-      const int t = t0 + 16 * j + kp;
+      const int t = t0 + 16 * j + c16;
       uint16_t* kdst = HOOK ? a.k_out + (hook_base + t) * FM_D : nullptr;
       const bool kst = hook_k && t < s1;
       _Float16 ksc = 0;
@@ -395,7 +389,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     float tmax = -INFINITY;
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
-      const int t = t0 + 16 * (k >> 2) + q4 + 4 * (k & 3);
+      const int t = t0 + 16 * (k >> 2) + 4 * q4 + (k & 3);
       x[k] = WHOLE || t < s1 ? sc[k >> 2][k & 3] : -INFINITY;
       tmax = fmaxf(tmax, x[k]);
     }
@@ -421,12 +415,12 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     // ---- V: expand the 8 positions x 8 elements of this lane so that MFMA e takes
     // element e of every position, accumulate
     auto hook_store_v = [&](int k, const h2 nat[4]) {
-      const int t = t0 + 16 * (k >> 2) + q4 + 4 * (k & 3);
+      const int t = t0 + 16 * (k >> 2) + 4 * q4 + (k & 3);
       if (hook_v && t < s1 && c16 < NB) store16(a.v_out + (hook_base + t) * FM_D + 8 * vb, nat);
     };
     // the 4 elements of a lane of the split layout
     auto hook_store_v4 = [&](int k, const h2 nat[2]) {
-      const int t = t0 + 16 * (k >> 2) + q4 + 4 * (k & 3);
+      const int t = t0 + 16 * (k >> 2) + 4 * q4 + (k & 3);
       if (hook_v && t < s1)
         *(u2*)(a.v_out + (hook_base + t) * FM_D + 8 * vb + 4 * hi8) = u2{as_u32(nat[0]), as_u32(nat[1])};
     };

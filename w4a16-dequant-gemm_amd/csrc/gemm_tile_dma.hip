@@ -30,7 +30,7 @@ namespace {
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
-// rows of W (TN: 256 or 128) and of X (TM: 128 or 64) per workgroup are template parameters
+// rows of W (TN: 256 or 128) and of X (TM: 128, 64 or 32) per workgroup are template parameters
 constexpr int TD_WAVES = 4, TD_THREADS = 64 * TD_WAVES;  // a wave: 64 rows of W x all 128 of X
 constexpr int TD_STAGES = 3;
 // a stage: TN rows of W (64 bytes each), TM rows of X (256 bytes each), two scale dwords and a
@@ -84,7 +84,7 @@ __device__ __forceinline__ h8 expand_word(uint32_t w, h2 cneg, h2 s2, uint32_t m
 // lie in a 128-k stage: 0 one group (gs a multiple of 128), 1 two (gs = 64), 2 four
 // (gs = 32, and the 32-blocks of MXFP4).  A lane's share of a 64-k half is 32
 // consecutive k, so even then it has one scale per half.  G: scales per row.
-// TM: rows of X per workgroup, 128 or 64 (a wave: 64 rows of W x all TM of X).  The
+// TM: rows of X per workgroup, 128, 64 or 32 (a wave: 64 rows of W x all TM of X).  The
 // smaller tile halves a workgroup's walk over K when the grid of the larger one
 // would leave most of the chip idle.
 // TN: rows of W per workgroup, 256 or 128 (a wave: TN / 4 of them = NI tiles of 32).
@@ -446,12 +446,13 @@ hipError_t launch(const WView& v, const w4_half* x, w4_half* c, w4_half* w_out, 
   return hipGetLastError();
 }
 
-// shape: 0 = 128 x 256 (rows of X x rows of W), 1 = 64 x 256, 2 = 64 x 128, 3 = 128 x 128
-// (the hooked kernels exist for the first only)
+// shape: 0 = 128 x 256 (rows of X x rows of W), 1 = 64 x 256, 2 = 64 x 128, 3 = 128 x 128,
+// 4 = 32 x 128 (the hooked kernels exist for the first only)
 template <int FMT, int GSM>
 hipError_t launch_hook(const WView& v, const w4_half* x, w4_half* c, w4_half* w_out, int M,
                        hipStream_t s, int tn, int tm, int shape) {
   if (w_out) return launch<FMT, GSM, true, 128, 256>(v, x, c, w_out, M, s, tn, tm);
+  if (shape == 4) return launch<FMT, GSM, false, 32, 128>(v, x, c, nullptr, M, s, tn, tm);
   if (shape == 3) return launch<FMT, GSM, false, 128, 128>(v, x, c, nullptr, M, s, tn, tm);
   if (shape == 2) return launch<FMT, GSM, false, 64, 128>(v, x, c, nullptr, M, s, tn, tm);
   if (shape == 1) return launch<FMT, GSM, false, 64, 256>(v, x, c, nullptr, M, s, tn, tm);
@@ -484,21 +485,24 @@ bool try_tile_dma(const WView& v, const w4_half* x, w4_half* c, int M, hipStream
   }
   // The smallest of the tile shapes whose grid still fits the chip's 256 compute
   // units in one round: a smaller tile shortens a workgroup's walk over K -- N = K =
-  // 4096, M = 512: 45.6 us with 128 x 256 tiles, 38.1 with 64 x 256, 27.0 with 64 x 128.
+  // 4096, M = 512: 45.6 us with 128 x 256 tiles, 38.1 with 64 x 256, 27.0 with 64 x 128;
+  // M = 256: 23.7 with 64 x 128 (128 workgroups), 21.8 with 32 x 128 (256).  On such grids a
+  // workgroup's K / 128 stages are a chain of 0.6 - 0.7 us each whatever the tile holds.
   // (Hooked
   // and unhooked calls add in the same order whatever the shape: a wave's sums do
   // not depend on how many rows its workgroup holds.)
   const long long n256 = (v.N + 255) / 256, n128 = (v.N + 127) / 128;
-  const long long m128 = (M + 127) / 128, m64 = (M + 63) / 64;
+  const long long m128 = (M + 127) / 128, m64 = (M + 63) / 64, m32 = (M + 31) / 32;
   int shape = 0;
   if (w_out == nullptr) {
     const bool planes3 = gsm == 2 && !v.mx && !v.symmetric;  // needs 256 rows of W per workgroup
-    if (!planes3 && n128 * m64 <= 256) shape = 2;
+    if (!planes3 && n128 * m32 <= 256) shape = 4;
+    else if (!planes3 && n128 * m64 <= 256) shape = 2;
     else if (!planes3 && n128 * m128 <= 256) shape = 3;
     else if (n256 * m64 <= 256) shape = 1;
   }
-  const long long tiles_n = (shape == 2 || shape == 3) ? n128 : n256;
-  const long long tiles_m = (shape == 0 || shape == 3) ? m128 : m64;
+  const long long tiles_n = (shape == 2 || shape == 3 || shape == 4) ? n128 : n256;
+  const long long tiles_m = (shape == 0 || shape == 3) ? m128 : shape == 4 ? m32 : m64;
   if (M < 65 || n256 * m128 < 8 || tiles_n * tiles_m > 0x7FFFFFFFLL) return false;
   if ((long long)v.N * v.K / 2 >= (1LL << 32) || (long long)M * v.K * 2 >= (1LL << 32)) return false;
   // one FP16 scale per stage: the dword around it must lie inside the array

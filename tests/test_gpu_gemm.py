@@ -63,6 +63,9 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         # multiple of 8: 86 chunks at K = 11008, 57 at K = 7296, 81 at K = 10368)
         (16, 256, 11008, 128), (64, 512, 14336, 64), (5, 128, 8192, 32), (33, 96, 7296, 128),
         (100, 64, 10368, 96),
+        # an even number of chunks per wave that is not all there: the last waves' whole-line
+        # pairs are clamped to the row's last pair (58 and 106 chunks for 8 x 8 and 8 x 14 slots)
+        (16, 64, 7424, 128), (40, 48, 13568, 64),
         # four rows per wave (N % 16 == 0, K = 2048 / 4096 / 8192, gs 32 ... 256): one to four
         # activation rows, one to eight scale loads per lane
         (3, 32, 4096, 32), (4, 48, 2048, 64), (2, 32, 8192, 32), (1, 16, 4096, 256), (4, 16, 4096, 128),

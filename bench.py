@@ -131,6 +131,7 @@ class Bench:
         y.w4bench_gemm_loop.argtypes = [vp, vp, ci, vp, vp, ci, ci, vp]
         y.w4bench_w4a4_loop.argtypes = [vp, vp, ci, vp, vp, ci, vp]
         y.w4bench_probe_loop.argtypes = [ci, vp, ci, sz, ci, vp, ci, vp]
+        y.w4bench_gemm_graph.argtypes = [vp, vp, ci, vp, vp, ci, ci, ci, ci, vp]
         y.w4bench_c1_timeline.argtypes = [vp, vp, vp, vp, ci, vp, vp]
         self.yard = y
 
@@ -441,6 +442,18 @@ def extras_floor(b, dps, x_d, c_d, with_c2=True):
     del srcs_c2
     torch.cuda.empty_cache()
     out["c1_timeline"] = b.c1_timeline(dps, x_d, c_d, 4096)
+    # the headline's launches replayed from a HIP graph (200 kernel nodes, one graph launch per
+    # repetition): what is left of the launch-to-launch interval when the host issues nothing
+    from devutil import ptr
+    fn = C.cast(b.capi.load().w4_gemm, C.c_void_p)
+    arr = (C.c_void_p * len(dps))(*[C.addressof(d.view) for d in dps])
+    ms = (C.c_float * 9)()
+    rc = b.yard.w4bench_gemm_graph(fn, arr, len(dps), ptr(x_d), ptr(c_d), 1, 200, 40, 9, ms)
+    if rc:
+        raise RuntimeError("graph replay failed: %d" % rc)
+    reps = [m / 200 * 1e3 for m in ms]
+    out["launch_floor"]["headline_graph_replay_us"] = sorted(reps)[4]
+    out["launch_floor"]["headline_graph_replay_reps_us"] = reps
     return out
 
 

@@ -148,3 +148,51 @@ extern "C" int w4bench_w4a4_loop(w4bench_w4a4_fn fn, const void* const* views, i
   }
   return 0;
 }
+
+// The same launches replayed from a HIP graph: `steps` calls of one GEMM entry point
+// (rotating through the views) are captured once on a stream of the benchmark's own
+// and the graph is launched `warm` + `reps` times; ms[r] receives the time of
+// repetition r (HIP events around one graph launch).  Returns 0 or a hipError_t.
+extern "C" int w4bench_gemm_graph(w4bench_gemm_fn fn, const void* const* views, int nviews,
+                                  const void* x, void* c, int M, int steps, int warm, int reps,
+                                  float* ms) {
+  hipStream_t s = nullptr;
+  hipGraph_t g = nullptr;
+  hipGraphExec_t ge = nullptr;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  int rc = 0;
+#define W4B(call)                         \
+  do {                                    \
+    const hipError_t e_ = (call);         \
+    if (e_ != hipSuccess && rc == 0) rc = (int)e_; \
+  } while (0)
+  W4B(hipStreamCreate(&s));
+  if (rc) return rc;
+  W4B(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+  if (rc == 0) {
+    for (int i = 0; i < steps && rc == 0; ++i)
+      if (fn(views[i % nviews], x, c, M, s, nullptr)) rc = (int)hipErrorUnknown;
+    hipGraph_t got = nullptr;
+    W4B(hipStreamEndCapture(s, &got));  // always ends the capture, also after a failed call
+    g = got;
+  }
+  if (rc == 0) W4B(hipGraphInstantiate(&ge, g, nullptr, nullptr, 0));
+  if (rc == 0) W4B(hipEventCreate(&e0));
+  if (rc == 0) W4B(hipEventCreate(&e1));
+  for (int r = 0; r < warm + reps && rc == 0; ++r) {
+    W4B(hipEventRecord(e0, s));
+    W4B(hipGraphLaunch(ge, s));
+    W4B(hipEventRecord(e1, s));
+    W4B(hipEventSynchronize(e1));
+    float t = 0.f;
+    W4B(hipEventElapsedTime(&t, e0, e1));
+    if (r >= warm) ms[r - warm] = t;
+  }
+#undef W4B
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  if (ge) (void)hipGraphExecDestroy(ge);
+  if (g) (void)hipGraphDestroy(g);
+  (void)hipStreamDestroy(s);
+  return rc;
+}

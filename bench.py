@@ -91,7 +91,7 @@ def _events_ms(torch, fn, steps, warmup):
 # for seconds of back-to-back calls; the decode-batch GEMMs show 8.9 -> 8.3 us.  Every
 # timed region is therefore preceded by SETTLE_MS of the same calls, untimed, on top of
 # the warm-up steps, so that the numbers are the steady state a serving loop sees.
-SETTLE_MS = 30.0
+SETTLE_MS = 60.0
 
 
 def _settle(torch, run, ms_per_call):

@@ -163,11 +163,15 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     }
   }
 
+  // page of a position: a shift when the page size is a power of two (the scalar unit has
+  // no divider: the quotient by a run-time page size is some twenty instructions, twice per tile)
+  const int pshift = PAGED && (a.page & (a.page - 1)) == 0 ? __builtin_ctz((unsigned)a.page) : -1;
+  auto page_of = [&](int t) { return pshift >= 0 ? t >> pshift : t / a.page; };
   // physical cache row of logical position t (t < S)
   auto phys = [&](int t, int pg_lo, long long base_lo, int pg_hi, long long base_hi, bool hi) -> long long {
     if (PAGED == 0) return rows0 + t;
     if (PAGED == 1) return (hi ? base_hi : base_lo) + (t - (hi ? pg_hi : pg_lo) * a.page);
-    const int pg = t / a.page;
+    const int pg = page_of(t);
     return rows0 + (long long)bt[pg] * a.page + (t - pg * a.page);
   };
 
@@ -202,7 +206,7 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
   auto slab_row = [&](int t) -> int {
     if (PAGED == 0) return t;
     const int tc = min(t, max(a.S - 16, 0));
-    const int pg = tc / a.page;
+    const int pg = page_of(tc);
     return bt[pg] * a.page + (tc - pg * a.page);
   };
 
@@ -261,8 +265,8 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     int pg_lo = 0, pg_hi = 0;
     long long base_lo = 0, base_hi = 0;
     if (PAGED == 1) {  // wave-uniform lookups: the page of each 16-position half
-      pg_lo = min(t0, s1 - 1) / a.page;
-      pg_hi = min(t0 + 16, s1 - 1) / a.page;
+      pg_lo = page_of(min(t0, s1 - 1));
+      pg_hi = page_of(min(t0 + 16, s1 - 1));
       base_lo = rows0 + (long long)bt[pg_lo] * a.page;
       base_hi = rows0 + (long long)bt[pg_hi] * a.page;
     }

@@ -88,11 +88,19 @@ __device__ __forceinline__ h8 expand_word(uint32_t w, h2 cneg, h2 s2, uint32_t m
 // smaller tile halves a workgroup's walk over K when the grid of the larger one
 // would leave most of the chip idle.
 // TN: rows of W per workgroup, 256 or 128 (a wave: TN / 4 of them = NI tiles of 32).
-template <int FMT, int GSM, bool HOOK, int TM, int TN>
-__global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
+// KG: sets of four waves per workgroup.  With two, each set walks one half of the K / 128
+// stages through stage buffers of its own (two waves per SIMD, whose instruction streams
+// interleave) and the second set's sums are added to the first set's at the end, through
+// LDS: on the thin grids of the small tiles a workgroup's stages are a chain of 0.6 us
+// each whatever they hold, and this halves the chain.  split_at: the hooked kernel, which
+// always has one set, starts a second accumulator at that stage and adds the two at the
+// end, so that it returns the bytes of the two-set kernel (no split: a stage past the last).
+template <int FMT, int GSM, bool HOOK, int TM, int TN, int KG>
+__global__ __launch_bounds__(TD_THREADS * KG) void w4_tile_dma_kernel(
     const uint32_t* __restrict__ wq, const void* __restrict__ scales,
     const uint32_t* __restrict__ zeros, const w4_half* __restrict__ x, w4_half* __restrict__ c,
-    w4_half* __restrict__ w_out, int N, int K, int G, int gs, int M, int tiles_n, int tiles_m) {
+    w4_half* __restrict__ w_out, int N, int K, int G, int gs, int M, int tiles_n, int tiles_m,
+    int split_at) {
   constexpr bool ASYM = FMT == 1, MX = FMT == 2;
   constexpr int NSC = (!MX && GSM == 2) ? 2 : 1;           // scale dwords per row and stage
   constexpr int TD_TM = TM, MJ = TM / 32;                  // 32-row tiles of X per wave
@@ -103,7 +111,9 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   constexpr int TD_XI = TM * 256 / 1024 / TD_WAVES;        // 1 KB load instructions of X per wave
   constexpr int LOADS = TD_WI + TD_XI + NSC + (ASYM ? 1 : 0);  // load instructions per wave and stage
   const int t = threadIdx.x, lane = t & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // in an SGPR: LDS addresses go to M0
+  const int wave_all = __builtin_amdgcn_readfirstlane(t >> 6);  // in an SGPR: LDS addresses go to M0
+  const int wave = KG == 2 ? (wave_all & 3) : wave_all;        // within its set of four
+  const int grp = KG == 2 ? (wave_all >> 2) : 0;               // the set
   const int r = lane & 31, h = lane >> 5;
   // Consecutive workgroup ids land on different XCDs (each with its own L2): give
   // each XCD a contiguous run of the tile order, m fastest, so that its
@@ -138,6 +148,12 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   const char* xb = (const char*)x;
 
   const int stages = K >> 7;
+  // this set's stages: d_first .. d_first + per_set - 1, those below `stages` (both sets run
+  // per_set iterations so that they meet at every barrier; a stage past the end is fetched
+  // from the last one and not multiplied)
+  const int per_set = (stages + KG - 1) / KG;
+  const int d_first = grp * per_set;
+  const int d_end = min(d_first + per_set, stages) > d_first ? min(d_first + per_set, stages) : d_first + 1;
   // The loads are asm so that the compiler neither tracks them (it would wait for
   // all of them before any LDS read) nor moves LDS reads across them; the vmcnt
   // waits below are by hand.  M0 carries the wave-uniform LDS address.
@@ -158,7 +174,7 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   // a time between the MFMAs of successive steps -- thirteen in a row would hold up
   // its one instruction stream for as long as four steps take.
   auto request_part = [&](int d, uint32_t buf, int part) {  // buf: byte offset of the stage's buffer
-    const uint32_t dd = (uint32_t)(d < stages ? d : stages - 1);  // past the end: valid, never used
+    const uint32_t dd = (uint32_t)(d < d_end ? d : d_end - 1);  // past the set's end: valid, never used
     const uint32_t st = lds0 + buf;
     if (part < TD_WI) {  // the stage's offset goes into the scalar base: no vector arithmetic
       dma16(wqb + dd * 64u, wo[part], st + (wave + TD_WAVES * part) * 1024);
@@ -290,20 +306,35 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   // Stage d + 2 is requested in pieces from step 7 of stage d - 1 (when the barrier
   // there has freed its buffer) to step 6 of stage d.  b0, b1, b2: byte offsets of
   // the buffers of stages d, d + 1, d + 2 (d + 3 takes b0 again).
-  uint32_t b0 = 0, b1 = TD_STAGE, b2 = 2 * TD_STAGE;
-  request(0, b0);
-  request(1, b1);
-  request_part(2, b2, 0);
-  request_part(2, b2, 1);
+  const uint32_t set_base = grp * (TD_STAGES * TD_STAGE);
+  uint32_t b0 = set_base, b1 = set_base + TD_STAGE, b2 = set_base + 2 * TD_STAGE;
+  request(d_first, b0);
+  request(d_first + 1, b1);
+  request_part(d_first + 2, b2, 0);
+  request_part(d_first + 2, b2, 1);
   __builtin_amdgcn_s_waitcnt(waitcnt_vm(LOADS + 2));  // stage 0 has landed
   __syncthreads();
   read_x(xv[0], b0, 0);
   read_w(wv[0], b0, 0);
   read_sc(b0);
-  set_group(0);
-  expand(av[0], 0, 0);
+  set_group(d_first);
+  expand(av[0], d_first, 0);
+  [[maybe_unused]] f16v acc_first[HOOK ? NI : 1][HOOK ? MJ : 1];
 #pragma unroll 1
-  for (int d = 0; d < stages; ++d) {
+  for (int it = 0; it < per_set; ++it) {
+    const int d = d_first + it;
+    if constexpr (HOOK) {
+      if (d == split_at) {  // what the second set of waves of the unhooked kernel starts with
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+#pragma unroll
+          for (int j = 0; j < MJ; ++j) {
+            acc_first[i][j] = acc[i][j];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+          }
+      }
+    }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       if (u == 7) {
@@ -328,12 +359,14 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
         if (u == 0) read_w(wv[1], b0, 1);
         expand(av[(u + 1) & 1], d, u + 1);
       }
+      if (KG == 1 || d < stages) {
 #pragma unroll
-      for (int i = 0; i < NI; ++i)
+        for (int i = 0; i < NI; ++i)
 #pragma unroll
-        for (int j = 0; j < MJ; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-              av[u & 1][i], __builtin_bit_cast(h8, xv[u & 1][j]), acc[i][j], 0, 0, 0);
+          for (int j = 0; j < MJ; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                av[u & 1][i], __builtin_bit_cast(h8, xv[u & 1][j]), acc[i][j], 0, 0, 0);
+      }
       // LDS reads first, then the expansion spread evenly under the MFMAs: a wave
       // can issue about six vector instructions in the shadow of one MFMA
       constexpr int NM = NI * MJ;  // MFMAs of a step
@@ -368,6 +401,36 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
     b2 = first;
   }
   __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));  // nothing may still be writing LDS at exit
+  if constexpr (HOOK) {
+    if (split_at < stages) {
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int j = 0; j < MJ; ++j) acc[i][j] = acc_first[i][j] + acc[i][j];
+    }
+  }
+  if constexpr (KG == 2) {
+    // the second set's sums go to the first through LDS (the stage buffers are free once
+    // every wave is here): first set + second set, in that order
+    __syncthreads();
+    float* mine = (float*)td_lds + (size_t)wave * (NI * MJ * 16 * 64);
+    if (grp == 1) {
+#pragma unroll
+      for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int j = 0; j < MJ; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) mine[((i * MJ + j) * 16 + e) * 64 + lane] = acc[i][j][e];
+    }
+    __syncthreads();
+    if (grp == 1) return;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int j = 0; j < MJ; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] += mine[((i * MJ + j) * 16 + e) * 64 + lane];
+  }
 
   // A lane holds, of each 32 x 32 tile, n = 8 q + 4 h + e for m = tile row r.  Whole
   // tiles go through LDS (free by now) so that every store instruction writes eight
@@ -425,46 +488,52 @@ __global__ __launch_bounds__(TD_THREADS) void w4_tile_dma_kernel(
   }
 }
 
-template <int FMT, int GSM, bool HOOK, int TM, int TN>
+template <int FMT, int GSM, bool HOOK, int TM, int TN, int KG = 1>
 hipError_t launch(const WView& v, const w4_half* x, w4_half* c, w4_half* w_out, int M,
-                  hipStream_t s, int tiles_n, int tiles_m) {
-  constexpr int TD_LDS = td_lds_bytes(TM, TN);
+                  hipStream_t s, int tiles_n, int tiles_m, int split_at) {
+  constexpr int TD_LDS = KG * td_lds_bytes(TM, TN);
+  static_assert(TD_LDS <= 160 * 1024, "the stage buffers of every set of waves fit LDS");
   // more than 64 KB of LDS has to be granted per device, once
   static bool granted[64] = {};
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
   if (dev < 0 || dev >= 64 || !granted[dev]) {
-    const hipError_t e = hipFuncSetAttribute((const void*)w4_tile_dma_kernel<FMT, GSM, HOOK, TM, TN>,
+    const hipError_t e = hipFuncSetAttribute((const void*)w4_tile_dma_kernel<FMT, GSM, HOOK, TM, TN, KG>,
                                              hipFuncAttributeMaxDynamicSharedMemorySize, TD_LDS);
     if (e != hipSuccess) return e;
     if (dev >= 0 && dev < 64) granted[dev] = true;
   }
-  w4_tile_dma_kernel<FMT, GSM, HOOK, TM, TN>
-      <<<dim3((unsigned)(tiles_n * tiles_m)), dim3(TD_THREADS), TD_LDS, s>>>(
+  w4_tile_dma_kernel<FMT, GSM, HOOK, TM, TN, KG>
+      <<<dim3((unsigned)(tiles_n * tiles_m)), dim3(TD_THREADS * KG), TD_LDS, s>>>(
           v.q, v.scales, v.zeros, x, c, w_out, v.N, v.K, v.mx ? v.B : v.G, v.gs, M, tiles_n,
-          tiles_m);
+          tiles_m, split_at);
   return hipGetLastError();
 }
 
 // shape: 0 = 128 x 256 (rows of X x rows of W), 1 = 64 x 256, 2 = 64 x 128, 3 = 128 x 128,
 // 4 = 32 x 128 (the hooked kernels exist for the first only)
+// sets: 2 = the small tiles with two sets of waves (the hooked kernel then splits its sum at
+// split_at, the first stage of the second set)
 template <int FMT, int GSM>
 hipError_t launch_hook(const WView& v, const w4_half* x, w4_half* c, w4_half* w_out, int M,
-                       hipStream_t s, int tn, int tm, int shape) {
-  if (w_out) return launch<FMT, GSM, true, 128, 256>(v, x, c, w_out, M, s, tn, tm);
-  if (shape == 4) return launch<FMT, GSM, false, 32, 128>(v, x, c, nullptr, M, s, tn, tm);
-  if (shape == 3) return launch<FMT, GSM, false, 128, 128>(v, x, c, nullptr, M, s, tn, tm);
-  if (shape == 2) return launch<FMT, GSM, false, 64, 128>(v, x, c, nullptr, M, s, tn, tm);
-  if (shape == 1) return launch<FMT, GSM, false, 64, 256>(v, x, c, nullptr, M, s, tn, tm);
-  return launch<FMT, GSM, false, 128, 256>(v, x, c, nullptr, M, s, tn, tm);
+                       hipStream_t s, int tn, int tm, int shape, int sets, int split_at) {
+  if (w_out) return launch<FMT, GSM, true, 128, 256>(v, x, c, w_out, M, s, tn, tm, split_at);
+  const int none = v.K;  // more than any stage index
+  if (shape == 4 && sets == 2) return launch<FMT, GSM, false, 32, 128, 2>(v, x, c, nullptr, M, s, tn, tm, none);
+  if (shape == 2 && sets == 2) return launch<FMT, GSM, false, 64, 128, 2>(v, x, c, nullptr, M, s, tn, tm, none);
+  if (shape == 4) return launch<FMT, GSM, false, 32, 128>(v, x, c, nullptr, M, s, tn, tm, none);
+  if (shape == 3) return launch<FMT, GSM, false, 128, 128>(v, x, c, nullptr, M, s, tn, tm, none);
+  if (shape == 2) return launch<FMT, GSM, false, 64, 128>(v, x, c, nullptr, M, s, tn, tm, none);
+  if (shape == 1) return launch<FMT, GSM, false, 64, 256>(v, x, c, nullptr, M, s, tn, tm, none);
+  return launch<FMT, GSM, false, 128, 256>(v, x, c, nullptr, M, s, tn, tm, none);
 }
 
 template <int FMT>
 hipError_t launch_gsm(int gsm, const WView& v, const w4_half* x, w4_half* c, w4_half* w_out,
-                      int M, hipStream_t s, int tn, int tm, int shape) {
-  if (gsm == 0) return launch_hook<FMT, 0>(v, x, c, w_out, M, s, tn, tm, shape);
-  if (gsm == 1) return launch_hook<FMT, 1>(v, x, c, w_out, M, s, tn, tm, shape);
-  return launch_hook<FMT, 2>(v, x, c, w_out, M, s, tn, tm, shape);
+                      int M, hipStream_t s, int tn, int tm, int shape, int sets, int split_at) {
+  if (gsm == 0) return launch_hook<FMT, 0>(v, x, c, w_out, M, s, tn, tm, shape, sets, split_at);
+  if (gsm == 1) return launch_hook<FMT, 1>(v, x, c, w_out, M, s, tn, tm, shape, sets, split_at);
+  return launch_hook<FMT, 2>(v, x, c, w_out, M, s, tn, tm, shape, sets, split_at);
 }
 
 }  // namespace
@@ -493,14 +562,22 @@ bool try_tile_dma(const WView& v, const w4_half* x, w4_half* c, int M, hipStream
   // not depend on how many rows its workgroup holds.)
   const long long n256 = (v.N + 255) / 256, n128 = (v.N + 127) / 128;
   const long long m128 = (M + 127) / 128, m64 = (M + 63) / 64, m32 = (M + 31) / 32;
+  // the shape an unhooked call takes; the hooked kernel has 128 x 256 tiles only, but follows
+  // the unhooked call's split of the sum over K (below)
   int shape = 0;
-  if (w_out == nullptr) {
+  {
     const bool planes3 = gsm == 2 && !v.mx && !v.symmetric;  // needs 256 rows of W per workgroup
     if (!planes3 && n128 * m32 <= 256) shape = 4;
     else if (!planes3 && n128 * m64 <= 256) shape = 2;
     else if (!planes3 && n128 * m128 <= 256) shape = 3;
     else if (n256 * m64 <= 256) shape = 1;
   }
+  // The two smallest tiles run with two sets of waves, each on one half of K (their stages
+  // are a serial chain; see the kernel): the sum over K is then (first half) + (second half).
+  const int stages = v.K / 128;
+  const int sets = (shape == 2 || shape == 4) && stages >= 8 ? 2 : 1;
+  const int split_at = sets == 2 ? (stages + 1) / 2 : v.K;
+  if (w_out) shape = 0;
   const long long tiles_n = (shape == 2 || shape == 3 || shape == 4) ? n128 : n256;
   const long long tiles_m = (shape == 0 || shape == 3) ? m128 : shape == 4 ? m32 : m64;
   if (M < 65 || n256 * m128 < 8 || tiles_n * tiles_m > 0x7FFFFFFFLL) return false;
@@ -511,9 +588,9 @@ bool try_tile_dma(const WView& v, const w4_half* x, w4_half* c, int M, hipStream
   if (!v.mx && !v.symmetric && (v.zeros == nullptr || ((uintptr_t)v.zeros & 3))) return false;
   if (w_out && ((uintptr_t)w_out & 15)) return false;
   const int tn = (int)tiles_n, tm = (int)tiles_m;
-  if (v.mx) *err = launch_hook<2, 2>(v, x, c, w_out, M, s, tn, tm, shape);
-  else if (v.symmetric) *err = launch_gsm<0>(gsm, v, x, c, w_out, M, s, tn, tm, shape);
-  else *err = launch_gsm<1>(gsm, v, x, c, w_out, M, s, tn, tm, shape);
+  if (v.mx) *err = launch_hook<2, 2>(v, x, c, w_out, M, s, tn, tm, shape, sets, split_at);
+  else if (v.symmetric) *err = launch_gsm<0>(gsm, v, x, c, w_out, M, s, tn, tm, shape, sets, split_at);
+  else *err = launch_gsm<1>(gsm, v, x, c, w_out, M, s, tn, tm, shape, sets, split_at);
   return true;
 }
 

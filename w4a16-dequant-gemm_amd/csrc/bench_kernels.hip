@@ -118,7 +118,7 @@ extern "C" int w4bench_c1_timeline(const void* q, const void* scales, const void
   if (N < 16 || N % 16) return (int)hipErrorInvalidValue;
   w4k::simt_rows4_kernel<0, 1, 2, false, 7, true>
       <<<N / 16, w4k::SIMT_WAVES * 64, 0, (hipStream_t)stream>>>(
-          (const uint32_t*)q, scales, nullptr, (const w4_half*)x, (w4_half*)c, N, 1,
+          (const uint32_t*)q, scales, nullptr, (const w4_half*)x, (w4_half*)c, N, 1, 128, 32,
           (uint64_t*)stamps);
   return (int)hipGetLastError();
 }

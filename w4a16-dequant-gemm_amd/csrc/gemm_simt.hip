@@ -467,12 +467,16 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_unrolled_kernel(
 template <int MX, int MT, int STEPS>
 static hipError_t launch_rows4(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s) {
   const dim3 grid((unsigned)(v.N / (SIMT_WAVES * ROWS4_R)), (unsigned)((M + MT - 1) / MT));
-  const int gsh = MX ? 5 : __builtin_ctz((unsigned)v.gs);
+  // a power of two 32 .. 256: its shift; any other gs % 8 == 0: 0 (gs >= 32) or 3 (gs >= 8)
+  const bool pow2 = MX || (v.gs & (v.gs - 1)) == 0;
+  const int gsh = MX ? 5 : pow2 && v.gs >= 32 && v.gs <= 256 ? __builtin_ctz((unsigned)v.gs) : v.gs >= 32 ? 0 : 3;
 #define W4_GO(ASYM, GSH)                                                               \
   simt_rows4_kernel<MX, MT, STEPS, ASYM, GSH, false><<<grid, SIMT_WAVES * 64, 0, s>>>( \
-      v.q, v.scales, v.zeros, x, c, v.N, M, nullptr)
+      v.q, v.scales, v.zeros, x, c, v.N, M, v.gs, v.G, nullptr)
 #define W4_GSH(ASYM)                                          \
   switch (gsh) {                                              \
+    case 0: W4_GO(ASYM, 0); break;                            \
+    case 3: W4_GO(ASYM, 3); break;                            \
     case 5: W4_GO(ASYM, 5); break;                            \
     case 6: W4_GO(ASYM, 6); break;                            \
     case 7: W4_GO(ASYM, 7); break;                            \
@@ -491,7 +495,7 @@ template <int MX, int MT>
 static bool try_rows4(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                       w4_half* w_out, hipError_t* err) {
   if (w_out || v.K % 2048 || v.N % (SIMT_WAVES * ROWS4_R)) return false;
-  if (!MX && (v.gs < 32 || v.gs > 256 || (v.gs & (v.gs - 1)))) return false;
+  if (!MX && (v.gs < 8 || v.gs % 8)) return false;
   if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)c & 7) || ((uintptr_t)v.scales & 3))
     return false;
   const int steps = v.K / 2048;

@@ -63,16 +63,22 @@ template <int MX, int MT, int STEPS, bool ASYM, int GSH, bool TL>
 __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_rows4_kernel(
     const uint32_t* __restrict__ q, const void* __restrict__ scales,
     const uint32_t* __restrict__ zeros, const w4_half* __restrict__ x, w4_half* __restrict__ c,
-    const int N, const int M, uint64_t* __restrict__ stamps) {
+    const int N, const int M, const int gs_any, const int G_any, uint64_t* __restrict__ stamps) {
   uint64_t ts[ROWS4_STAMPS];
   if (TL) ts[0] = rows4_now();
   constexpr int R = ROWS4_R, K = STEPS * 2048, WPR = K / 8, NQ = R * STEPS;
-  constexpr int G = MX ? K / 32 : (K >> GSH);             // groups (blocks) per row
-  constexpr int SB = MX ? R * G : R * G * 2;              // scale bytes of a wave's rows
-  constexpr int SD = SB / 4;                              // ... as dwords
-  constexpr int NSL = (SD + 63) / 64;                     // scale loads per lane
-  constexpr int WG = (G + 7) / 8;                         // zero-point words per row
-  constexpr int NZL = ASYM ? (R * WG + 63) / 64 : 0;      // zero-point loads per lane
+  // GSH 5..8: gs = 1 << GSH, one group per 32-k slice.  GSH 0 / 3: any gs % 8 == 0 with
+  // gs >= 32 / gs >= 8 (gs_any, G_any groups per row): a group per packed word; the
+  // arrays and load counts below are sized for the most groups a row can have.
+  constexpr bool ANY = !MX && GSH < 5;
+  constexpr int NG = ANY ? 4 : 1;                         // group lookups per slice
+  constexpr int GCAP = MX ? K / 32 : ANY ? (K >> (GSH == 0 ? 5 : 3)) : (K >> GSH);
+  const int G = ANY ? G_any : GCAP;                       // groups (blocks) per row
+  const int SD = MX ? R * G / 4 : R * G / 2;              // scale dwords of a wave's rows
+  constexpr int NSL = ((MX ? R * GCAP / 4 : R * GCAP / 2) + 63) / 64;  // scale loads per lane
+  constexpr int WGCAP = (GCAP + 7) / 8;
+  const int WG = (G + 7) / 8;                             // zero-point words per row
+  constexpr int NZL = ASYM ? (R * WGCAP + 63) / 64 : 0;   // zero-point loads per lane
   constexpr int XL = MT * STEPS;                          // activation loads per thread
   __shared__ u4 xs[MT * STEPS * 256];
   __shared__ uint32_t ss[SIMT_WAVES][NSL * 64];
@@ -89,7 +95,7 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_rows4_kernel(
     const int m = min(i / (STEPS * 256), M - 1 - m0), g8 = i % (STEPS * 256);
     W4_GLOAD16(xv[t], x + (size_t)(m0 + m) * K + g8 * 8);  // rows past M: a valid row, never stored
   }
-  const uint32_t* srun = (const uint32_t*)((const uint8_t*)scales + (size_t)n0 * (SB / R));
+  const uint32_t* srun = (const uint32_t*)((const uint8_t*)scales + (size_t)n0 * (MX ? G : 2 * G));
 #pragma unroll
   for (int t = 0; t < NSL; ++t) {
     const int i = min(t * 64 + lane, SD - 1);
@@ -131,15 +137,21 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_rows4_kernel(
   __syncthreads();
 
   // group parameters of this lane's slices, read back from LDS
-  uint32_t sc[NQ];
-  int zp[NQ];
+  uint32_t sc[NQ][NG];
+  int zp[NQ][NG];
 #pragma unroll
   for (int i = 0; i < NQ; ++i) {
     const int st = i / R, r = i % R;
-    const int g = MX ? st * 64 + lane : (st * 2048 + lane * 32) >> GSH;
-    if (MX) sc[i] = ((const uint8_t*)ss[wave])[r * G + g];
-    else sc[i] = ((const uint16_t*)ss[wave])[r * G + g];
-    zp[i] = ASYM ? (int)((zs[wave][r * WG + (g >> 3)] >> (4 * (g & 7))) & 0xFu) : 8;
+    int g4[4];
+    if (ANY) groups_of_slice(st * 2048 + lane * 32, gs_any, -1, G - 1, g4);
+    else g4[0] = MX ? st * 64 + lane : (st * 2048 + lane * 32) >> GSH;
+#pragma unroll
+    for (int j = 0; j < NG; ++j) {
+      const int g = g4[j];
+      if (MX) sc[i][j] = ((const uint8_t*)ss[wave])[r * G + g];
+      else sc[i][j] = ((const uint16_t*)ss[wave])[r * G + g];
+      zp[i][j] = ASYM ? (int)((zs[wave][r * WG + (g >> 3)] >> (4 * (g & 7))) & 0xFu) : 8;
+    }
   }
 
   float acc[R][MT];
@@ -165,13 +177,12 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_rows4_kernel(
     vm_wait<(NQ - 1 - i > 0 ? NQ - 1 - i : 0)>();
     landed(qw[i]);
     if (TL) ts[4 + i] = rows4_now();
-    const float mxs = mx_scale(sc[i]);
-    const W4Group grp = w4_group((uint16_t)sc[i], zp[i]);
+    const float mxs = mx_scale(sc[i][0]);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       h2 d[4];
       if (MX) dq_mx(qw[i][j], mxs, d);
-      else dq_w4(qw[i][j], grp, d);
+      else dq_w4(qw[i][j], w4_group((uint16_t)sc[i][ANY ? j : 0], zp[i][ANY ? j : 0]), d);
 #pragma unroll
       for (int m = 0; m < MT; ++m)
 #pragma unroll

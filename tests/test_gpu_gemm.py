@@ -63,6 +63,12 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         # multiple of 8: 86 chunks at K = 11008, 57 at K = 7296, 81 at K = 10368)
         (16, 256, 11008, 128), (64, 512, 14336, 64), (5, 128, 8192, 32), (33, 96, 7296, 128),
         (100, 64, 10368, 96),
+        # four rows per wave with a group lookup per packed word (group sizes that are no power of
+        # two, or below 32)
+        (1, 64, 4096, 48), (4, 32, 2048, 8), (2, 48, 4096, 96), (3, 16, 2048, 24),
+        # the small tiles of the large-M kernel with two sets of waves on an odd number of stages
+        # (9 and 15: the second set's last stage does not exist)
+        (130, 256, 1152, 128), (200, 384, 1920, 64),
         # an even number of chunks per wave that is not all there: the last waves' whole-line
         # pairs are clamped to the row's last pair (58 and 106 chunks for 8 x 8 and 8 x 14 slots)
         (16, 64, 7424, 128), (40, 48, 13568, 64),

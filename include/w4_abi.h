@@ -79,6 +79,12 @@ const char* w4_last_error(void);
 /* M at or above this goes to the matrix-core kernel in w4_gemm / w4_gemm_mx.
  * include/w4/dispatch.cuh:25 (re-measured for gfx950). */
 int w4_dispatch_mma_min_m(void);
+/* The same for one weight matrix: rows of packed words that are not 16-byte aligned
+ * (K % 32 != 0) leave the vector kernels their word-by-word form, and on large matrices
+ * (N * K >= 2^25) the matrix-core kernel is ahead from M = 3 (N = 11008, K = 4104: M = 3 / 4
+ * 31.5 / 32.7 us against 19.5); everywhere else this is w4_dispatch_mma_min_m().
+ * No counterpart in the reference, whose crossover is one constant (dispatch.cuh:25). */
+int w4_dispatch_mma_min_m_for(int N, int K);
 
 /* ---- packed-weight GEMM: c[M,N] = x[M,K] * W[N,K]^T, FP16 in/out ---------- */
 /* w: N*K halves, bit-identical to the host dequant_all.  dequant.cuh:62-82 */

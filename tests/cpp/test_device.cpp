@@ -114,7 +114,7 @@ void gemm_gates(Checks& t) {
       Dev<__half> cd((size_t)c.M * c.N), hook((size_t)c.N * c.K);
       gemm(dp, xd.p, cd.p, c.M, 0, hook.p);
       t.expect(same(hook.get(), w_ref), "dispatcher w_out bitwise");
-      t.expect(same(cd.get(), out[c.M < dispatch_mma_min_m() ? 0 : 1]), "dispatcher output == its callee");
+      t.expect(same(cd.get(), out[c.M < dispatch_mma_min_m(c.N, c.K) ? 0 : 1]), "dispatcher output == its callee");
     }
   for (size_t i = 0; i < sizeof kShapes / sizeof *kShapes; ++i) {
     const Shape c = kShapes[i];

@@ -37,6 +37,11 @@ def test_validation_runs_without_a_device():
     else:
         raise AssertionError("a malformed view was accepted")
     assert capi.load().w4_dispatch_mma_min_m() >= 1
+    lib = capi.load()
+    # one constant, lowered only for large matrices whose rows are not 16-byte aligned
+    assert lib.w4_dispatch_mma_min_m_for(4096, 4096) == lib.w4_dispatch_mma_min_m()
+    assert lib.w4_dispatch_mma_min_m_for(64, 4104) == lib.w4_dispatch_mma_min_m()
+    assert lib.w4_dispatch_mma_min_m_for(11008, 4104) == 3
 
 
 def test_quantize_contracts():

@@ -122,7 +122,7 @@ def test_w4_gemm_gates(i, sym):
     assert np.array_equal(cf, cf2) and np.array_equal(cm, cm2)
     # dispatcher: same bytes as the callee it selects, hook intact
     cd, wd = _run(c.gemm, dp.view, x_d, M, N, K)
-    want = cf if M < c.load().w4_dispatch_mma_min_m() else cm
+    want = cf if M < c.load().w4_dispatch_mma_min_m_for(N, K) else cm
     assert np.array_equal(cd, want) and np.array_equal(wd, w_ref)
     # two-pass baseline: dequant + plain FP16 GEMM
     c2 = halves(M * N, 0x7E00)

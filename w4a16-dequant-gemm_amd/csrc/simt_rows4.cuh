@@ -110,6 +110,13 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_rows4_kernel(
   for (int i = 0; i < NQ; ++i) {  // block-major: the four rows of a 2048-k block share its activations
     const int st = i / R, r = i % R;
     W4_GLOAD16_NT(qw[i], q + (size_t)(n0 + r) * WPR + st * 256 + lane * 4);
+    // The four waves place their runs in step: a barrier after every request.  Memory
+    // serves requests roughly in the order they were made; a wave that placed all its
+    // requests at once got all its runs late when it came late, with all of its
+    // arithmetic still ahead (the slowest wave ended 0.6 us after the median one).
+    // Round by round, every wave's run i lands at about the same time and the
+    // arithmetic keeps pace with the stream (C1: 3.63 - 3.72 -> 3.50 us in the same runs).
+    if (i + 1 < NQ) asm volatile("s_barrier" ::: "memory");
   }
 
   if (TL) ts[1] = rows4_now();

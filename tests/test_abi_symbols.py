@@ -42,6 +42,9 @@ def test_validation_runs_without_a_device():
     assert lib.w4_dispatch_mma_min_m_for(4096, 4096) == lib.w4_dispatch_mma_min_m()
     assert lib.w4_dispatch_mma_min_m_for(64, 4104) == lib.w4_dispatch_mma_min_m()
     assert lib.w4_dispatch_mma_min_m_for(11008, 4104) == 3
+    assert lib.w4_dispatch_mma_min_m_for(4096, 11008) == 3
+    assert lib.w4_dispatch_mma_min_m_for(4096, 4128) == 3
+    assert lib.w4_dispatch_mma_min_m_for(4096, 6144) == 2
 
 
 def test_quantize_contracts():

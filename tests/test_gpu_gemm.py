@@ -72,6 +72,10 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         # an even number of chunks per wave that is not all there: the last waves' whole-line
         # pairs are clamped to the row's last pair (58 and 106 chunks for 8 x 8 and 8 x 14 slots)
         (16, 64, 7424, 128), (40, 48, 13568, 64),
+        # ... with the requests pipelined chunk by chunk (M <= 32): odd and even chunk counts, ragged last waves
+        (17, 64, 10368, 96), (32, 32, 14336, 32), (9, 48, 7296, 64), (12, 32, 11264, 128), (3, 16, 13440, 64),
+        (3, 32, 5120, 128), (8, 16, 6144, 64), (12, 16, 7168, 32), (16, 32, 9216, 128), (24, 16, 10240, 64),
+        (5, 16, 12288, 128), (13, 16, 15360, 32), (4, 32, 16384, 128), (3, 16, 4224, 32), (20, 16, 4352, 64),
         # four rows per wave (N % 16 == 0, K = 2048 / 4096 / 8192, gs 32 ... 256): one to four
         # activation rows, one to eight scale loads per lane
         (3, 32, 4096, 32), (4, 48, 2048, 64), (2, 32, 8192, 32), (1, 16, 4096, 256), (4, 16, 4096, 128),
@@ -151,7 +155,7 @@ def test_mx_gemm_gates(i):
     assert np.array_equal(wm, w_ref), "mx mma w_out bitwise"
     assert orc.rel_l2(cm.view(np.float16), ref) <= TOL
     cd, wd = _run(c.gemm_mx, dp.view, x_d, M, N, K)
-    want = cf if M < c.load().w4_dispatch_mma_min_m() else cm
+    want = cf if M < c.load().w4_dispatch_mma_min_m_for(N, K) else cm
     assert np.array_equal(cd, want) and np.array_equal(wd, w_ref)
 
 

@@ -170,6 +170,8 @@ const char* w4_last_error(void) { return g_msg; }
 int w4_dispatch_mma_min_m(void) { return DISPATCH_MMA_MIN_M; }
 int w4_dispatch_mma_min_m_for(int N, int K) {
   if (K % 32 != 0 && K % 8 == 0 && (long long)N * K >= (1LL << 25)) return 3;
+  if (K > 4096 && K <= 6144 && K % 128 == 0) return 2;  // 5.6 - 5.9 us against 6.3 at N = 4096
+  if (K > 4096 && K % 32 == 0) return 3;
   return DISPATCH_MMA_MIN_M;
 }
 
@@ -241,8 +243,9 @@ int w4_gemm_mma_mx(const w4_packed_mx_view* p, const w4_half* x, w4_half* c, int
 
 int w4_gemm_mx(const w4_packed_mx_view* p, const w4_half* x, w4_half* c, int M,
                w4_stream stream, w4_half* w_out) {
-  return M < DISPATCH_MMA_MIN_M ? w4_gemm_fused_mx(p, x, c, M, stream, w_out)
-                                : w4_gemm_mma_mx(p, x, c, M, stream, w_out);
+  const int min_m = p ? w4_dispatch_mma_min_m_for(p->N, p->K) : DISPATCH_MMA_MIN_M;
+  return M < min_m ? w4_gemm_fused_mx(p, x, c, M, stream, w_out)
+                   : w4_gemm_mma_mx(p, x, c, M, stream, w_out);
 }
 
 // ---- attention -------------------------------------------------------------------

@@ -898,12 +898,16 @@ static hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M
   const bool wvec = (v.K % 32 == 0) && (((uintptr_t)v.q) & 15) == 0;
   const bool resident = wvec && decode_resident_applies(v, x, c, M) &&
                         (w_out == nullptr || ((uintptr_t)w_out & 15) == 0);
+  // long K, M <= 32: the same sums with the requests pipelined chunk by chunk
+  const bool longk = wvec && decode_longk_applies(v, x, c, M) &&
+                     (w_out == nullptr || ((uintptr_t)w_out & 15) == 0);
+  if (longk && w_out == nullptr) return launch_decode_longk(v, x, c, M, s);
   if (resident && w_out == nullptr) return launch_decode_resident(v, x, c, M, s);
   // ... and of its sibling for odd group sizes and ragged K (M <= 64, W4 only)
-  const bool general = !resident && !MX && decode_general_applies(v, x, c, M) &&
+  const bool general = !resident && !longk && !MX && decode_general_applies(v, x, c, M) &&
                        (w_out == nullptr || ((uintptr_t)w_out & 15) == 0);
   if (general && w_out == nullptr) return launch_decode_general(v, x, c, M, s);
-  if (!resident && !general) {
+  if (!resident && !general && !longk) {
     if (try_tile_dma(v, x, c, M, s, w_out, &terr)) return terr;
     if (try_tile<MX>(v, x, c, M, s, w_out, &terr)) return terr;
   }
@@ -914,7 +918,7 @@ static hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M
   if (aligned) {
     // Measured on N = 4096 .. 14336, K = 4096 .. 11008: the K-split kernel wins for
     // M <= 16 unless N is large enough to give the streaming kernel a full grid.
-    const bool ksplit = M <= 8 || (M <= 16 && v.N < 8192) || resident || general;
+    const bool ksplit = M <= 8 || (M <= 16 && v.N < 8192) || resident || general || longk;
     if (ksplit) {
       if (MX) return launch_decode<2>(v, x, c, M, s, w_out, wvec);
       return v.symmetric ? launch_decode<0>(v, x, c, M, s, w_out, wvec)

@@ -29,6 +29,7 @@
 namespace w4k {
 
 constexpr int SIMT_R = 2;               // weight rows per wave
+constexpr int KS_R = 4;                 // weight rows per workgroup of the K-split kernel
 constexpr int SIMT_LDS_HALVES = 16384;  // activations resident in LDS at once (32 KiB)
 
 __device__ __forceinline__ u4 load_x8_guarded(const w4_half* __restrict__ x, int M, int K,
@@ -509,7 +510,10 @@ static bool try_rows4(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
 }
 
 // One or two activation rows, long or odd K (K % 32 == 0, K <= 16384; e.g. 11008,
-// 14336, 6144): the W waves of a workgroup share R = 2 weight rows and split K into
+// 14336, 6144): the W waves of a workgroup share R = 4 weight rows (a wave's slice of
+// the activations serves all of them: two rows per workgroup read the activations
+// from L2 twice as often and took 8.4 instead of 7.0 us at N = 4096, K = 11008; eight
+// rows leave too few workgroups) and split K into
 // runs of whole 32-k slices (W is chosen so that the lanes are nearly all busy:
 // 6 waves for K = 11008, 7 for 14336); each wave is the unrolled kernel on its run
 // (activations straight from L2, everything requested before it is consumed,
@@ -517,8 +521,14 @@ static bool try_rows4(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
 // and the partial sums meet in LDS in wave order.
 template <int MX, int MT, int R, int W, int STEPS, bool ASYM, bool GS32, bool HOOK>
 __global__ __launch_bounds__(W * 64) void simt_ksplit_kernel(
-    const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
-    const int gs_shift, w4_half* __restrict__ w_out) {
+    const uint32_t* __restrict__ q_, const void* __restrict__ scales_,
+    const w4_half* __restrict__ x, w4_half* __restrict__ c, const int K_, const int N_,
+    const int M, const int gs_shift, const int G_, const int gs_,
+    const uint32_t* __restrict__ zeros_, w4_half* __restrict__ w_out) {
+  // the leading arguments arrive in registers with the wave: the code stream is addressed
+  // without a round trip to the argument segment
+  const struct { const uint32_t* q; const void* scales; const uint32_t* zeros; int K, N, G, B, gs; }
+      p{q_, scales_, zeros_, K_, N_, G_, G_, gs_};
   __shared__ float red[W][R][MT];
   constexpr int NS = (MX || GS32) ? 1 : 4;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -569,8 +579,9 @@ __global__ __launch_bounds__(W * 64) void simt_ksplit_kernel(
 #pragma unroll
   for (int s = 0; s < STEPS; ++s)
 #pragma unroll
-    for (int r = 0; r < R; ++r)
+    for (int r = 0; r < R; ++r) {
       qw[s][r] = __builtin_nontemporal_load((const u4*)(p.q + (size_t)(n0 + r) * wpr + (k0[s] >> 3)));
+    }
 
   float acc[R][MT];
 #pragma unroll
@@ -646,15 +657,17 @@ static hipError_t launch_ksplit(const WView& v, const w4_half* x, w4_half* c, in
   const bool gs32 = MX || v.gs % 32 == 0;
   const bool pow2 = !MX && (v.gs & (v.gs - 1)) == 0;
   const int sh = pow2 ? __builtin_ctz((unsigned)v.gs) : -1;
-  const dim3 grid((unsigned)(v.N / SIMT_R), (unsigned)((M + MT - 1) / MT));
+  const dim3 grid((unsigned)(v.N / KS_R), (unsigned)((M + MT - 1) / MT));
 #define W4_GO(ASYM, GS32)                                                                 \
   do {                                                                                    \
     if (w_out)                                                                            \
-      simt_ksplit_kernel<MX, MT, SIMT_R, W, STEPS, ASYM, GS32, true>                      \
-          <<<grid, W * 64, 0, s>>>(v, x, c, M, sh, w_out);                                \
+      simt_ksplit_kernel<MX, MT, KS_R, W, STEPS, ASYM, GS32, true>                      \
+          <<<grid, W * 64, 0, s>>>(v.q, v.scales, x, c, v.K, v.N, M, sh, MX ? v.B : v.G,  \
+                                   v.gs, v.zeros, w_out);                                 \
     else                                                                                  \
-      simt_ksplit_kernel<MX, MT, SIMT_R, W, STEPS, ASYM, GS32, false>                     \
-          <<<grid, W * 64, 0, s>>>(v, x, c, M, sh, w_out);                                \
+      simt_ksplit_kernel<MX, MT, KS_R, W, STEPS, ASYM, GS32, false>                     \
+          <<<grid, W * 64, 0, s>>>(v.q, v.scales, x, c, v.K, v.N, M, sh, MX ? v.B : v.G,  \
+                                   v.gs, v.zeros, w_out);                                 \
   } while (0)
   if (!MX && !v.symmetric) {
     if (gs32) W4_GO(true, true); else W4_GO(true, false);
@@ -669,7 +682,7 @@ template <int MX, int MT>
 static bool try_ksplit(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                        w4_half* w_out, hipError_t* err) {
   // four rows fetched per wave cost more than the staged kernel's barrier (20.7 vs 19 us at K = 11008)
-  if (MT > 2 || v.K % 32 || v.K > 16384 || v.K < 2048 || v.N % SIMT_R) return false;
+  if (MT > 2 || v.K % 32 || v.K > 16384 || v.K < 2048 || v.N % KS_R) return false;
   // shapes of the unrolled kernel stay with it (and, hooked, with the kernel that sums like it)
   const int blocks = v.K / 2048;
   if (v.K % 2048 == 0 && (blocks == 1 || blocks == 2 || blocks == 4) && blocks * MT <= 8 &&

@@ -51,6 +51,13 @@ bool decode_resident_applies(const WView& v, const w4_half* x, const w4_half* c,
 hipError_t launch_decode_resident(const WView& v, const w4_half* x, w4_half* c, int M,
                                   hipStream_t s);
 
+// gemm_decode_longk.hip: M <= 32 at long K (8, 11 or 14 chunks of 128 k per wave), one
+// 16-row tile per workgroup with activations and codes requested chunk by chunk while
+// earlier chunks multiply; same order of additions as the two kernels above.
+bool decode_longk_applies(const WView& v, const w4_half* x, const w4_half* c, int M);
+hipError_t launch_decode_longk(const WView& v, const w4_half* x, w4_half* c, int M,
+                               hipStream_t s);
+
 // gemm_decode_general.hip: M <= 64 for any group size (multiple of 8) and any K % 8 == 0
 // with 1024 < K <= 5120, group parameters through LDS; same order of additions as the
 // K-split decode kernels of gemm_mfma.hip.

@@ -577,6 +577,23 @@ def extras_gemm(b, full):
         rows.append({"weights": "w4_sym_gs128", "M": M2, "fused_us": ms * 1e3, "two_pass_us": ms2 * 1e3,
                      "fused_TFLOPs": 2.0 * M2 * N * K / ms * 1e-9})
     out["c4_prefill_other_M"] = rows
+    if full:
+        # the down-projection side of the MLP shapes (long K) through the dispatcher: timing
+        # only, on random codes (the parity tests hold these shapes against the oracle)
+        rows = []
+        for (N2, K2) in ((4096, 11008), (4096, 14336)):
+            vs = [v[0] for v in rand_w4_views(b, N2, K2, 128, True, 10)]
+            for M2 in (1, 2, 4, 8, 16, 32, 64):
+                x2 = torch.randn(M2 * K2, device="cuda").to(torch.float16)
+                c2 = torch.empty(M2 * N2, dtype=torch.float16, device="cuda")
+                us, raw = b.gemm_us("w4_gemm", vs, x2, c2, M2)
+                nb = w4_bytes(N2, K2, 128, True, M2)
+                rows.append({"N": N2, "K": K2, "gs": 128, "M": M2, "us": us, "reps_us": raw, "bytes": nb,
+                             "GBs": nb / us * 1e-3,
+                             "dispatcher": "simt" if M2 < capi.load().w4_dispatch_mma_min_m_for(N2, K2) else "mfma"})
+            del vs
+            torch.cuda.empty_cache()
+        out["long_k_w4_sym_gs128"] = rows
     return out
 
 
@@ -918,6 +935,15 @@ def probe(b, which, args):
             x = torch.randn(M * K, device="cuda").to(torch.float16)
             c = torch.empty(M * N, dtype=torch.float16, device="cuda")
             out["%s_M%d_us" % (fn, M)] = b.gemm_us(fn, views, x, c, M)[0]
+    elif which == "longk":  # down-projection shapes: K-split vector kernel at M=1, pipelined matrix-core kernel at M=4 and 16
+        for (N, K) in ((4096, 11008), (4096, 14336)):
+            views = [v[0] for v in rand_w4_views(b, N, K, 128, True, 12)]
+            for M in (1, 4, 16):
+                x = torch.randn(M * K, device="cuda").to(torch.float16)
+                c = torch.empty(M * N, dtype=torch.float16, device="cuda")
+                out["w4_gemm_K%d_M%d_us" % (K, M)] = b.gemm_us("w4_gemm", views, x, c, M)[0]
+            del views
+            torch.cuda.empty_cache()
     elif which == "attention":  # C5 flash decode over FP16 / W4 / paged W4 / FP8 caches
         b.steps = 200
         out.update(extras_attention(b, False))
@@ -952,7 +978,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--reps", type=int, default=9, help="repetitions of the K timed steps (median reported)")
     ap.add_argument("--extras", choices=["none", "quick", "full"], default="quick")
-    ap.add_argument("--probe", choices=["floor", "c1", "decode", "prefill", "quantize", "w4a4", "attention"],
+    ap.add_argument("--probe", choices=["floor", "c1", "decode", "longk", "prefill", "quantize", "w4a4", "attention"],
                     default=None, help="run only a short fixed workload (for counter collection) and exit")
     args = ap.parse_args()
     if args.gpus != 1:

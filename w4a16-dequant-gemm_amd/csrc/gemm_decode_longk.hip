@@ -44,13 +44,12 @@ __device__ __forceinline__ void lk_for(F&& f, std::integer_sequence<int, I...>) 
 
 typedef __attribute__((address_space(3))) void* lds_ptr;
 constexpr int LK_WAVES = 8, LK_THREADS = 64 * LK_WAVES;
-// Chunk buffers in a wave's ring (a buffer is NQ KB per row tile, the ring at most
-// 16 KB; deeper rings measured no better, and small ones let a compute unit hold two
-// workgroups when N gives it more than one tile), and units of codes requested ahead.
-#ifndef LK_MAXBUF
-#define LK_MAXBUF 4
-#endif
-constexpr int lk_nbuf(int MT, int NQ) { return 16 / (MT * NQ) < LK_MAXBUF ? 16 / (MT * NQ) : LK_MAXBUF; }
+// Chunk buffers in a wave's ring (a buffer is NQ KB per row tile): as many as 8 KB hold,
+// at least 2 and at most 4.  Deeper rings measured no better, and a workgroup that
+// stays within 64 KB lets a compute unit hold two of them when N gives it more than one
+// tile (N = 8192, K = 8192, M = 16: 18.6 -> 17.2 us).  Units of codes requested ahead:
+// half as many chunks' worth, at least 2.
+constexpr int lk_nbuf(int MT, int NQ) { return 8 / (MT * NQ) < 2 ? 2 : 8 / (MT * NQ) < 4 ? 8 / (MT * NQ) : 4; }
 constexpr int lk_lau(int MT, int NQ) { return lk_nbuf(MT, NQ) / 2 > 2 ? lk_nbuf(MT, NQ) / 2 : 2; }
 constexpr int lk_waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
 extern __shared__ __attribute__((aligned(16))) uint8_t lk_lds[];

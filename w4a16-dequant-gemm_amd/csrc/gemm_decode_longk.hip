@@ -328,11 +328,23 @@ __global__ __launch_bounds__(LK_THREADS) void mfma_decode_longk_kernel(
   }
 }
 
-// Chunks per wave if K is this kernel's (whole chunks, 5 .. 16 per wave: 4224 .. 16384), else 0.
+// Chunks per wave if K is this kernel's (whole chunks, 2 .. 16 per wave: 1152 .. 16384), else 0.
 int longk_chunks(int K) {
   if (K % 128) return 0;
   const int per_wave = (K / 128 + LK_WAVES - 1) / LK_WAVES;
-  return (per_wave >= 5 && per_wave <= 16) ? per_wave : 0;
+  return (per_wave >= 2 && per_wave <= 16) ? per_wave : 0;
+}
+
+// Compute units of the current device (per-device cache); 0 on error.
+int lk_cus() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < 64 && cached[dev]) return cached[dev];
+  int n = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < 64) cached[dev] = n;
+  return n;
 }
 
 template <int FMT, int CH, int MT, int NQ>
@@ -367,6 +379,9 @@ hipError_t longk_m(const WView& v, const w4_half* x, w4_half* c, int M, hipStrea
 template <int FMT>
 hipError_t longk_fmt(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s) {
   switch (longk_chunks(v.K)) {
+    case 2: return longk_m<FMT, 2>(v, x, c, M, s);
+    case 3: return longk_m<FMT, 3>(v, x, c, M, s);
+    case 4: return longk_m<FMT, 4>(v, x, c, M, s);
     case 5: return longk_m<FMT, 5>(v, x, c, M, s);
     case 6: return longk_m<FMT, 6>(v, x, c, M, s);
     case 7: return longk_m<FMT, 7>(v, x, c, M, s);
@@ -385,12 +400,23 @@ hipError_t longk_fmt(const WView& v, const w4_half* x, w4_half* c, int M, hipStr
 
 }  // namespace
 
-// Long K (5 to 16 whole chunks of 128 k per wave), whole 16-row tiles, a lane's 32-k
-// slice inside one group, M <= 32, 16-byte aligned codes and activations.
+// 5 to 16 whole chunks of 128 k per wave (2 to 4 on thin grids, see below), whole 16-row
+// tiles, a lane's 32-k slice inside one group, M <= 32, 16-byte aligned codes and
+// activations.
 bool decode_longk_applies(const WView& v, const w4_half* x, const w4_half* c, int M) {
   if (M < 1 || M > 32 || v.N % 16 || longk_chunks(v.K) == 0) return false;
   if (!v.mx && v.gs % 32) return false;
   if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)c & 7)) return false;
+  if (longk_chunks(v.K) < 5) {
+    // Shorter K: only where the kernels that share x between the tiles of a workgroup
+    // would have one tile per workgroup too (N / 16 <= compute units).  At K = 2048 and
+    // 4096, the resident kernel's own, this one is ahead while few quads of x are
+    // fetched and most compute units have a tile (N = 4096, K = 4096, M = 5 / 8: 5.5 ->
+    // 4.8 / 5.0 us; M = 16: 5.6 -> 5.9; N = 2048, M = 8: 5.35 -> 5.66).
+    const int tiles = v.N / 16, cus = lk_cus();
+    if (cus < 1 || tiles > cus) return false;
+    if ((v.K == 2048 || v.K == 4096) && (M > 8 || 2 * tiles <= cus)) return false;
+  }
   return true;
 }
 

@@ -16,8 +16,10 @@ from devutil import DevKV, DevPacked, bits, halves, ptr, to_dev
 
 pytestmark = pytest.mark.gpu
 
-# (M, N, K, gs, symmetric): decode shape, decode batch, thin grid of small tiles
-GEMMS = [(1, 256, 4096, 128, True), (8, 4128, 2048, 64, False), (100, 256, 2048, 128, True)]
+# (M, N, K, gs, symmetric): decode shape, decode batch, thin grid of small tiles, long K (two row tiles:
+# the pipelined kernel asks for its 128 KB of LDS on first use, inside the capture)
+GEMMS = [(1, 256, 4096, 128, True), (8, 4128, 2048, 64, False), (100, 256, 2048, 128, True),
+         (24, 64, 11008, 128, False)]
 
 
 @pytest.mark.parametrize("i", range(len(GEMMS)))

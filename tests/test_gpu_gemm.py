@@ -76,6 +76,8 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         (17, 64, 10368, 96), (32, 32, 14336, 32), (9, 48, 7296, 64), (12, 32, 11264, 128), (3, 16, 13440, 64),
         (3, 32, 5120, 128), (8, 16, 6144, 64), (12, 16, 7168, 32), (16, 32, 9216, 128), (24, 16, 10240, 64),
         (5, 16, 12288, 128), (13, 16, 15360, 32), (4, 32, 16384, 128), (3, 16, 4224, 32), (20, 16, 4352, 64),
+        # ... four row tiles (M <= 64): units of one row tile in the ring
+        (33, 32, 11008, 128), (64, 16, 14336, 32), (50, 32, 8192, 64), (47, 16, 5120, 128), (64, 16, 16384, 128),
         # ... and K <= 4096 on grids of at most one tile per compute unit
         (6, 2064, 4096, 128), (8, 4096, 2048, 32), (7, 32, 3072, 64), (20, 48, 2560, 32), (32, 16, 1536, 128),
         (3, 16, 1152, 32),

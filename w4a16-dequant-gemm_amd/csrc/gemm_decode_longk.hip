@@ -1,4 +1,4 @@
-// Decode-batch W4A16 / MXFP4 GEMM (M <= 32) for long K (more than four 128-k chunks
+// Decode-batch W4A16 / MXFP4 GEMM (M <= 64) for long K (more than four 128-k chunks
 // per wave: K = 4224 .. 16384 in whole chunks, the down-projection side of the usual
 // MLP shapes).  mma.cuh:63-230 is the reference's kernel for this
 // path.
@@ -14,9 +14,9 @@
 // it and then multiplies: the stream (5 .. 6 us) and the expansion of the codes
 // (3 .. 4 us of vector-ALU work per SIMD) come one after the other.  Here a wave runs
 // a software pipeline over its chunks:
-//   * its LDS region is a ring of NBUF = 4 / MT chunk buffers (4 KB per 16 activation
-//     rows); chunk i + NBUF of x is requested (global_load_lds_dwordx4, whole lines,
-//     XOR-swizzled) as soon as chunk i has been read back into registers;
+//   * its LDS region is a ring of 2 to 4 units of x (a unit: one chunk of one tile of 16
+//     activation rows); unit u + NBUF is requested (global_load_lds_dwordx4, whole
+//     lines, XOR-swizzled) as soon as unit u has been read back into registers;
 //   * codes are requested a unit (two chunks) at a time, two units ahead; with an even
 //     number of chunks per wave and rows of whole 256-byte pairs of lines the two
 //     loads of a unit take whole lines (rows 0..7, rows 8..15) and pair_fix()
@@ -44,13 +44,19 @@ __device__ __forceinline__ void lk_for(F&& f, std::integer_sequence<int, I...>) 
 
 typedef __attribute__((address_space(3))) void* lds_ptr;
 constexpr int LK_WAVES = 8, LK_THREADS = 64 * LK_WAVES;
-// Chunk buffers in a wave's ring (a buffer is NQ KB per row tile): as many as 8 KB hold,
-// at least 2 and at most 4.  Deeper rings measured no better, and a workgroup that
-// stays within 64 KB lets a compute unit hold two of them when N gives it more than one
-// tile (N = 8192, K = 8192, M = 16: 18.6 -> 17.2 us).  Units of codes requested ahead:
-// half as many chunks' worth, at least 2.
-constexpr int lk_nbuf(int MT, int NQ) { return 8 / (MT * NQ) < 2 ? 2 : 8 / (MT * NQ) < 4 ? 8 / (MT * NQ) : 4; }
-constexpr int lk_lau(int MT, int NQ) { return lk_nbuf(MT, NQ) / 2 > 2 ? lk_nbuf(MT, NQ) / 2 : 2; }
+constexpr int LK_MAX_M = 64;
+// A unit of activations is one 128-k chunk of one tile of 16 rows (NQ KB: NQ quads of
+// rows).  Units in a wave's ring: with one row tile as many as 8 KB hold, at least 2 and
+// at most 4 (deeper rings measured no better, and a workgroup that stays within 64 KB
+// lets a compute unit hold two of them when N gives it more than one tile: N = 8192,
+// K = 8192, M = 16: 18.6 -> 17.2 us); with several row tiles four units of 4 KB, so that
+// the stream from L2 goes on while a unit is read back into registers (with whole
+// chunks of 2 or 4 units as the granule the two took turns).  Units of codes (two
+// chunks) requested ahead: half as many as chunks in the ring, at least 2.
+constexpr int lk_nbuf(int MT, int NQ) {
+  return MT > 1 ? 4 : 8 / NQ < 2 ? 2 : 8 / NQ < 4 ? 8 / NQ : 4;
+}
+constexpr int lk_lau(int MT, int NQ) { return lk_nbuf(MT, NQ) / MT / 2 > 2 ? lk_nbuf(MT, NQ) / MT / 2 : 2; }
 constexpr int lk_waitcnt_vm(int n) { return (n & 0xF) | ((n >> 4) << 14) | 0x0F70; }
 extern __shared__ __attribute__((aligned(16))) uint8_t lk_lds[];
 
@@ -65,47 +71,43 @@ __device__ __forceinline__ h8 lk_expand_word(uint32_t w, h2 cneg, h2 s2, uint32_
   return __builtin_bit_cast(h8, out);
 }
 
-// The issue order of a wave, replayed at compile time.  allowed[i]: how many vector
-// memory requests may still be outstanding when chunk i is multiplied (those issued
-// after the last one chunk i needs).  NSC: parameter loads per chunk.
-template <int CH>
+// The issue order of a wave, replayed at compile time.  allowed[u]: how many vector
+// memory requests may still be outstanding when unit u of the activations (chunk
+// u / MT, row tile u % MT) is read back -- those issued after the last one it needs;
+// the first unit of a chunk also needs the chunk's codes.  NSC: parameter loads per chunk.
+template <int UN>
 struct LkSched {
-  int allowed[CH];
+  int allowed[UN];
   int peak;
 };
 template <int CH, int MT, int NQ, int NSC>
-constexpr LkSched<CH> lk_schedule() {
-  constexpr int NBUF = lk_nbuf(MT, NQ), LK_LAU = lk_lau(MT, NQ), NX = NQ * MT;
-  LkSched<CH> s{};
-  int xlast[CH] = {}, clast[CH] = {};
+constexpr LkSched<CH * MT> lk_schedule() {
+  constexpr int NBUF = lk_nbuf(MT, NQ), LAU = lk_lau(MT, NQ), UN = CH * MT;
+  LkSched<UN> s{};
+  int xlast[UN] = {}, clast[CH] = {};
   int seq = NSC * CH;  // the parameter loads go first
-  for (int u = 0; u < LK_LAU; ++u) {
-    for (int i = 2 * u; i < 2 * u + 2; ++i)
-      if (i < NBUF && i < CH) seq += NX, xlast[i] = seq - 1;
-    if (2 * u < CH) {
-      seq += (2 * u + 1 < CH) ? 2 : 1;
-      clast[2 * u] = seq - 1;
-      if (2 * u + 1 < CH) clast[2 * u + 1] = seq - 1;
-    }
+  int cu = 0;          // units of codes issued
+  auto codes = [&](int u) {
+    if (2 * u >= CH) return;
+    seq += (2 * u + 1 < CH) ? 2 : 1;
+    clast[2 * u] = seq - 1;
+    if (2 * u + 1 < CH) clast[2 * u + 1] = seq - 1;
+  };
+  for (int u = 0; u < NBUF && u < UN; ++u) {
+    seq += NQ, xlast[u] = seq - 1;
+    if ((u + 1) % (2 * MT) == 0 && cu < LAU) codes(cu++);
   }
-  for (int i = 2 * LK_LAU; i < NBUF && i < CH; ++i) seq += NX, xlast[i] = seq - 1;
+  while (cu < LAU) codes(cu++);
   s.peak = seq;
   int done = -1;  // the youngest request known to have landed
-  for (int i = 0; i < CH; ++i) {
-    int need = xlast[i];
-    if (clast[i] > need) need = clast[i];
+  for (int u = 0; u < UN; ++u) {
+    int need = xlast[u];
+    if (clast[u / MT] > need) need = clast[u / MT];
     if (need > done) done = need;
-    s.allowed[i] = seq - 1 - done;
+    s.allowed[u] = seq - 1 - done;
     if (seq - 1 - done > s.peak) s.peak = seq - 1 - done;
-    if (i + NBUF < CH) seq += NX, xlast[i + NBUF] = seq - 1;
-    if (i % 2 == 0) {
-      const int u = i / 2 + LK_LAU;
-      if (2 * u < CH) {
-        seq += (2 * u + 1 < CH) ? 2 : 1;
-        clast[2 * u] = seq - 1;
-        if (2 * u + 1 < CH) clast[2 * u + 1] = seq - 1;
-      }
-    }
+    if (u + NBUF < UN) seq += NQ, xlast[u + NBUF] = seq - 1;
+    if (u % MT == MT - 1 && (u / MT) % 2 == 0) codes(u / MT / 2 + LAU);
   }
   return s;
 }
@@ -125,10 +127,11 @@ __global__ __launch_bounds__(LK_THREADS) void mfma_decode_longk_kernel(
     const uint32_t* __restrict__ zeros, const w4_half* __restrict__ x, w4_half* __restrict__ c,
     const int N, const int K, const int M, const int gs_shift, const int G, const int gs) {
   constexpr bool MX = FMT == 2;
-  constexpr int NBUF = lk_nbuf(MT, NQ), LK_LAU = lk_lau(MT, NQ), NSC = FMT == 1 ? 2 : 1;
-  constexpr LkSched<CH> SCH = lk_schedule<CH, MT, NQ, NSC>();
+  constexpr int NBUF = lk_nbuf(MT, NQ), LK_LAU = lk_lau(MT, NQ), NSC = FMT == 1 ? 2 : 1, UN = CH * MT;
+  constexpr LkSched<UN> SCH = lk_schedule<CH, MT, NQ, NSC>();
   static_assert(SCH.peak < 64, "vmcnt is a 6-bit counter");
-  constexpr int XBYTES = NBUF * MT * NQ * 1024;  // the wave's ring: NBUF buffers of MT x NQ KB
+  static_assert(MT == 1 || NQ == 4, "several row tiles: whole tiles of 16 rows");
+  constexpr int XBYTES = NBUF * NQ * 1024;  // the wave's ring: NBUF units of NQ KB
   const int WPR = K >> 3, nchunks = K >> 7;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -141,24 +144,23 @@ __global__ __launch_bounds__(LK_THREADS) void mfma_decode_longk_kernel(
   // ---- requests ----
   const uint32_t region = (uint32_t)(uintptr_t)(lds_ptr)lk_lds + (uint32_t)wave * XBYTES;
   const char* xb = (const char*)x;
-  // chunk i of this wave's slice of x -> buffer i % NBUF: block (mt, rq) = rows
-  // 16 mt + 4 rq .. + 3; lane l fetches row l / 16 of the four, 16-byte piece
-  // (l % 16) ^ (row % 16) of the chunk's 256 bytes.  Rows past M repeat row M - 1.
-  auto request_x = [&](int i) {
-    const int cidx = chunk_of(i);
+  // unit u = (chunk u / MT, row tile u % MT) of this wave's slice of x -> buffer u % NBUF:
+  // block rq = rows 4 rq .. + 3 of the tile; lane l fetches row l / 16 of the four,
+  // 16-byte piece (l % 16) ^ (row % 16) of the chunk's 256 bytes.  Rows past M repeat
+  // row M - 1.
+  auto request_x = [&](int u) {
+    const int cidx = chunk_of(u / MT), mt = u % MT;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int rq = 0; rq < NQ; ++rq) {
-        const int r16 = 4 * rq + (lane >> 4), row = m0 + 16 * mt + r16;
-        const uint32_t off = (uint32_t)min(row, M - 1) * (uint32_t)(K * 2) + (uint32_t)cidx * 256u +
-                             (uint32_t)(((lane & 15) ^ r16) * 16);
-        const uint32_t dst = region + (uint32_t)(((i % NBUF) * MT + mt) * NQ + rq) * 1024u;
-        asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
-                     :
-                     : "v"(off), "s"(xb), "s"(dst)
-                     : "memory", "m0");
-      }
+    for (int rq = 0; rq < NQ; ++rq) {
+      const int r16 = 4 * rq + (lane >> 4), row = m0 + 16 * mt + r16;
+      const uint32_t off = (uint32_t)min(row, M - 1) * (uint32_t)(K * 2) + (uint32_t)cidx * 256u +
+                           (uint32_t)(((lane & 15) ^ r16) * 16);
+      const uint32_t dst = region + (uint32_t)((u % NBUF) * NQ + rq) * 1024u;
+      asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1"
+                   :
+                   : "v"(off), "s"(xb), "s"(dst)
+                   : "memory", "m0");
+    }
   };
   constexpr bool PAIRC = CH % 2 == 0;
   const bool paired = PAIRC && (K & 255) == 0;
@@ -220,18 +222,23 @@ __global__ __launch_bounds__(LK_THREADS) void mfma_decode_longk_kernel(
   }
   __builtin_amdgcn_sched_barrier(0);
   // (the scheduling barriers pin the order that lk_schedule() replays)
+  {
+    int cu = 0;
 #pragma unroll
-  for (int u = 0; u < LK_LAU; ++u) {
+    for (int u = 0; u < NBUF && u < UN; ++u) {
+      request_x(u);
+      __builtin_amdgcn_sched_barrier(0);
+      if ((u + 1) % (2 * MT) == 0 && cu < LK_LAU) {
+        if (2 * cu < CH) request_codes(cu);
+        ++cu;
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
 #pragma unroll
-    for (int i = 2 * u; i < 2 * u + 2; ++i)
-      if (i < NBUF && i < CH) request_x(i);
-    __builtin_amdgcn_sched_barrier(0);
-    if (2 * u < CH) request_codes(u);
+    for (int k = 0; k < LK_LAU; ++k)
+      if (k >= cu && 2 * k < CH) request_codes(k);
     __builtin_amdgcn_sched_barrier(0);
   }
-#pragma unroll
-  for (int i = 2 * LK_LAU; i < NBUF && i < CH; ++i) request_x(i);
-  __builtin_amdgcn_sched_barrier(0);
   uint32_t mask = 0x00F0000Fu, magic = 0x54006400u;
   asm volatile("" : "+s"(mask));   // opaque: as literals they cost two instructions
   asm volatile("" : "+v"(magic));  // instead of one and-or
@@ -240,38 +247,36 @@ __global__ __launch_bounds__(LK_THREADS) void mfma_decode_longk_kernel(
   for (int mt = 0; mt < MT; ++mt) acc[mt] = f4{0.f, 0.f, 0.f, 0.f};
 
   const uint8_t* mine = lk_lds + wave * XBYTES;
-  lk_for([&](auto ic) {
-    constexpr int i = decltype(ic)::value;
-    __builtin_amdgcn_s_waitcnt(lk_waitcnt_vm(SCH.allowed[i]));
-    // the registers of this chunk's codes are defined from here on
-    asm volatile("" : "+v"(qw[i]), "+v"(sc[i]));
-    if (FMT == 1) asm volatile("" : "+v"(zw[i]));
-    if (i % 2 == 0 && i + 1 < CH) asm volatile("" : "+v"(qw[i + 1]));
+  u4 xv[MT][4];  // B operands: MFMA j contracts k = 128 chunk + 32 b + 8 j .. + 7 = piece 4 b + j
+  lk_for([&](auto uc) {
+    constexpr int u = decltype(uc)::value, i = u / MT, mt = u % MT;
+    __builtin_amdgcn_s_waitcnt(lk_waitcnt_vm(SCH.allowed[u]));
+    if (mt == 0) {
+      // the registers of this chunk's codes are defined from here on
+      asm volatile("" : "+v"(qw[i]), "+v"(sc[i]));
+      if (FMT == 1) asm volatile("" : "+v"(zw[i]));
+      if (i % 2 == 0 && i + 1 < CH) asm volatile("" : "+v"(qw[i + 1]));
+    }
     __builtin_amdgcn_sched_barrier(0);
-    if (i % 2 == 0 && i + 1 < CH) pair_fix(i / 2);
-    // B operands: MFMA j contracts k = 128 chunk + 32 b + 8 j .. + 7 = piece 4 b + j
-    u4 xv[MT][4];
+    if (mt == 0 && i % 2 == 0 && i + 1 < CH) pair_fix(i / 2);
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        // (lanes of rows past the fetched quads read the last fetched one)
-        xv[mt][j] = *(const u4*)(mine + (((i % NBUF) * MT + mt) * NQ + min(r >> 2, NQ - 1)) * 1024 +
-                                 ((r & 3) * 16 + ((4 * b + j) ^ r)) * 16);
-      }
+    for (int j = 0; j < 4; ++j) {
+      // (lanes of rows past the fetched quads read the last fetched one)
+      xv[mt][j] = *(const u4*)(mine + ((u % NBUF) * NQ + min(r >> 2, NQ - 1)) * 1024 +
+                               ((r & 3) * 16 + ((4 * b + j) ^ r)) * 16);
+    }
     if (wave * CH + i >= nchunks) {  // a chunk past the end of the row: zero activations
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) xv[mt][j] = u4{0u, 0u, 0u, 0u};
+      for (int j = 0; j < 4; ++j) xv[mt][j] = u4{0u, 0u, 0u, 0u};
       // keeps this a branch that only the ragged tail takes (as selects it is 16
       // instructions per chunk for every wave, a fifth of the chunk's vector-ALU work)
       asm volatile("" ::: "memory");
     }
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the buffer is free
     __builtin_amdgcn_sched_barrier(0);
-    if (i + NBUF < CH) request_x(i + NBUF);
+    if (u + NBUF < UN) request_x(u + NBUF);
     __builtin_amdgcn_sched_barrier(0);
+    if (mt != MT - 1) return;  // the chunk's other row tiles first
     if (i % 2 == 0 && 2 * (i / 2 + LK_LAU) < CH) request_codes(i / 2 + LK_LAU);
     __builtin_amdgcn_sched_barrier(0);
 
@@ -295,11 +300,11 @@ __global__ __launch_bounds__(LK_THREADS) void mfma_decode_longk_kernel(
         a = lk_expand_word(qw[i][j], cneg, s2, mask, magic);
       }
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(h8, xv[mt][j]), acc[mt],
+      for (int m2 = 0; m2 < MT; ++m2)
+        acc[m2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(h8, xv[m2][j]), acc[m2],
                                                          0, 0, 0);
     }
-  }, std::make_integer_sequence<int, CH>{});
+  }, std::make_integer_sequence<int, UN>{});
 
   // Fixed-order combine of the 8 K slices: entry mt of wave w goes to red[w][mt]; wave
   // e < MT then sums entry e in wave order and stores it.  The rings are free once
@@ -349,7 +354,7 @@ int lk_cus() {
 
 template <int FMT, int CH, int MT, int NQ>
 hipError_t longk_go(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s) {
-  constexpr int lds_bytes = LK_WAVES * lk_nbuf(MT, NQ) * MT * NQ * 1024;
+  constexpr int lds_bytes = LK_WAVES * lk_nbuf(MT, NQ) * NQ * 1024;
   static bool granted[64] = {};  // more than 64 KB of LDS has to be granted per device, once
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
@@ -373,7 +378,8 @@ hipError_t longk_m(const WView& v, const w4_half* x, w4_half* c, int M, hipStrea
   if (M <= 8) return longk_go<FMT, CH, 1, 2>(v, x, c, M, s);
   if (M <= 12) return longk_go<FMT, CH, 1, 3>(v, x, c, M, s);
   if (M <= 16) return longk_go<FMT, CH, 1, 4>(v, x, c, M, s);
-  return longk_go<FMT, CH, 2, 4>(v, x, c, M, s);
+  if (M <= 32) return longk_go<FMT, CH, 2, 4>(v, x, c, M, s);
+  return longk_go<FMT, CH, 4, 4>(v, x, c, M, s);  // grid.y walks 64 rows at a time
 }
 
 template <int FMT>
@@ -401,10 +407,10 @@ hipError_t longk_fmt(const WView& v, const w4_half* x, w4_half* c, int M, hipStr
 }  // namespace
 
 // 5 to 16 whole chunks of 128 k per wave (2 to 4 on thin grids, see below), whole 16-row
-// tiles, a lane's 32-k slice inside one group, M <= 32, 16-byte aligned codes and
+// tiles, a lane's 32-k slice inside one group, M <= 64, 16-byte aligned codes and
 // activations.
 bool decode_longk_applies(const WView& v, const w4_half* x, const w4_half* c, int M) {
-  if (M < 1 || M > 32 || v.N % 16 || longk_chunks(v.K) == 0) return false;
+  if (M < 1 || M > LK_MAX_M || v.N % 16 || longk_chunks(v.K) == 0) return false;
   if (!v.mx && v.gs % 32) return false;
   if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)c & 7)) return false;
   if (longk_chunks(v.K) < 5) {

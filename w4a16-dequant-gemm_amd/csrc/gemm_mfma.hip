@@ -898,7 +898,7 @@ static hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M
   const bool wvec = (v.K % 32 == 0) && (((uintptr_t)v.q) & 15) == 0;
   const bool resident = wvec && decode_resident_applies(v, x, c, M) &&
                         (w_out == nullptr || ((uintptr_t)w_out & 15) == 0);
-  // long K, M <= 32: the same sums with the requests pipelined chunk by chunk
+  // long K, M <= 64: the same sums with the requests pipelined chunk by chunk
   const bool longk = wvec && decode_longk_applies(v, x, c, M) &&
                      (w_out == nullptr || ((uintptr_t)w_out & 15) == 0);
   if (longk && w_out == nullptr) return launch_decode_longk(v, x, c, M, s);

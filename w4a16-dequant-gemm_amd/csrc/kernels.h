@@ -51,7 +51,7 @@ bool decode_resident_applies(const WView& v, const w4_half* x, const w4_half* c,
 hipError_t launch_decode_resident(const WView& v, const w4_half* x, w4_half* c, int M,
                                   hipStream_t s);
 
-// gemm_decode_longk.hip: M <= 32 at long K (8, 11 or 14 chunks of 128 k per wave), one
+// gemm_decode_longk.hip: M <= 64 at long K (5 to 16 chunks of 128 k per wave; 2 to 4 on thin grids), one
 // 16-row tile per workgroup with activations and codes requested chunk by chunk while
 // earlier chunks multiply; same order of additions as the two kernels above.
 bool decode_longk_applies(const WView& v, const w4_half* x, const w4_half* c, int M);

@@ -14,7 +14,8 @@
 //    contiguous 32-byte-aligned run of 32 G bytes (the zero-point words one of
 //    64 words(G) bytes): the workgroup copies the runs of its T tiles with 16-byte
 //    loads, and every lane then reads the scale and the zero-point word of each of
-//    its packed words from LDS (one group lookup per word, computed once per kernel).
+//    its packed words from LDS (group indices computed once per kernel; a lookup per
+//    word, or two per slice where gs >= 32 allows it).
 //    Gathering them from memory costs a separate request per (row, group) touched:
 //    at gs = 48, N = 11008 that was as much as the shared activations saved.
 //  * rows of packed words are read with 16-byte loads at 4-byte aligned addresses
@@ -49,11 +50,13 @@ __device__ __forceinline__ h8 dg_expand_word(uint32_t w, h2 cneg, h2 s2, uint32_
 
 // ASYM: zero-points.  CH = ceil(ceil(K / 128) / 8) chunks per wave.  T tiles of 16 rows
 // per workgroup (tile blockIdx.x + gridDim.x t), MT tiles of 16 activation rows
-// (blockIdx.y walks M in steps of 16 MT); CPX, if not 0, chunks of x per phase.  A tile's scales are copied with PS = 3 16-byte
+// (blockIdx.y walks M in steps of 16 MT); CPX, if not 0, chunks of x per phase.  GM: how a
+// slice's groups are looked up (2: gs >= 32, first and last word only; 1: gs = 8 or 16,
+// one zero-point word per slice; 0: per word).  A tile's scales are copied with PS = 3 16-byte
 // loads per thread (2 G <= 1536 of them; indices past the run repeat its last piece and
 // are not written).  Arguments are scalars and pointers so that they arrive preloaded
 // in SGPRs.
-template <bool ASYM, int CH, int T, int MT, int CPX>
+template <bool ASYM, int CH, int T, int MT, int CPX, int GM>
 __global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
     const uint32_t* __restrict__ q, const w4_half* __restrict__ scales,
     const uint32_t* __restrict__ zeros, const w4_half* __restrict__ x, w4_half* __restrict__ c,
@@ -175,16 +178,28 @@ __global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
   // Group of each packed word of this lane (the same for every tile), as byte offsets
   // into a tile's parameter block: scale at 2 (r G + g), zero-point word at
   // SB + 4 (r WG + g / 8), nibble g % 8.
-  uint32_t soff[CH][4], zoff[CH][4], zsh[CH][4];
+  // G2 (gs >= 32): the four words of a lane's 32-k slice lie in at most two groups, that
+  // of the first word and that of the last; only those two are looked up, and the
+  // words between take one or the other (four LDS reads and ten vector instructions
+  // less per slice: 13.2 -> 12.4 us at gs = 48, M = 8).
+  // GM == 1 (gs = 8 or 16, which divide 32): the groups of a slice start at a multiple of
+  // 32 / gs, so their zero-points sit in one word, read once per slice.
+  constexpr bool G2 = GM == 2, ZS = GM == 1;
+  constexpr int NL = G2 ? 2 : 4;
+  uint32_t soff[CH][NL], zoff[CH][NL], zsh[CH][NL];
+  bool first[CH][2];  // G2: words 1 and 2 are in the first word's group
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
     int g4[4];
     groups_of_slice(lane_k(i), gs, gs_shift, G - 1, g4);
+    first[i][0] = g4[1] == g4[0];
+    first[i][1] = g4[2] == g4[0];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      soff[i][j] = (uint32_t)(r * G + g4[j]) * 2u;
-      zoff[i][j] = (uint32_t)SB + (uint32_t)(r * WG + (g4[j] >> 3)) * 4u;
-      zsh[i][j] = 4u * (uint32_t)(g4[j] & 7);
+    for (int l = 0; l < NL; ++l) {
+      const int g = g4[G2 ? 3 * l : l];
+      soff[i][l] = (uint32_t)(r * G + g) * 2u;
+      zoff[i][l] = (uint32_t)SB + (uint32_t)(r * WG + (g >> 3)) * 4u;
+      zsh[i][l] = 4u * (uint32_t)(g & 7);
     }
   }
 
@@ -231,9 +246,23 @@ __global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
             if (i >= CH) continue;
             xv[mt][cc][j] = *(const u4*)(mine + ((mt * CP + cc) * 4 + (r >> 2)) * 1024 +
                                          ((r & 3) * 16 + ((4 * b + j) ^ r)) * 16);
-            // chunks past the row's last one, and k past K inside it, contribute nothing
-            if (wave * CH + i >= nchunks || lane_k(i) + 8 * j >= K) xv[mt][cc][j] = u4{0u, 0u, 0u, 0u};
           }
+    }
+    // chunks past the row's last one, and k past K inside it, contribute nothing: a branch
+    // that only the waves at the ragged end of the row take (as selects it was 16
+    // vector instructions per chunk for every wave: 0.5 - 1.7 us per call)
+#pragma unroll
+    for (int cc = 0; cc < CP; ++cc) {
+      const int i = ph * CP + cc;
+      if (i >= CH) continue;
+      if (wave * CH + i >= nchunks - ((K & 127) ? 1 : 0)) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (wave * CH + i >= nchunks || lane_k(i) + 8 * j >= K) xv[mt][cc][j] = u4{0u, 0u, 0u, 0u};
+        asm volatile("" ::: "memory");
+      }
     }
     if (ph + 1 < PH) {
       // the region is free once these reads have returned: ask for the next phase now
@@ -261,13 +290,29 @@ __global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
         if (i >= CH) continue;
         if (ph == 0 && cc == 0) pair_fix(t);
         const uint8_t* pt = params + t * PB;
+        h2 cn[NL], sp[NL];
+        uint32_t zword = 0u;
+        if (ASYM && ZS) zword = *(const uint32_t*)(pt + zoff[i][0]);
+#pragma unroll
+        for (int l = 0; l < NL; ++l) {
+          const uint32_t sbits = *(const uint16_t*)(pt + soff[i][l]);
+          uint32_t z = 8u;
+          if (ASYM) z = ((ZS ? zword : *(const uint32_t*)(pt + zoff[i][l])) >> zsh[i][l]) & 0xFu;
+          cn[l] = as_h2(0xD400E400u | (z << 20) | z);
+          sp[l] = splat_bits(sbits);
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const uint32_t sbits = *(const uint16_t*)(pt + soff[i][j]);
-          uint32_t z = 8u;
-          if (ASYM) z = (*(const uint32_t*)(pt + zoff[i][j]) >> zsh[i][j]) & 0xFu;
-          const h2 cneg = as_h2(0xD400E400u | (z << 20) | z);
-          const h8 a = dg_expand_word(qw[t][i][j], cneg, splat_bits(sbits), mask, magic);
+          h2 cneg, s2;
+          if (!G2) {
+            cneg = cn[j < NL ? j : 0], s2 = sp[j < NL ? j : 0];
+          } else if (j == 0 || j == 3) {
+            cneg = cn[j ? 1 : 0], s2 = sp[j ? 1 : 0];
+          } else {
+            cneg = first[i][j - 1] ? cn[0] : cn[1];
+            s2 = first[i][j - 1] ? sp[0] : sp[1];
+          }
+          const h8 a = dg_expand_word(qw[t][i][j], cneg, s2, mask, magic);
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt)
             acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(h8, xv[mt][cc][j]),
@@ -378,8 +423,8 @@ bool general_plan(const WView& v, const w4_half* x, const w4_half* c, int M, Gen
   return true;
 }
 
-template <bool ASYM, int CH, int T, int MT, int CPX>
-hipError_t general_go(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
+template <bool ASYM, int CH, int T, int MT, int CPX, int GM>
+hipError_t general_gm(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                       const GeneralPlan& pl) {
   // more than 64 KB of LDS has to be granted per device, once per instantiation
   static bool granted[64] = {};
@@ -388,7 +433,7 @@ hipError_t general_go(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
   if (dev < 0 || dev >= 64 || !granted[dev] || granted_bytes[dev] < pl.lds) {
     const hipError_t e =
-        hipFuncSetAttribute((const void*)mfma_decode_general_kernel<ASYM, CH, T, MT, CPX>,
+        hipFuncSetAttribute((const void*)mfma_decode_general_kernel<ASYM, CH, T, MT, CPX, GM>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, pl.lds);
     if (e != hipSuccess) return e;
     if (dev >= 0 && dev < 64) granted[dev] = true, granted_bytes[dev] = pl.lds;
@@ -396,9 +441,19 @@ hipError_t general_go(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
   const int tiles = v.N / 16;
   const int sh = (v.gs & (v.gs - 1)) == 0 ? __builtin_ctz((unsigned)v.gs) : -1;
   const dim3 grid((unsigned)((tiles + T - 1) / T), (unsigned)((M + 16 * MT - 1) / (16 * MT)));
-  mfma_decode_general_kernel<ASYM, CH, T, MT, CPX><<<grid, DG_THREADS, pl.lds, s>>>(
+  mfma_decode_general_kernel<ASYM, CH, T, MT, CPX, GM><<<grid, DG_THREADS, pl.lds, s>>>(
       v.q, (const w4_half*)v.scales, v.zeros, x, c, v.N, v.K, v.gs, sh, v.G, M, tiles);
   return hipGetLastError();
+}
+
+template <bool ASYM, int CH, int T, int MT, int CPX>
+hipError_t general_go(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
+                      const GeneralPlan& pl) {
+  if (v.gs >= 32) return general_gm<ASYM, CH, T, MT, CPX, 2>(v, x, c, M, s, pl);
+  if constexpr (ASYM) {
+    if (32 % v.gs == 0) return general_gm<ASYM, CH, T, MT, CPX, 1>(v, x, c, M, s, pl);
+  }
+  return general_gm<ASYM, CH, T, MT, CPX, 0>(v, x, c, M, s, pl);
 }
 
 template <bool ASYM, int CH, int T>

@@ -81,8 +81,8 @@ const char* w4_last_error(void);
 int w4_dispatch_mma_min_m(void);
 /* The same for one weight matrix: rows of packed words that are not 16-byte aligned
  * (K % 32 != 0) leave the vector kernels their word-by-word form, and on large matrices
- * (N * K >= 2^25) the matrix-core kernel is ahead from M = 3 (N = 11008, K = 4104: M = 3 / 4
- * 31.5 / 32.7 us against 19.5).  So it is for K above 4096 (K % 32 == 0; W4 and MXFP4):
+ * (N * K >= 2^25) the matrix-core kernel is ahead from M = 2 (N = 11008, K = 4104: M = 2 / 4
+ * 19.2 / 32.6 us against 18.5).  So it is for K above 4096 (K % 32 == 0; W4 and MXFP4):
  * three or four activation rows cost the vector kernels a second pass over their
  * staged activations, the matrix-core kernel fetches only the rows that exist
  * (N = 4096, K = 11008, M = 3: 18.2 us against 9.0; up to K = 6144 in whole chunks of

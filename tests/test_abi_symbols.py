@@ -41,7 +41,7 @@ def test_validation_runs_without_a_device():
     # one constant, lowered only for large matrices whose rows are not 16-byte aligned
     assert lib.w4_dispatch_mma_min_m_for(4096, 4096) == lib.w4_dispatch_mma_min_m()
     assert lib.w4_dispatch_mma_min_m_for(64, 4104) == lib.w4_dispatch_mma_min_m()
-    assert lib.w4_dispatch_mma_min_m_for(11008, 4104) == 3
+    assert lib.w4_dispatch_mma_min_m_for(11008, 4104) == 2
     assert lib.w4_dispatch_mma_min_m_for(4096, 11008) == 3
     assert lib.w4_dispatch_mma_min_m_for(4096, 4128) == 3
     assert lib.w4_dispatch_mma_min_m_for(4096, 6144) == 2

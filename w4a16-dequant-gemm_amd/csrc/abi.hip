@@ -169,7 +169,7 @@ const char* w4_last_error(void) { return g_msg; }
 
 int w4_dispatch_mma_min_m(void) { return DISPATCH_MMA_MIN_M; }
 int w4_dispatch_mma_min_m_for(int N, int K) {
-  if (K % 32 != 0 && K % 8 == 0 && (long long)N * K >= (1LL << 25)) return 3;
+  if (K % 32 != 0 && K % 8 == 0 && (long long)N * K >= (1LL << 25)) return 2;
   if (K > 4096 && K <= 6144 && K % 128 == 0) return 2;  // 5.6 - 5.9 us against 6.3 at N = 4096
   if (K > 4096 && K % 32 == 0) return 3;
   return DISPATCH_MMA_MIN_M;

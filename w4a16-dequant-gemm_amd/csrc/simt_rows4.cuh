@@ -116,7 +116,9 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_rows4_kernel(
     // arithmetic still ahead (the slowest wave ended 0.6 us after the median one).
     // Round by round, every wave's run i lands at about the same time and the
     // arithmetic keeps pace with the stream (C1: 3.63 - 3.72 -> 3.50 us in the same runs).
-    if (i + 1 < NQ) asm volatile("s_barrier" ::: "memory");
+    // With three or four activation rows a wave has enough arithmetic per run to keep
+    // up by itself, and the barriers cost (N = 11008: 9.3 -> 9.1 us without them).
+    if (MT <= 2 && i + 1 < NQ) asm volatile("s_barrier" ::: "memory");
   }
 
   if (TL) ts[1] = rows4_now();

@@ -237,6 +237,25 @@ __device__ __forceinline__ int round_half_away_small(float v) {
 }
 __device__ __forceinline__ int round_half_away_small(double v) { return (int)round_half_away(v); }
 
+// round_half_away(v / sf) for FP16-representable v and sf > 0 without the division: a
+// candidate from v * (1 / sf) (a few ulp off, so within one of the answer while
+// |v / sf| <= 64; beyond that every code saturates), then the two tests that define the
+// answer, v - (c -+ 1/2) sf against zero, each one fused multiply-add whose sign is
+// the exact sign (it rounds an exact real, and a nonzero difference of multiples of
+// 2^-25 cannot underflow).  A third fewer vector instructions than the correctly
+// rounded quotient plus its rounding, in a kernel that is bound by them.
+__device__ __forceinline__ int round_quotient_half_away(float v, float sf, float rsf) {
+  const float a = fabsf(v);  // half away from zero: round the magnitude half up, restore the sign
+  const float t = fminf(a * rsf, 64.0f);
+  const float c = rintf(t);
+  const float lo = fmaf(0.5f - c, sf, a);   // |v| - (c - 1/2) sf
+  const float hi = fmaf(-0.5f - c, sf, a);  // |v| - (c + 1/2) sf
+  int m = (int)c;
+  m -= lo < 0.0f ? 1 : 0;  // (straight-line code: as branches this was slower than the division)
+  m += hi >= 0.0f ? 1 : 0;
+  return v < 0.0f ? -m : m;
+}
+
 __device__ __forceinline__ void load8(const double* p, double v[8]) {
   typedef double d2 __attribute__((ext_vector_type(2)));
 #pragma unroll
@@ -279,7 +298,8 @@ __global__ __launch_bounds__(QT) void quantize_rows_fast_kernel(
   bool bad = false;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    bad |= !(fabs((double)v[j]) <= (sizeof(T) == 2 ? 65504.0 : DBL_MAX));
+    if (sizeof(T) == 2) bad |= !(fabsf((float)v[j]) <= 65504.0f);
+    else bad |= !(fabs((double)v[j]) <= DBL_MAX);
     lo = v[j] < lo ? v[j] : lo;
     hi = v[j] > hi ? v[j] : hi;
   }
@@ -351,9 +371,12 @@ __global__ __launch_bounds__(QT) void quantize_rows_fast_kernel(
     *(u2*)(q8 + w * 8) = out;
   } else {
     uint32_t word = 0;
+    const float rsf = __builtin_amdgcn_rcpf(sf);
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const int c = round_half_away_small(v[j] / sfa) + zero;
+      int c;
+      if constexpr (sizeof(T) == 2) c = round_quotient_half_away((float)v[j], sf, rsf) + zero;
+      else c = round_half_away_small(v[j] / sfa) + zero;
       word |= (uint32_t)(c < 0 ? 0 : (c > 15 ? 15 : c)) << (4 * j);
     }
     q32[w] = word;

@@ -77,6 +77,33 @@ __device__ __forceinline__ uint32_t encode_e4m3(float x) {
   return sign | (uint32_t)(code > 0x7E ? 0x7E : code);
 }
 
+// encode_e4m3(v / s) for FP16-representable v and s without the division.  x = v * (1 / s)
+// is within 2^-22 (relative) of the exact quotient q.  q has 11-bit numerator and
+// denominator, so it is either exactly on a midpoint of the E4M3 grid (odd multiples
+// of half a step, at most 31) or at least 2^-16 (relative) away from every one: if x
+// is within 2^-20 of a midpoint, q is that midpoint and the tie goes to the even code;
+// otherwise x and q round alike.  (The host rounds the FP64 quotient to FP32 first,
+// which for the same reason never moves it onto or across a midpoint.)
+__device__ __forceinline__ uint32_t encode_e4m3_quotient(float v, float rs) {
+  const float x = v * rs;
+  const uint32_t sign = (__builtin_bit_cast(uint32_t, x) >> 24) & 0x80u;
+  // straight-line code (as early returns per element the compiler made 16 divergent
+  // regions per thread): saturation is the grid's own top, 448 = 14 steps of 2^5
+  const float a = fminf(fabsf(x), 448.0f);
+  int ex = (int)((__builtin_bit_cast(uint32_t, a) >> 23) & 0xFFu) - 127;
+  ex = ex < -6 ? -6 : ex;
+  const float y = a * __builtin_bit_cast(float, (uint32_t)(130 - ex) << 23);  // exact; 0 .. 16 steps
+  const float f = floorf(y);
+  const float d = fabsf((y - f) - 0.5f);  // distance from the midpoint, exact
+  float r = rintf(y);
+  r = d < y * 0x1p-20f ? f + (float)((int)f & 1) : r;
+  const int steps = (int)r;
+  int code = (ex + 7) * 8 + (steps - 8);  // with ex = -6 this is `steps` itself, subnormal or not
+  code = code > 0x7E ? 0x7E : code;
+  code = x != x ? 0x7F : code;
+  return sign | (uint32_t)code;
+}
+
 __device__ __forceinline__ int pow2_at_least(int n) {
   int p = 1;
   while (p < n) p <<= 1;
@@ -364,7 +391,10 @@ __global__ __launch_bounds__(QT) void quantize_rows_fast_kernel(
   if (MODE == QM_F8) {
     uint32_t b[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) b[j] = encode_e4m3((float)(v[j] / sfa));
+    for (int j = 0; j < 8; ++j) {
+      if constexpr (sizeof(T) == 2) b[j] = encode_e4m3_quotient((float)v[j], __builtin_amdgcn_rcpf(sf));
+      else b[j] = encode_e4m3((float)(v[j] / sfa));
+    }
     u2 out;
     out[0] = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
     out[1] = b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24);

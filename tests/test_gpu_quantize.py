@@ -303,6 +303,55 @@ def test_quantize_cache_f16_sources_on_rounding_ties(f8):
     assert np.array_equal(_host(qv).view(ref.q_v.dtype), ref.q_v)
 
 
+def test_quantize_cache_f8_f16_sources_on_e4m3_midpoints():
+    """FP16 sources whose quotients v / s sit exactly on, and one FP16 ulp either side of, the
+    midpoints of the E4M3 grid (normal and subnormal), for scales with short significands so
+    that midpoint times scale is an FP16 number: the device rounds v * (1 / s) and must give
+    the bytes of the host's division, ties to the even code included."""
+    c = w4amd.capi()
+    rng = np.random.default_rng(777)
+    D = gs = 16
+    rows = []
+    for _ in range(8000):
+        s = np.float16((1 + rng.integers(0, 16) / 16.0) * 2.0 ** rng.integers(-20, 6))
+        with np.errstate(over="ignore"):
+            top = np.float16(448.0 * float(s))
+        if not np.isfinite(top) or float(top) == 0.0:
+            continue
+        e = rng.integers(-6, 9, 14)
+        k = rng.integers(8, 16, 14)
+        mids = (k + 0.5) * 2.0 ** (e - 3)
+        sub = rng.integers(0, 4, 14) == 0
+        mids[sub] = (rng.integers(0, 8, int(sub.sum())) + 0.5) * 2.0 ** -9
+        sgn = rng.integers(0, 2, 14) * 2 - 1
+        with np.errstate(over="ignore"):
+            vals = (sgn * mids * float(s)).astype(np.float16)
+        nudge = rng.integers(-1, 2, 14)
+        vals = (vals.view(np.int16) + nudge.astype(np.int16)).view(np.float16)
+        vals[~np.isfinite(vals) | (np.abs(vals) > np.abs(top))] = 0
+        rows.append(np.concatenate([[top, np.float16(0)], vals]))
+    k16 = np.array(rows, np.float16)
+    v16 = k16[::-1].copy()
+    H, S = 1, k16.shape[0]
+    k, v = k16.astype(np.float64).ravel(), v16.astype(np.float64).ravel()
+    # the rows are what they are meant to be: a fair share of exact midpoints
+    q = np.abs(k16[:, 2:].astype(np.float64) / k16[:, :1].astype(np.float64) * 448.0)
+    steps = q / 2.0 ** (np.floor(np.log2(np.maximum(q, 2.0 ** -6))) - 3)
+    assert np.mean(np.abs(steps - np.floor(steps) - 0.5) == 0) > 0.2
+    kd, vd, st = to_dev(k16.ravel()), to_dev(v16.ravel()), _status()
+    sk = torch.zeros(S, dtype=torch.int16, device=DEV)
+    sv = torch.zeros(S, dtype=torch.int16, device=DEV)
+    ref = orc.quantize_cache_f8(k, v, H, S, D, gs)
+    qk = torch.zeros(S * D, dtype=torch.uint8, device=DEV)
+    qv = torch.zeros(S * D, dtype=torch.uint8, device=DEV)
+    c.quantize_cache_f8(c.kv_f8_view(H, S, D, gs, 1, ptr(qk), ptr(sk), ptr(qv), ptr(sv)),
+                        ptr(kd), ptr(vd), ptr(st), src_f16=True)
+    assert int(_host(st)[0]) == 0
+    assert np.array_equal(_host(sk).view(np.uint16), ref.s_k)
+    assert np.array_equal(_host(qk), ref.q_k)
+    assert np.array_equal(_host(qv), ref.q_v)
+
+
 def test_quantize_cache_f16_sources_every_group_maximum():
     """Every finite FP16 magnitude as the maximum of a group: the scales of FP16 sources
     (an FP32 division on the device, FP64 -> FP32 -> FP16 on the host) agree for all of them."""

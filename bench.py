@@ -801,7 +801,42 @@ def extras_attention(b, full):
     res["fp8_head_scale"] = {"ms": ms, "reps_ms": raw, "bytes": nb8s, "GBs": nb8s / ms * 1e-6,
                              "frac_of_hbm_peak": nb8s / ms * 1e-6 / HBM_PEAK_GBS, "gate": gate}
     res["cpu"] = cpu
-    return {"c5_flash_decode": res}
+    out = {"c5_flash_decode": res}
+    if full:
+        out["attention_sweep_w4_gs128"] = attention_sweep(b)
+    return out
+
+
+def attention_sweep(b):
+    """The shapes of the reference's attention benchmark (bench_attention.cu: H in {32, 8}, S from
+    512 to 32768, D = 128, gs = 128, one query token): W4 flash decode on random codes, rotating
+    through enough cache copies to stay cold.  Timing only (the parity tests hold the kernels)."""
+    torch, capi, st = b.torch, b.capi, b.stream
+    D, gs = 128, 128
+    G, wd = D // gs, D // 8
+    rows = []
+    for H in (32, 8):
+        for S in (512, 2048, 4096, 8192, 32768):
+            nb = 2 * (H * S * wd * 4 + H * S * G * 2)
+            ncopy = min(64, max(2, int(600e6 // nb) + 1))
+            views, keep = [], []
+            for _ in range(ncopy):
+                t = [torch.randint(-2**31, 2**31 - 1, (H * S * wd,), dtype=torch.int32, device="cuda"),
+                     (torch.rand(H * S * G, device="cuda") * 0.2 + 0.1).to(torch.float16),
+                     torch.randint(-2**31, 2**31 - 1, (H * S * wd,), dtype=torch.int32, device="cuda"),
+                     (torch.rand(H * S * G, device="cuda") * 0.2 + 0.1).to(torch.float16)]
+                keep.append(t)
+                views.append(capi.kv_view(H, S, D, gs, G, True, t[0].data_ptr(), t[1].data_ptr(), 0,
+                                          t[2].data_ptr(), t[3].data_ptr(), 0))
+            q = torch.randn(H * D, device="cuda").to(torch.float16)
+            o = torch.empty(H * D, dtype=torch.int16, device="cuda")
+            ms, raw = _reps_ms(torch, lambda i: capi.attention_w4_flash(views[i % ncopy], q.data_ptr(),
+                                                                        o.data_ptr(), st, group=1), 50, 2)
+            rows.append({"H": H, "S": S, "us": ms * 1e3, "reps_us": [r * 1e3 for r in raw], "bytes": nb,
+                         "GBs": nb / ms * 1e-6})
+            del views, keep
+            torch.cuda.empty_cache()
+    return rows
 
 
 def extras_w4a4(b, full):

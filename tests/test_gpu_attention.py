@@ -23,7 +23,10 @@ ATT = [(1, 1, 64, 32), (2, 7, 64, 8), (4, 128, 128, 128), (2, 300, 96, 32), (3, 
        # and gs = 8 (D = 128 on the general kernel)
        (2, 1, 128, 32), (3, 33, 128, 32), (2, 129, 128, 64), (1, 777, 128, 32), (1, 300, 128, 8),
        # head dimension 64 on the matrix-core kernel (gs a multiple of 16)
-       (2, 100, 64, 16), (1, 1, 64, 64), (3, 257, 64, 32)]
+       (2, 100, 64, 16), (1, 1, 64, 64), (3, 257, 64, 32),
+       # either side of the longest cache that one split per slab serves (its kernel writes the
+       # output itself, no merge launch)
+       (2, 512, 128, 32), (2, 513, 128, 32), (1, 512, 64, 16), (2, 400, 128, 64)]
 BIG = [(2, 5000, 64, 32), (1, 9000, 128, 64)]
 # more slabs than workgroups wanted: one split per slab, 9 to 11 tiles per wave
 LONG_SPLITS = [(520, 1300, 128, 32), (600, 1100, 64, 32)]
@@ -107,7 +110,7 @@ def test_w4_flash_grouped_query_head_dim_64(group):
 
 F8 = [(1, 1, 64, 32), (2, 7, 64, 8), (4, 128, 128, 128), (2, 300, 96, 32), (3, 65, 40, 8),
       (1, 9000, 128, 64), (2, 1, 128, 32), (2, 100, 128, 32), (1, 300, 128, 16), (2, 200, 64, 16),
-      (1, 2500, 64, 64)]
+      (1, 2500, 64, 64), (2, 512, 128, 32), (2, 513, 128, 32)]
 
 
 @pytest.mark.parametrize("i", range(len(F8)))

@@ -367,6 +367,12 @@ FlashPlan flash_plan(const FlashArgs& a) {
   int want = (per_cu * 256 + a.H - 1) / a.H;  // splits per slab
   if (want < 1) want = 1;
   if (want > tiles) want = tiles;
+  // Short caches: one split per slab, whose matrix-core kernel writes the output
+  // itself.  The first kernel takes 5.4 us for one tile of 256 positions per workgroup
+  // and 2 us more for every further one, the merge kernel 3.4 us (8.8 us per call for
+  // any S from 512 to 2048 with 32 heads): one more tile costs less than the merge,
+  // two cost more (S = 512: 8.8 -> 7.9 us; S = 1024 would be 9.2 -> 11.9).
+  if (flash_mfma_applies(a) && a.S <= FL_DIRECT_MAX_S) want = 1;
   const int tiles_per = (tiles + want - 1) / want;
   FlashPlan p;
   p.split_len = tiles_per * FL_TILE;
@@ -423,6 +429,7 @@ hipError_t launch_flash(const FlashArgs& a, float* scratch, hipStream_t s) {
   hipError_t e;
   if (try_flash_mfma(a, pl, scratch, s, &e)) {
     if (e != hipSuccess) return e;
+    if (pl.nsplit == 1) return hipSuccess;  // that kernel wrote the output
     flash_phase2<<<(unsigned)(a.H * a.group), P2_THREADS, 0, s>>>(scratch, a.out, pl.nsplit, a.D);
     return hipGetLastError();
   }

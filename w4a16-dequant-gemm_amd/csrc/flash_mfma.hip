@@ -580,6 +580,29 @@ __global__ __launch_bounds__(FM_WAVES * 64) void flash_mfma_phase1(const FlashAr
     mine[FM_D + 1] = m_run * inv_sqrt_d;  // the maximum of the scaled scores
   }
   __syncthreads();
+  if (nsplit == 1) {
+    // One split per slab (short caches): no partials and no second launch.  The value
+    // is the one the merge kernel gives for a single split, sum * (1 / l).
+    for (int i = threadIdx.x; i < nh * FM_D; i += FM_WAVES * 64) {
+      const int h = i / FM_D, j = i - h * FM_D;
+      float mw[FM_WAVES], M = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < FM_WAVES; ++w) {
+        mw[w] = wo[w][h * LDW + FM_D + 1];
+        M = fmaxf(M, mw[w]);
+      }
+      float sum = 0.0f, l = 0.0f;
+#pragma unroll
+      for (int w = 0; w < FM_WAVES; ++w) {
+        const float e = __expf(mw[w] - M);
+        sum += e * wo[w][h * LDW + j];
+        l += e * wo[w][h * LDW + FM_D];
+      }
+      const _Float16 hv = (_Float16)(sum * (1.0f / l));
+      a.out[((long long)slab * a.group + qh0 + h) * FM_D + j] = __builtin_bit_cast(uint16_t, hv);
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < nh * (FM_D + 1); i += FM_WAVES * 64) {
     const int h = i / (FM_D + 1), j = i - h * (FM_D + 1);  // j < 128: O[j]; j == 128: l
     float mw[FM_WAVES], M = -INFINITY;

@@ -91,6 +91,7 @@ struct FlashArgs {
 enum { KIND_F16 = 0, KIND_W4 = 1, KIND_F8 = 2 };  // FlashArgs::kind
 
 // Split of the sequence over workgroups (shared by both phase-1 kernels).
+constexpr int FL_DIRECT_MAX_S = 512;  // longest cache served by one split per slab
 struct FlashPlan {
   int split_len, nsplit;
 };

@@ -172,6 +172,11 @@ int w4_dispatch_mma_min_m_for(int N, int K) {
   if (K % 32 != 0 && K % 8 == 0 && (long long)N * K >= (1LL << 25)) return 2;
   if (K > 4096 && K <= 6144 && K % 128 == 0) return 2;  // 5.6 - 5.9 us against 6.3 at N = 4096
   if (K > 4096 && K % 32 == 0) return 3;
+  // wide matrices at K <= 4096: from about 45 M weights the resident-activation kernel is
+  // ahead at M = 3 and 4 (N = 11008 / 14336, K = 4096, gs = 128: 8.6 / 9.6 us against
+  // 9.4 - 9.8 / 11.7 - 11.8; MXFP4 N = 14336: 8.8 against 9.8 - 10.3; gs = 32 is the exception,
+  // 10.5 against 9.2 - 9.6); N = 8192 still belongs to the vector kernel (6.8 - 7.0 against 7.4)
+  if (K % 32 == 0 && (long long)N * K >= 44000000LL) return 3;
   return DISPATCH_MMA_MIN_M;
 }
 

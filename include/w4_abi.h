@@ -91,6 +91,9 @@ int w4_dispatch_mma_min_m(void);
  * w4_dispatch_mma_min_m().  No counterpart in the reference, whose crossover is one
  * constant (dispatch.cuh:25). */
 int w4_dispatch_mma_min_m_for(int N, int K);
+/* The same for an MXFP4 matrix (what w4_gemm_mx uses): as above, and 2 for K above 4096 other
+ * than 8192 (N = 4096, K = 14336, M = 2: 9.8 us against 11.5).  No counterpart in the reference. */
+int w4_dispatch_mma_min_m_for_mx(int N, int K);
 
 /* ---- packed-weight GEMM: c[M,N] = x[M,K] * W[N,K]^T, FP16 in/out ---------- */
 /* w: N*K halves, bit-identical to the host dequant_all.  dequant.cuh:62-82 */

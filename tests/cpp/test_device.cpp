@@ -142,7 +142,7 @@ void gemm_gates(Checks& t) {
     t.expect(cross(out[0], out[1], ref) <= 2e-3, "mx vector vs matrix kernel");
     Dev<__half> cd((size_t)c.M * c.N);
     gemm_mx(dp, xd.p, cd.p, c.M);
-    t.expect(same(cd.get(), out[c.M < dispatch_mma_min_m(c.N, c.K) ? 0 : 1]), "mx dispatcher output == its callee");
+    t.expect(same(cd.get(), out[c.M < dispatch_mma_min_m_mx(c.N, c.K) ? 0 : 1]), "mx dispatcher output == its callee");
   }
 }
 

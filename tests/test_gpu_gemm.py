@@ -160,7 +160,7 @@ def test_mx_gemm_gates(i):
     assert np.array_equal(wm, w_ref), "mx mma w_out bitwise"
     assert orc.rel_l2(cm.view(np.float16), ref) <= TOL
     cd, wd = _run(c.gemm_mx, dp.view, x_d, M, N, K)
-    want = cf if M < c.load().w4_dispatch_mma_min_m_for(N, K) else cm
+    want = cf if M < c.load().w4_dispatch_mma_min_m_for_mx(N, K) else cm
     assert np.array_equal(cd, want) and np.array_equal(wd, w_ref)
 
 

@@ -52,11 +52,15 @@ __device__ __forceinline__ h8 expand_word(uint32_t w, h2 cneg, h2 s2, uint32_t m
 // workgroup: tile g + gridDim.x t for t < T (tiles past the end are computed on
 // the last tile's rows and not stored).  MT tiles of 16 activation rows (M <= 16 MT).
 //
+// CPV, if not 0, chunks of x per phase: two at MT = 1 halve the region to 8 KB, so that a
+// compute unit holds two workgroups when the grid has more of them than compute units
+// (N = 28672, K = 4096, M = 8: 18.7 -> 17.2 us; on one-round grids the same split is slower,
+// 8.5 -> 9.5 us at N = 11008).
 // A wave's LDS region holds 16 KB: with MT > 1 its slice of x goes through it in MT
 // phases of CP = 4 / MT chunks of 128 k (all MT row tiles of a chunk at a time); the
 // next phase is requested as soon as the current one sits in registers, so it
 // lands while the current one multiplies.
-template <int FMT, int CH, bool POW2, int GSV, int T, int MT>
+template <int FMT, int CH, bool POW2, int GSV, int T, int MT, int CPV = 0>
 __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
     const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
     const int gs_shift, const int tiles) {
@@ -66,7 +70,7 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
   // are fetched from a clamped address and meet zero activations)
   const int K = p.K, WPR = K >> 3, nchunks = K >> 7;
   constexpr bool EXACT = CH == 2 || CH == 4;  // K = 1024 CH by the launcher: every chunk exists
-  constexpr int CP = (4 / MT) < CH ? (4 / MT) : CH;  // chunks per phase
+  constexpr int CP = CPV ? CPV : (4 / MT) < CH ? (4 / MT) : CH;  // chunks per phase
   constexpr int PH = (CH + CP - 1) / CP;              // phases (the last may be partial)
   constexpr int XBYTES = MT * CP * 4096;              // the wave's LDS region
   const int lane = threadIdx.x & 63;
@@ -407,10 +411,12 @@ int resident_chunks(int K) {
   return (per_wave == 8 || per_wave == 11 || per_wave == 14) ? per_wave : 0;
 }
 
-template <int FMT, int CH, bool POW2, int GSV, int T, int MT>
+int device_cus();
+
+template <int FMT, int CH, bool POW2, int GSV, int T, int MT, int CPV = 0>
 hipError_t launch_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
                     int tiles, unsigned grid) {
-  constexpr int CP = (4 / MT) < CH ? (4 / MT) : CH;
+  constexpr int CP = CPV ? CPV : (4 / MT) < CH ? (4 / MT) : CH;
   constexpr int lds_bytes = DR_WAVES * MT * CP * 4096;
   static_assert(DR_WAVES * T * MT * 1024 <= lds_bytes, "the reduction reuses the x regions");
   // more than 64 KB of LDS has to be granted per device, once
@@ -419,12 +425,12 @@ hipError_t launch_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStre
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
   if (dev < 0 || dev >= 64 || !granted[dev]) {
     const hipError_t e =
-        hipFuncSetAttribute((const void*)mfma_decode_resident_kernel<FMT, CH, POW2, GSV, T, MT>,
+        hipFuncSetAttribute((const void*)mfma_decode_resident_kernel<FMT, CH, POW2, GSV, T, MT, CPV>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return e;
     if (dev >= 0 && dev < 64) granted[dev] = true;
   }
-  mfma_decode_resident_kernel<FMT, CH, POW2, GSV, T, MT>
+  mfma_decode_resident_kernel<FMT, CH, POW2, GSV, T, MT, CPV>
       <<<dim3(grid, (unsigned)((M + 16 * MT - 1) / (16 * MT))), DR_THREADS, lds_bytes, s>>>(v, x, c, M, sh,
                                                                                           tiles);
   return hipGetLastError();
@@ -433,7 +439,13 @@ hipError_t launch_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStre
 template <int FMT, int CH, bool POW2, int GSV, int T>
 hipError_t launch_mt(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
                      int tiles, unsigned grid) {
-  if (M <= 16) return launch_t<FMT, CH, POW2, GSV, T, 1>(v, x, c, M, s, sh, tiles, grid);
+  if (M <= 16) {
+    if constexpr (CH == 4 && T == 4) {
+      // more workgroups than compute units: half the LDS each, two per compute unit
+      if ((int)grid > device_cus()) return launch_t<FMT, CH, POW2, GSV, T, 1, 2>(v, x, c, M, s, sh, tiles, grid);
+    }
+    return launch_t<FMT, CH, POW2, GSV, T, 1>(v, x, c, M, s, sh, tiles, grid);
+  }
   if (M <= 32) return launch_t<FMT, CH, POW2, GSV, T, 2>(v, x, c, M, s, sh, tiles, grid);
   return launch_t<FMT, CH, POW2, GSV, T, 4>(v, x, c, M, s, sh, tiles, grid);
 }

@@ -130,6 +130,7 @@ __global__ __launch_bounds__(LK_THREADS) void mfma_decode_longk_kernel(
   constexpr int NBUF = lk_nbuf(MT, NQ), LK_LAU = lk_lau(MT, NQ), NSC = FMT == 1 ? 2 : 1, UN = CH * MT;
   constexpr LkSched<UN> SCH = lk_schedule<CH, MT, NQ, NSC>();
   static_assert(SCH.peak < 64, "vmcnt is a 6-bit counter");
+  static_assert(SCH.allowed[UN - 1] == 0, "the last unit waits for every request");
   static_assert(MT == 1 || NQ == 4, "several row tiles: whole tiles of 16 rows");
   constexpr int XBYTES = NBUF * NQ * 1024;  // the wave's ring: NBUF units of NQ KB
   const int WPR = K >> 3, nchunks = K >> 7;

@@ -80,7 +80,9 @@ struct Shape { int M, N, K, gs; };
 const Shape kShapes[] = {{1, 64, 64, 8},    {8, 128, 96, 16},  {16, 256, 100, 32}, {4, 96, 72, 48},
                          {2, 32, 128, 64},  {3, 40, 256, 128}, {5, 72, 40, 8},     {17, 64, 128, 16},
                          {33, 48, 104, 24}, {20, 32, 100, 8},  {65, 96, 100, 16},  {1, 256, 4096, 128},
-                         {12, 80, 2048, 32}};
+                         {12, 80, 2048, 32},
+                         // long K: K-split vector kernel (M <= 2), pipelined matrix-core kernel above
+                         {2, 32, 11008, 128}, {3, 32, 8192, 64},   {24, 16, 14336, 32}};
 
 void gemm_gates(Checks& t) {
   const BlasHandle blas = make_blas();

@@ -80,6 +80,8 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         (33, 32, 11008, 128), (64, 16, 14336, 32), (50, 32, 8192, 64), (47, 16, 5120, 128), (64, 16, 16384, 128),
         # more workgroups of four tiles than compute units: two chunks of activations per phase
         (6, 16448, 4096, 64),
+        # ... and five to seven tiles per workgroup in one round (fused gate / up projections)
+        (9, 22016, 4096, 128), (16, 28672, 4096, 32),
         # ... and K <= 4096 on grids of at most one tile per compute unit
         (6, 2064, 4096, 128), (8, 4096, 2048, 32), (7, 32, 3072, 64), (20, 48, 2560, 32), (32, 16, 1536, 128),
         (3, 16, 1152, 32),

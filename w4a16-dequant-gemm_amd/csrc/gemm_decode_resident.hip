@@ -461,7 +461,15 @@ hipError_t launch_ch(const WView& v, const w4_half* x, w4_half* c, int M, hipStr
       case 1: return launch_mt<FMT, CH, POW2, GSV, 1>(v, x, c, M, s, sh, tiles, grid);
       case 2: return launch_mt<FMT, CH, POW2, GSV, 2>(v, x, c, M, s, sh, tiles, grid);
       case 3: return launch_mt<FMT, CH, POW2, GSV, 3>(v, x, c, M, s, sh, tiles, grid);
-      default: return launch_mt<FMT, CH, POW2, GSV, 4>(v, x, c, M, s, sh, tiles, grid);
+      case 4: return launch_mt<FMT, CH, POW2, GSV, 4>(v, x, c, M, s, sh, tiles, grid);
+      default:
+        // five to seven tiles: K = 4096, one activation row tile (decode_resident_tiles())
+        if constexpr (CH == 4) {
+          if (T == 5) return launch_t<FMT, CH, POW2, GSV, 5, 1>(v, x, c, M, s, sh, tiles, grid);
+          if (T == 6) return launch_t<FMT, CH, POW2, GSV, 6, 1>(v, x, c, M, s, sh, tiles, grid);
+          if (T == 7) return launch_t<FMT, CH, POW2, GSV, 7, 1>(v, x, c, M, s, sh, tiles, grid);
+        }
+        return hipErrorInvalidValue;
     }
   }
 }
@@ -540,7 +548,10 @@ int decode_resident_tiles(const WView& v, const w4_half* x, const w4_half* c, in
   // tiles per workgroup: enough that one workgroup per compute unit covers N, at
   // most four (more workgroups than compute units beyond that)
   int T = (v.N / 16 + cus - 1) / cus;
-  if (T > 4) T = 4;
+  // (five to seven at K = 4096 with one activation row tile, where one round of longer
+  // workgroups beats two rounds of four-tile ones: N = 22016 / 28672, the fused gate and up
+  // projections of the 11008- and 14336-wide MLPs)
+  if (T > 4 && !(T <= 7 && M <= 16 && v.K == 4096)) T = 4;
   if (resident_chunks(v.K) > 4) T = 1;
   // the one combination that does not fit the register file: four tiles, four row
   // tiles, zero-points and per-chunk scale loads

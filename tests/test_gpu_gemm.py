@@ -80,8 +80,6 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         (33, 32, 11008, 128), (64, 16, 14336, 32), (50, 32, 8192, 64), (47, 16, 5120, 128), (64, 16, 16384, 128),
         # more workgroups of four tiles than compute units: two chunks of activations per phase
         (6, 16448, 4096, 64),
-        # ... and five to seven tiles per workgroup in one round (fused gate / up projections)
-        (9, 22016, 4096, 128), (16, 28672, 4096, 32),
         # ... and K <= 4096 on grids of at most one tile per compute unit
         (6, 2064, 4096, 128), (8, 4096, 2048, 32), (7, 32, 3072, 64), (20, 48, 2560, 32), (32, 16, 1536, 128),
         (3, 16, 1152, 32),
@@ -94,6 +92,10 @@ CFGS = [(1, 64, 64, 8), (8, 128, 96, 16), (16, 256, 100, 32), (4, 96, 72, 48),
         (9, 4128, 4096, 48), (50, 4128, 4104, 8), (16, 8208, 2048, 24), (64, 4112, 3072, 48),
         (30, 64, 5000, 40), (8, 32, 1160, 8), (33, 48, 2568, 16)]
 TOL, CROSS = 1e-3, 2e-3  # rel L2 vs the FP64 oracle; between two gated paths
+# five to eight tiles per workgroup in one round (fused gate / up projections, a 32000-row
+# head), one and two activation row tiles: (M, N, K, gs, symmetric)
+WIDE = [(9, 22016, 4096, 128, True), (16, 28672, 4096, 32, False), (7, 32000, 4096, 64, True),
+        (24, 20480, 4096, 128, False), (32, 28672, 4096, 64, True)]
 
 
 def _run(fn, view, x_d, M, N, K, hook=True):
@@ -101,6 +103,25 @@ def _run(fn, view, x_d, M, N, K, hook=True):
     w_d = halves(N * K, 0x7E00) if hook else None
     fn(view, ptr(x_d), ptr(c_d), M, 0, ptr(w_d))
     return bits(c_d), (bits(w_d) if hook else None)
+
+
+@pytest.mark.parametrize("i", range(len(WIDE)))
+def test_w4_wide_grids(i):
+    """The matrix-core entry on grids of more than four tiles per compute unit: oracle gate,
+    hook bytes, hooked == unhooked."""
+    c = w4amd.capi()
+    M, N, K, gs, sym = WIDE[i]
+    seed = 0x51DE ^ (i * 977)
+    p = orc.quantize(orc.normal_weights(N * K, seed), N, K, gs, sym)
+    w_ref = orc.dequant_all(p)
+    x = orc.normal_activations(M * K, seed + 1)
+    ref = orc.gemm_oracle(x, M, K, w_ref, N)
+    dp, x_d = DevPacked(p), to_dev(x)
+    cm, wm = _run(c.gemm_mma, dp.view, x_d, M, N, K)
+    assert np.array_equal(wm, w_ref), "mma w_out bitwise"
+    assert orc.rel_l2(cm.view(np.float16), ref) <= TOL
+    cm2, _ = _run(c.gemm_mma, dp.view, x_d, M, N, K, hook=False)
+    assert np.array_equal(cm, cm2)
 
 
 @pytest.mark.parametrize("sym", [True, False], ids=["sym", "asym"])

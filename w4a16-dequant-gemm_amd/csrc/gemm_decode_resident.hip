@@ -204,7 +204,10 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
       for (int i = 0; i < CH; ++i) {
         // half index PER i + sub: dword (PER i + sub) / 2, upper half if odd
         uint32_t d;
-        if constexpr (PER == 4) d = (sub & 2) ? w[2 * i + 1] : w[2 * i];
+        // (a bitwise select: written as a conditional the compiler indexed the array
+        // with the condition, which put it in scratch memory -- two stores and four
+        // dependent loads per tile through the memory path, 1.8 us per call at gs = 32)
+        if constexpr (PER == 4) d = w[2 * i] ^ ((w[2 * i] ^ w[2 * i + 1]) & (0u - (uint32_t)((sub >> 1) & 1)));
         else if constexpr (PER == 2) d = w[i];
         else d = w[i >> 1];
         const bool hi = PER == 1 ? (i & 1) : (sub & 1);
@@ -463,11 +466,19 @@ hipError_t launch_ch(const WView& v, const w4_half* x, w4_half* c, int M, hipStr
       case 3: return launch_mt<FMT, CH, POW2, GSV, 3>(v, x, c, M, s, sh, tiles, grid);
       case 4: return launch_mt<FMT, CH, POW2, GSV, 4>(v, x, c, M, s, sh, tiles, grid);
       default:
-        // five to seven tiles: K = 4096, one activation row tile (decode_resident_tiles())
+        // five to eight tiles: K = 4096, one activation row tile (decode_resident_tiles())
         if constexpr (CH == 4) {
-          if (T == 5) return launch_t<FMT, CH, POW2, GSV, 5, 1>(v, x, c, M, s, sh, tiles, grid);
-          if (T == 6) return launch_t<FMT, CH, POW2, GSV, 6, 1>(v, x, c, M, s, sh, tiles, grid);
-          if (T == 7) return launch_t<FMT, CH, POW2, GSV, 7, 1>(v, x, c, M, s, sh, tiles, grid);
+          if (M <= 16) {
+            if (T == 5) return launch_t<FMT, CH, POW2, GSV, 5, 1>(v, x, c, M, s, sh, tiles, grid);
+            if (T == 6) return launch_t<FMT, CH, POW2, GSV, 6, 1>(v, x, c, M, s, sh, tiles, grid);
+            if (T == 7) return launch_t<FMT, CH, POW2, GSV, 7, 1>(v, x, c, M, s, sh, tiles, grid);
+            if (T == 8) return launch_t<FMT, CH, POW2, GSV, 8, 1>(v, x, c, M, s, sh, tiles, grid);
+          } else {
+            if (T == 5) return launch_t<FMT, CH, POW2, GSV, 5, 2>(v, x, c, M, s, sh, tiles, grid);
+            if (T == 6) return launch_t<FMT, CH, POW2, GSV, 6, 2>(v, x, c, M, s, sh, tiles, grid);
+            if (T == 7) return launch_t<FMT, CH, POW2, GSV, 7, 2>(v, x, c, M, s, sh, tiles, grid);
+            if (T == 8) return launch_t<FMT, CH, POW2, GSV, 8, 2>(v, x, c, M, s, sh, tiles, grid);
+          }
         }
         return hipErrorInvalidValue;
     }
@@ -548,10 +559,10 @@ int decode_resident_tiles(const WView& v, const w4_half* x, const w4_half* c, in
   // tiles per workgroup: enough that one workgroup per compute unit covers N, at
   // most four (more workgroups than compute units beyond that)
   int T = (v.N / 16 + cus - 1) / cus;
-  // (five to seven at K = 4096 with one activation row tile, where one round of longer
+  // (five to eight at K = 4096 with one activation row tile, where one round of longer
   // workgroups beats two rounds of four-tile ones: N = 22016 / 28672, the fused gate and up
   // projections of the 11008- and 14336-wide MLPs)
-  if (T > 4 && !(T <= 7 && M <= 16 && v.K == 4096)) T = 4;
+  if (T > 4 && !(T <= 8 && M <= 32 && v.K == 4096)) T = 4;
   if (resident_chunks(v.K) > 4) T = 1;
   // the one combination that does not fit the register file: four tiles, four row
   // tiles, zero-points and per-chunk scale loads

@@ -249,7 +249,10 @@ hipError_t launch_decode(const w4_packed_mx_view& w, const void* xq, const uint8
   // its X rows through L2): worth it from three X tiles on, while a workgroup per
   // CU remains (N = 14336, M = 64: 21.8 us with three row tiles, 29.5 us with one)
   const int nt = MT >= 3 ? tiles * mblocks / 256 : 1;
-  if (nt >= 3) return launch_decode_nt<MT, 3, XF8>(w, xq, xs, M, c, s);
+  // (four X tiles times three row tiles do not fit the register file: that instantiation
+  // spills 37 - 85 VGPRs, N = 14336, M = 64: 22.2 / 42.7 us with MXFP4 / MXFP8 activations
+  // against 18.3 / 27.1 with two row tiles)
+  if (nt >= 3 && MT < 4) return launch_decode_nt<MT, 3, XF8>(w, xq, xs, M, c, s);
   if (nt >= 2) return launch_decode_nt<MT, 2, XF8>(w, xq, xs, M, c, s);
   return launch_decode_nt<MT, 1, XF8>(w, xq, xs, M, c, s);
 }

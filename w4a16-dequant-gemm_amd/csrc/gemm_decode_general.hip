@@ -403,6 +403,8 @@ bool general_plan(const WView& v, const w4_half* x, const w4_half* c, int M, Gen
   // phase to make room for the parameter blocks
   int want = (v.N / 16 + cus - 1) / cus;
   if (want > 4) want = 4;
+  // (four tiles, four activation row tiles and five chunks per wave spill 12 - 28 VGPRs)
+  if (mt == 4 && ch == 5 && want > 3) want = 3;
   auto fit = [&](int cpd, int* lds) {
     const int cp = cpd < ch ? cpd : ch;
     const int xbytes = DG_WAVES * mt * cp * 4096;

@@ -414,6 +414,10 @@ bool decode_longk_applies(const WView& v, const w4_half* x, const w4_half* c, in
   if (M < 1 || M > LK_MAX_M || v.N % 16 || longk_chunks(v.K) == 0) return false;
   if (!v.mx && v.gs % 32) return false;
   if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)c & 7)) return false;
+  // K up to 5120 on grids of more than one tile per compute unit, W4: from M = 9 the kernel
+  // that shares a workgroup's activations between several tiles is ahead (N = 16384,
+  // K = 5120, M = 16 / 32 / 64: 17.7 / 20.0 / 35.8 us against 21.3 / 31.3 / 42.0; M = 8: 17.2 against 17.0)
+  if (longk_chunks(v.K) == 5 && !v.mx && M > 8 && v.N / 16 > lk_cus()) return false;
   if (longk_chunks(v.K) < 5) {
     // Shorter K: only where the kernels that share x between the tiles of a workgroup
     // would have one tile per workgroup too (N / 16 <= compute units).  At K = 2048 and

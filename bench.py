@@ -1,15 +1,19 @@
 #!/usr/bin/env python3
 """Benchmark of the fused-dequant hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--reps R] [--extras none|quick|full]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--reps R] [--extras none|quick|full] [--out FILE]
     python bench.py --probe floor|c1|decode|prefill|quantize|w4a4|attention
 
-Prints ONE JSON line.  The headline workload is the W4A16 symmetric gs=128,
+The LAST line of stdout is the graded record: one JSON object of under 1.5 KB
+(metric, value, ms_per_step, config, roofline, cpu_baseline and a dozen summary
+scalars).  The detailed records come before it, one JSON line per section
+({"section": ...}, each a few KB), and --out FILE writes everything as one
+document.  The headline workload is the W4A16 symmetric gs=128,
 M=1, N=K=4096 fused GEMM; one "step" is one call of w4_gemm on it.  After W
 untimed warm-up steps the benchmark times R repetitions of exactly K steps each
 (HIP events on the launch stream around a C launch loop, no interpreter between
 launches); `ms_per_step` is the median repetition, every repetition is kept in
-`extra.headline.cold_reps_ms`.  `value` is the achieved HBM rate: algorithmic
+the `headline` section (`cold_reps_ms`).  `value` is the achieved HBM rate: algorithmic
 bytes (packed codes + scales + x + c = 8 667 136 B) divided by that time, with
 the weights rotated through enough distinct copies that no step finds its
 matrix in the 256 MB last-level cache ("cold").
@@ -20,7 +24,7 @@ k_out / v_out) equals the oracle's bytes, the unhooked call gives the same
 output bytes as the hooked one, and sampled outputs are within rel L2 1e-3 of
 the FP64 oracle.  The same figure with one hot copy, the measured streaming
 read and copy rates, the launch floor, the other configs of the scope table
-and the CPU oracle's times for the same operations ride along in `extra`.
+and the CPU oracle's times for the same operations are the section lines.
 """
 import argparse
 import ctypes as C
@@ -33,6 +37,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
+FINAL_LINE_MAX = 1536  # bytes: the graded record must survive a harness that keeps a short tail of stdout
 MFMA_F16_PEAK_TFLOPS = 2500.0
 PREWARM_LAUNCHES = 2000
 TOL = 1e-3
@@ -1013,6 +1018,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--reps", type=int, default=9, help="repetitions of the K timed steps (median reported)")
     ap.add_argument("--extras", choices=["none", "quick", "full"], default="quick")
+    ap.add_argument("--out", default=None, help="also write the full record (graded line + every section) to this file")
     ap.add_argument("--probe", choices=["floor", "c1", "decode", "longk", "prefill", "quantize", "w4a4", "attention"],
                     default=None, help="run only a short fixed workload (for counter collection) and exit")
     args = ap.parse_args()
@@ -1060,25 +1066,92 @@ def main():
         legs.update({"c5_" + k: v for k, v in extra["c5_flash_decode"]["cpu"].items()})
     line = {
         "metric": "M=1 W4 GEMM us + achieved HBM GB/s (% of peak); M=2048 MFMA TFLOP/s",
-        "value": cold_gbs, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": h["cold_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "value": _r(cold_gbs, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": _r(h["cold_ms"], 7), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "W4A16 symmetric gs=128 fused GEMM, M=1, N=4096, K=4096 (north_star target "
-                               "shape; weights rotated through %d HBM copies; median of %d repetitions of "
-                               "%d steps)" % (h["copies"], len(h["cold_reps_ms"]), args.steps),
-                   "entry": "w4_gemm", "bytes_per_step": h["bytes"], "reps": len(h["cold_reps_ms"])},
-        "roofline": {"bound": "hbm", "achieved": cold_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": cold_gbs / HBM_PEAK_GBS, "traffic": HEADLINE_TRAFFIC_BYTES},
-        "cpu_baseline": {"value": h["bytes"] / cpu["fused_equiv_s"] * 1e-9, "unit": "GB/s",
-                         "cores": 1, "kind": "port", "cpu_model": host["model"],
-                         "host_logical_cpus": host["logical_cpus"], "host_usable_cpus": host["usable_cpus"],
-                         "sample": "oracle dequant_all + gemm_oracle on the same 4096x4096 matrix, one thread, "
-                                   "median of 5 (%.3f s); other legs in `legs` (seconds, one thread, once each)"
-                                   % cpu["fused_equiv_s"],
-                         "legs": legs},
-        "extra": extra,
+        "config": {"workload": "C1: W4A16 sym gs=128 fused GEMM M=1 N=K=4096, cold weights (%d HBM copies), "
+                               "median of %d x %d steps" % (h["copies"], len(h["cold_reps_ms"]), args.steps),
+                   "entry": "w4_gemm", "bytes_per_step": h["bytes"]},
+        "roofline": {"bound": "hbm", "achieved": _r(cold_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": _r(cold_gbs / HBM_PEAK_GBS, 4), "traffic": HEADLINE_TRAFFIC_BYTES},
+        "cpu_baseline": {"value": _r(h["bytes"] / cpu["fused_equiv_s"] * 1e-9, 5), "unit": "GB/s",
+                         "cores": 1, "kind": "port",
+                         "sample": "oracle dequant_all+gemm_oracle, same 4096x4096 matrix, 1 thread of %d, "
+                                   "median of 5 (%.3f s)" % (host["usable_cpus"], cpu["fused_equiv_s"])},
+        "summary": summarize(extra, cold_gbs),
     }
-    print(json.dumps(line))
+    emit(line, extra, legs, args.out)
+
+
+def _r(v, n):
+    return round(float(v), n)
+
+
+def summarize(extra, cold_gbs):
+    """At most a dozen scalars for the graded line: yardsticks, C4, the worst C2 / C3 cases, C5 per format."""
+    s = {"c1_us": _r(extra["cold_us"], 3),
+         "copy_GBs": _r(extra["yardstick"]["copy_GBs"], 0),
+         "c1_frac_of_copy": _r(extra["cold_frac_of_measured_copy"], 3)}
+    if "launch_floor" in extra:
+        s["read_only_c1_us"] = _r(extra["launch_floor"]["read_c1_8MiB_us"], 3)
+    if "c4_prefill" in extra:
+        c4 = extra["c4_prefill"]
+        s["c4_TFLOPs"] = _r(c4["fused_TFLOPs"], 1)
+        s["c4_frac_mfma"] = _r(c4["frac_of_mfma_peak"], 3)
+        s["c4_two_pass_TFLOPs"] = _r(c4["two_pass_TFLOPs"], 1)
+        s["c4_hipblaslt_TFLOPs"] = _r(c4["hipblaslt_only_TFLOPs"], 1)
+    for key, name in (("c2_w4_asym", "c2"), ("c3_mxfp4", "c3")):
+        rows = extra.get(key)
+        if rows:
+            w = min(rows, key=lambda r: r["frac_of_hbm_peak"])
+            b = max(rows, key=lambda r: r["frac_of_hbm_peak"])
+            s[name + "_worst_frac_hbm"] = _r(w["frac_of_hbm_peak"], 3)
+            s[name + "_worst_case"] = "N%d K%d M%d" % (w["N"], w["K"], w["M"]) + (" gs%d" % w["gs"] if "gs" in w else "")
+            s[name + "_best_frac_hbm"] = _r(b["frac_of_hbm_peak"], 3)
+    c5 = extra.get("c5_flash_decode")
+    if c5:
+        s["c5_frac_hbm"] = {k: _r(c5[k]["frac_of_hbm_peak"], 3) for k in
+                            ("fp16", "w4_gs32", "paged_w4_page16", "fp8_row_scale", "fp8_head_scale") if k in c5}
+    s["wall_s"] = _r(extra["bench_wall_s"], 1)
+    return s
+
+
+def section_lines(extra, legs):
+    """The detailed records as one JSON line per section, each small enough to survive a log tail."""
+    scalars = {k: v for k, v in extra.items() if not isinstance(v, (dict, list))}
+    lines = [{"section": "run", **scalars, "host_cpu": extra.get("host_cpu")},
+             {"section": "cpu_baseline_legs_s", **legs}]
+    for k, v in extra.items():
+        if k == "host_cpu" or not isinstance(v, (dict, list)):
+            continue
+        if isinstance(v, list) and len(json.dumps(v)) > 5000:  # long sweeps: a few rows per line
+            step = max(1, len(v) * 4000 // len(json.dumps(v)))
+            for i in range(0, len(v), step):
+                lines.append({"section": k, "part": i // step, "rows": v[i:i + step]})
+        elif k == "c1_timeline":
+            lines.append({"section": k, "waves": v.get("waves"), "tick_ns": v.get("tick_ns"),
+                          "launches": v.get("launches", [])[:1]})
+        else:
+            lines.append({"section": k, "data": v})
+    return lines
+
+
+def emit(line, extra, legs, out_path):
+    """Sections first, the graded record last and short: a harness that keeps only the end of stdout
+    still gets metric, value, roofline and cpu_baseline whole."""
+    for rec in section_lines(extra, legs):
+        print(json.dumps(rec))
+    if out_path:
+        try:
+            os.makedirs(os.path.dirname(os.path.abspath(out_path)), exist_ok=True)
+            with open(out_path, "w") as f:
+                json.dump({**line, "cpu_baseline_legs_s": legs, "extra": extra}, f)
+        except OSError as e:
+            print("bench.py: could not write %s: %s" % (out_path, e), file=sys.stderr)
+    final = json.dumps(line)
+    assert len(final) < FINAL_LINE_MAX, "graded line grew to %d bytes" % len(final)
+    sys.stdout.flush()
+    print(final, flush=True)
 
 
 if __name__ == "__main__":

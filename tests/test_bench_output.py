@@ -22,6 +22,8 @@ def _canned_extra():
            "frac_of_hbm_peak": 0.6 / M ** 0.25} for M in (1, 16, 128)]
     fmt = {"ms": 0.058, "reps_ms": reps[:5], "bytes": 301989888, "GBs": 5168.8, "frac_of_hbm_peak": 0.646,
            "gate": {"hooks_bitwise": True, "unhooked_equals_hooked": True, "rel_l2_sampled": 2.8e-4}}
+    paged = {"ms": 0.062, "reps_ms": reps[:5], "bytes_logical": 301989888, "bytes_unique": 273678336,
+             "GBs_unique": 4415.0, "frac_of_hbm_peak_unique": 0.552, "vs_contiguous": 0.97, "gate": fmt["gate"]}
     return {
         "headline": {"N": 4096, "K": 4096, "gs": 128, "M": 1, "bytes": 8667136, "copies": 47,
                      "cold_ms": 0.0036, "cold_reps_ms": reps, "warm_reps_ms": reps},
@@ -35,7 +37,8 @@ def _canned_extra():
         "c3_mxfp4": c3,
         "c4_prefill": {"M": 2048, "fused_TFLOPs": 905.1, "two_pass_TFLOPs": 875.2,
                        "hipblaslt_only_TFLOPs": 995.4, "frac_of_mfma_peak": 0.362, "fused_reps_ms": reps},
-        "c5_flash_decode": {"B": 8, "w4_gs32": fmt, "paged_w4_page16": fmt, "fp16": fmt,
+        "c5_flash_decode": {"B": 8, "w4_gs32": fmt, "paged_w4_page16": paged,
+                            "w4_gs32_noalloc_entry": {"ms": 0.0599, "reps_ms": reps[:5], "equals_allocating_entry": True}, "fp16": fmt,
                             "fp8_row_scale": fmt, "fp8_head_scale": fmt, "cpu": {"a_s": 0.07}},
         "bench_wall_s": 28.1,
     }

@@ -20,9 +20,9 @@ matrix in the 256 MB last-level cache ("cold").
 
 Every timed case first passes its gate at bench size on data quantized by the
 CPU oracle from the distribution its config names: the dequant hook (w_out /
-k_out / v_out) equals the oracle's bytes, the unhooked call gives the same
-output bytes as the hooked one, and sampled outputs are within rel L2 1e-3 of
-the FP64 oracle.  The same figure with one hot copy, the measured streaming
+k_out / v_out) equals the oracle's bytes, the unhooked call is within rel L2
+2e-3 of the hooked one (attention: the same bytes), and sampled outputs of both
+are within rel L2 1e-3 of the FP64 oracle.  The same figure with one hot copy, the measured streaming
 read and copy rates, the launch floor, the other configs of the scope table
 and the CPU oracle's times for the same operations are the section lines.
 """
@@ -41,6 +41,7 @@ FINAL_LINE_MAX = 1536  # bytes: the graded record must survive a harness that ke
 MFMA_F16_PEAK_TFLOPS = 2500.0
 PREWARM_LAUNCHES = 2000
 TOL = 1e-3
+CROSS_TOL = 2e-3  # between two gated GEMM paths (the reference's fused-vs-two-pass bound, tests/test_gpu.cu:184-193)
 # HBM bytes one launch of the headline kernel moves, from two rocprofv3 --pmc runs
 # of `python3 bench.py --probe c1` (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch
 # of simt_rows4_kernel), each scaled by what the same counter reads for the 1 GiB
@@ -330,7 +331,8 @@ def quant_rel_l2(np, w, w16):
 
 class Gate:
     """Bench-size correctness gate of one packed matrix: hook bytes against the oracle's
-    dequant, unhooked output == hooked output, sampled rows within TOL of the FP64 oracle."""
+    dequant (bit-exact), unhooked output within CROSS_TOL of the hooked output, sampled rows of
+    both within TOL of the FP64 oracle."""
 
     def __init__(self, b, mx, p, w_ref, N, K):
         self.b, self.mx, self.p, self.w_ref, self.N, self.K = b, mx, p, w_ref, N, K
@@ -354,15 +356,18 @@ class Gate:
         c_u = halves(M * N, 0x7E00)
         fn(view, ptr(x_d), ptr(c_u), M, self.b.stream, 0)
         got_h, got_u = bits(c_h), bits(c_u)
-        same = bool(np.array_equal(got_h, got_u))
+        fh, fu = got_h.view(np.float16).astype(np.float64), got_u.view(np.float16).astype(np.float64)
+        cross = float(np.sqrt(np.sum((fu - fh) ** 2) / max(np.sum(fh * fh), 1e-300)))
         ms = min(M, 16)  # activation rows sampled for the FP64 oracle
         xs = np.ascontiguousarray(x_host.reshape(M, K)[:ms])
         ref = orc.gemm_oracle(xs, ms, K, self.w_rows, len(self.rows))
         got = got_u.view(np.float16).reshape(M, N)[:ms][:, self.rows]
         rel = orc.rel_l2(got, ref)
-        ok = hook_ok and same and rel <= TOL
-        self.results.append({"case": label, "hook_bitwise": hook_ok, "unhooked_equals_hooked": same,
-                             "rel_l2_sampled": rel, "ok": ok})
+        got_hk = got_h.view(np.float16).reshape(M, N)[:ms][:, self.rows]
+        rel_h = orc.rel_l2(got_hk, ref)
+        ok = hook_ok and cross <= CROSS_TOL and rel <= TOL and rel_h <= TOL
+        self.results.append({"case": label, "hook_bitwise": hook_ok, "unhooked_vs_hooked_rel_l2": cross,
+                             "rel_l2_sampled": rel, "rel_l2_sampled_hooked": rel_h, "ok": ok})
         if not ok:
             raise RuntimeError("bench-size gate failed: %s" % json.dumps(self.results[-1]))
         return ok

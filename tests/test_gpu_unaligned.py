@@ -20,7 +20,7 @@ import torch
 
 import orc
 import w4amd
-from devutil import DEV, bits, f64, ptr
+from devutil import DEV, bits, cross_gate, f64, ptr
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-3
@@ -89,11 +89,8 @@ def test_w4_gemm_unaligned_bases(i, sym):
             assert c_d.guards_intact() and w_d.guards_intact(), "wrote outside c / w_out"
             c2 = out_buf(M * N, oc)
             fn(view, x_d.ptr, c2.ptr, M, 0, 0)
-            # a w_out that is not 16-byte aligned sends the hooked call to a kernel with
-            # narrower stores and another order of additions: same gate, other bytes
-            if ow % 16 == 0:
-                assert np.array_equal(c2.get(), c_d.get()), "hooked and unhooked bytes differ"
-            assert orc.rel_l2(c2.get().view(np.float16), ref) <= TOL and c2.guards_intact()
+            cross_gate(c_d.get(), c2.get(), ref, fn.__name__)
+            assert c2.guards_intact()
         w_d = out_buf(N * K, ow)
         c.dequant(view, w_d.ptr)
         assert np.array_equal(w_d.get(), w_ref) and w_d.guards_intact()

@@ -160,6 +160,45 @@ __device__ __forceinline__ float dot2(h2 a, h2 b, float acc) {
   return __builtin_amdgcn_fdot2(a, b, acc, false);
 }
 
+// ---- W4 with the scale and the zero-point outside the inner loop ---------------------
+// For results that are not dequantized weights (GEMM outputs of calls without the w_out
+// hook):  sum_k x_k s (n_k - z)  =  s * ( sum_k x_k (b_k + n_k)  -  sum_k x_k (b_k + z) ),
+// where b_k is the constant that makes a masked nibble an FP16 number with no arithmetic
+// at all: 1024 for even k (nibble in the low bits of the significand of 1024.0) and 64
+// for odd k (four bits higher, in that of 64.0).  Products of two halves are exact in
+// FP32; the biased sum of a 32-k slice stays below 2^17 for activations of unit size,
+// so the cancellation costs about 2^-24 * 2^17 against a slice sum of ~ 2^5.
+// px: eight activations paired like the codes, (x0,x4),(x1,x5),(x2,x6),(x3,x7).
+// ASYM: b += sum_k x_k b_k, a += sum_k x_k over the word (the caller subtracts b + z a).
+// Symmetric (z = 8 for every group): b += sum_k x_k (b_k + 8), a is left alone.
+template <bool ASYM>
+__device__ __forceinline__ void w4_bias_sums(const u4& px, float& b, float& a) {
+  const h2 ke = splat((_Float16)(ASYM ? 1024.0f : 1032.0f)), ko = splat((_Float16)(ASYM ? 64.0f : 72.0f));
+  b = dot2(as_h2(px[0]), ke, b);
+  b = dot2(as_h2(px[1]), ko, b);
+  b = dot2(as_h2(px[2]), ke, b);
+  b = dot2(as_h2(px[3]), ko, b);
+  if (ASYM) {
+    const h2 one = splat((_Float16)1.0f);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) a = dot2(as_h2(px[e]), one, a);
+  }
+}
+// t + sum_k x_k (b_k + n_k) over the word w: a shift, four and-or, four dot products.
+__device__ __forceinline__ float w4_dot_biased(uint32_t w, const u4& px, float t) {
+  uint32_t m_lo = 0x64006400u, m_hi = 0x54005400u;
+  asm("" : "+v"(m_lo), "+v"(m_hi));  // in registers: as literals each and-or becomes two instructions
+  const uint32_t w8 = w >> 8;
+  t = dot2(as_h2(and_or(w, 0x000F000Fu, m_lo)), as_h2(px[0]), t);   // 1024 + (n0, n4)
+  t = dot2(as_h2(and_or(w, 0x00F000F0u, m_hi)), as_h2(px[1]), t);   // 64 + (n1, n5)
+  t = dot2(as_h2(and_or(w8, 0x000F000Fu, m_lo)), as_h2(px[2]), t);  // 1024 + (n2, n6)
+  t = dot2(as_h2(and_or(w8, 0x00F000F0u, m_hi)), as_h2(px[3]), t);  // 64 + (n3, n7)
+  return t;
+}
+__device__ __forceinline__ float half_bits_to_float(uint32_t b16) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)b16);
+}
+
 // Wave64 sum of `v` with DPP adds only (no LDS traffic): quad swaps, row
 // mirrors, then the two row broadcasts.  Lane 63 ends with the total.
 template <int CTRL, int ROWMASK>

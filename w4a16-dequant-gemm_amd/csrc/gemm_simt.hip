@@ -474,16 +474,18 @@ static hipError_t launch_rows4(const WView& v, const w4_half* x, w4_half* c, int
 #define W4_GO(ASYM, GSH)                                                               \
   simt_rows4_kernel<MX, MT, STEPS, ASYM, GSH, false><<<grid, SIMT_WAVES * 64, 0, s>>>( \
       v.q, v.scales, v.zeros, x, c, v.N, M, v.gs, v.G, nullptr)
-#define W4_GSH(ASYM)                                          \
-  switch (gsh) {                                              \
-    case 0: W4_GO(ASYM, 0); break;                            \
-    case 3: W4_GO(ASYM, 3); break;                            \
-    case 5: W4_GO(ASYM, 5); break;                            \
-    case 6: W4_GO(ASYM, 6); break;                            \
-    case 7: W4_GO(ASYM, 7); break;                            \
-    default: W4_GO(ASYM, 8); break;                           \
+  // (a group lookup per packed word with eight activation rows needs more registers than
+  // a lane has: try_rows4 leaves those calls to the kernels below)
+#define W4_GSH(ASYM)                                                          \
+  switch (gsh) {                                                              \
+    case 0: if constexpr (MT <= 4) W4_GO(ASYM, 0); break;                     \
+    case 3: if constexpr (MT <= 4) W4_GO(ASYM, 3); break;                     \
+    case 5: W4_GO(ASYM, 5); break;                                            \
+    case 6: W4_GO(ASYM, 6); break;                                            \
+    case 7: W4_GO(ASYM, 7); break;                                            \
+    default: W4_GO(ASYM, 8); break;                                           \
   }
-  if (MX) W4_GO(false, 5);
+  if constexpr (MX) W4_GO(false, 5);
   else if (v.symmetric) { W4_GSH(false) }
   else { W4_GSH(true) }
 #undef W4_GSH
@@ -497,14 +499,16 @@ static bool try_rows4(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
                       w4_half* w_out, hipError_t* err) {
   if (w_out || v.K % 2048 || v.N % (SIMT_WAVES * ROWS4_R)) return false;
   if (!MX && (v.gs < 8 || v.gs % 8)) return false;
+  const bool one_group_per_slice = MX || ((v.gs & (v.gs - 1)) == 0 && v.gs >= 32 && v.gs <= 256);
+  if (MT > 4 && !one_group_per_slice) return false;
   if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)c & 7) || ((uintptr_t)v.scales & 3))
     return false;
   const int steps = v.K / 2048;
   if (steps * MT > 8) return false;  // LDS: MT * K halves, at most 32 KiB
   switch (steps) {
     case 1: *err = launch_rows4<MX, MT, 1>(v, x, c, M, s); return true;
-    case 2: *err = launch_rows4<MX, MT, 2>(v, x, c, M, s); return true;
-    case 4: if (MT <= 2) { *err = launch_rows4<MX, MT <= 2 ? MT : 1, 4>(v, x, c, M, s); return true; } return false;
+    case 2: if constexpr (MT <= 4) { *err = launch_rows4<MX, MT <= 4 ? MT : 1, 2>(v, x, c, M, s); return true; } return false;
+    case 4: if constexpr (MT <= 2) { *err = launch_rows4<MX, MT <= 2 ? MT : 1, 4>(v, x, c, M, s); return true; } return false;
     default: return false;
   }
 }
@@ -598,6 +602,40 @@ __global__ __launch_bounds__(W * 64) void simt_ksplit_kernel(
         xr[m][j] = MX ? xv[s][m][j] : pair_strided(xv[s][m][j]);
         if (!on[s]) xr[m][j] = u4{0u, 0u, 0u, 0u};
       }
+    if constexpr (!MX && !HOOK) {
+      // no dequantized weight leaves this instantiation: biased codes, the scale and the
+      // zero-point applied once per group in FP32 (w4_dot_biased); the bias sums of the
+      // lane's slice serve all R rows
+      float pb[MT][NS], pa[MT][NS];
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+#pragma unroll
+        for (int e = 0; e < NS; ++e) pb[m][e] = pa[m][e] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w4_bias_sums<ASYM>(xr[m][j], pb[m][NS == 1 ? 0 : j], pa[m][NS == 1 ? 0 : j]);
+      }
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        float t[MT];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int e = NS == 1 ? 0 : j;
+          if (NS == 4 || j == 0) {
+            const float z = (float)((zw[s][r][e] >> zsh[s][e]) & 0xFu);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) t[m] = ASYM ? -__builtin_fmaf(z, pa[m][e], pb[m][e]) : -pb[m][e];
+          }
+#pragma unroll
+          for (int m = 0; m < MT; ++m) t[m] = w4_dot_biased(qw[s][r][j], xr[m][j], t[m]);
+          if (NS == 4 || j == 3) {
+            const float sf = half_bits_to_float(sc[s][r][e]);
+#pragma unroll
+            for (int m = 0; m < MT; ++m) acc[r][m] = __builtin_fmaf(sf, t[m], acc[r][m]);
+          }
+        }
+      }
+      continue;
+    }
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const float mxs = mx_scale(sc[s][r][0]);
@@ -730,8 +768,8 @@ static bool try_unrolled(const WView& v, const w4_half* x, w4_half* c, int M, hi
   if (steps * MT > 8) return false;  // LDS: MT * K halves, at most 32 KiB
   switch (steps) {
     case 1: *err = launch_unrolled<MX, MT, 1>(v, x, c, M, s); return true;
-    case 2: *err = launch_unrolled<MX, MT, 2>(v, x, c, M, s); return true;
-    case 4: if (MT <= 2) { *err = launch_unrolled<MX, MT <= 2 ? MT : 1, 4>(v, x, c, M, s); return true; } return false;
+    case 2: if constexpr (MT <= 4) { *err = launch_unrolled<MX, MT <= 4 ? MT : 1, 2>(v, x, c, M, s); return true; } return false;
+    case 4: if constexpr (MT <= 2) { *err = launch_unrolled<MX, MT <= 2 ? MT : 1, 4>(v, x, c, M, s); return true; } return false;
     default: return false;
   }
 }

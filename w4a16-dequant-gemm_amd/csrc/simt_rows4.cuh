@@ -71,6 +71,17 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_rows4_kernel(
   // gs >= 32 / gs >= 8 (gs_any, G_any groups per row): a group per packed word; the
   // arrays and load counts below are sized for the most groups a row can have.
   constexpr bool ANY = !MX && GSH < 5;
+#ifndef W4_ROWS4_FOLD
+#define W4_ROWS4_FOLD 1
+#endif
+  constexpr bool FOLD = W4_ROWS4_FOLD && !MX;             // W4: scale and zero-point applied per group, in FP32
+  constexpr int PW = ANY ? 4 : 1;                         // bias sums kept per packed word / per 32-k slice
+  // Where the bias sums are formed: by the threads that stage the activations (once per
+  // workgroup, before the barrier), or by every lane from its own registers at the head
+  // of a 2048-k block.  With zero-points (two sums per slice) and one group per slice the
+  // second is faster by 2 - 4 % (N = 11008, gs = 128, M = 1 / 2: 5.46 / 6.48 against
+  // 5.55 / 6.74 us): it adds nothing in front of the barrier.
+  constexpr bool STAGED = FOLD && (ANY || !ASYM);
   constexpr int NG = ANY ? 4 : 1;                         // group lookups per slice
   constexpr int GCAP = MX ? K / 32 : ANY ? (K >> (GSH == 0 ? 5 : 3)) : (K >> GSH);
   const int G = ANY ? G_any : GCAP;                       // groups (blocks) per row
@@ -83,6 +94,8 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_rows4_kernel(
   __shared__ u4 xs[MT * STEPS * 256];
   __shared__ uint32_t ss[SIMT_WAVES][NSL * 64];
   __shared__ uint32_t zs[SIMT_WAVES][ASYM ? NZL * 64 : 1];
+  __shared__ float xb[STAGED ? MT * STEPS * 64 * PW : 1];          // sum of x_k * bias_k (symmetric: bias_k + 8)
+  __shared__ float xa[STAGED && ASYM ? MT * STEPS * 64 * PW : 1];  // sum of x_k
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n0 = (blockIdx.x * SIMT_WAVES + wave) * R;
   const int m0 = blockIdx.y * MT;
@@ -130,7 +143,31 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_rows4_kernel(
     const int i = t * SIMT_WAVES * 64 + threadIdx.x;
     const int m = i / (STEPS * 256), g8 = i % (STEPS * 256);
     const int slot = (g8 & ~255) + (g8 & 3) * 64 + ((g8 & 255) >> 2);
-    xs[m * STEPS * 256 + slot] = MX ? xv[t] : pair_strided(xv[t]);
+    const u4 px = MX ? xv[t] : pair_strided(xv[t]);
+    xs[m * STEPS * 256 + slot] = px;
+    if constexpr (STAGED) {
+      // What the biased codes add to a dot product does not depend on the row: the
+      // thread that stages a word's eight activations sums them against the biases
+      // here, under the latency of the weights (even k: 1024, odd k: 64; with z = 8
+      // for every group the zero-point rides along), and a quad of lanes adds up a slice.
+      float vb = 0.0f, va = 0.0f;
+      w4_bias_sums<ASYM>(px, vb, va);
+      if (ANY) {
+        xb[m * STEPS * 256 + slot] = vb;
+        if (ASYM) xa[m * STEPS * 256 + slot] = va;
+      } else {
+        vb = dpp_add<0xB1, 0xF>(vb);
+        vb = dpp_add<0x4E, 0xF>(vb);
+        if (ASYM) {
+          va = dpp_add<0xB1, 0xF>(va);
+          va = dpp_add<0x4E, 0xF>(va);
+        }
+        if ((threadIdx.x & 3) == 0) {  // g8 & 3 == threadIdx.x & 3: the quad is one lane's slice
+          xb[m * STEPS * 64 + (g8 >> 8) * 64 + ((g8 & 255) >> 2)] = vb;
+          if (ASYM) xa[m * STEPS * 64 + (g8 >> 8) * 64 + ((g8 & 255) >> 2)] = va;
+        }
+      }
+    }
   }
   vm_wait<NQ>();  // scales and zero-points: into this wave's own LDS region
 #pragma unroll
@@ -148,6 +185,7 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_rows4_kernel(
   // group parameters of this lane's slices, read back from LDS
   uint32_t sc[NQ][NG];
   int zp[NQ][NG];
+  float sf[FOLD ? NQ : 1][NG], zf[FOLD && ASYM ? NQ : 1][NG];
 #pragma unroll
   for (int i = 0; i < NQ; ++i) {
     const int st = i / R, r = i % R;
@@ -160,6 +198,10 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_rows4_kernel(
       if (MX) sc[i][j] = ((const uint8_t*)ss[wave])[r * G + g];
       else sc[i][j] = ((const uint16_t*)ss[wave])[r * G + g];
       zp[i][j] = ASYM ? (int)((zs[wave][r * WG + (g >> 3)] >> (4 * (g & 7))) & 0xFu) : 8;
+      if constexpr (FOLD) {
+        sf[i][j] = half_bits_to_float(sc[i][j]);
+        if constexpr (ASYM) zf[i][j] = (float)zp[i][j];
+      }
     }
   }
 
@@ -173,6 +215,7 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_rows4_kernel(
   // step i expands the 1 KiB run (2048-k block i / R, row i % R); the runs were
   // requested in this order, so run i has landed when at most NQ - 1 - i are outstanding
   u4 xr[MT][4];
+  float pb[MT][PW], pa[MT][PW];  // FOLD: this lane's bias sums of the current block
   auto step = [&](auto ic) {
     constexpr int i = decltype(ic)::value;
     constexpr int st = i / R, r = i % R;
@@ -186,6 +229,46 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_rows4_kernel(
     vm_wait<(NQ - 1 - i > 0 ? NQ - 1 - i : 0)>();
     landed(qw[i]);
     if (TL) ts[4 + i] = rows4_now();
+    if constexpr (FOLD) {
+      // Nothing of this kernel's result is a dequantized weight (a call with the w_out
+      // hook never comes here): biased codes, scale and zero-point applied per group in
+      // FP32 (w4_dot_biased): 5 + 4 MT instead of 13 + 4 MT vector instructions per word.
+      if (r == 0 && STAGED) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+          for (int j = 0; j < PW; ++j) {
+            const int at = ANY ? m * STEPS * 256 + st * 256 + j * 64 + lane : m * STEPS * 64 + st * 64 + lane;
+            pb[m][j] = xb[at];
+            if (ASYM) pa[m][j] = xa[at];
+          }
+      }
+      if (r == 0 && !STAGED) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          pb[m][0] = pa[m][0] = 0.0f;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) w4_bias_sums<ASYM>(xr[m][j], pb[m][0], pa[m][0]);
+        }
+      }
+      float t[MT];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int jg = ANY ? j : 0;
+        if (ANY || j == 0) {
+#pragma unroll
+          for (int m = 0; m < MT; ++m)
+            t[m] = ASYM ? -__builtin_fmaf(zf[ASYM ? i : 0][jg], pa[m][jg], pb[m][jg]) : -pb[m][jg];
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m) t[m] = w4_dot_biased(qw[i][j], xr[m][j], t[m]);
+        if (ANY || j == 3) {
+#pragma unroll
+          for (int m = 0; m < MT; ++m) acc[r][m] = __builtin_fmaf(sf[i][jg], t[m], acc[r][m]);
+        }
+      }
+      return;
+    }
     const float mxs = mx_scale(sc[i][0]);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {

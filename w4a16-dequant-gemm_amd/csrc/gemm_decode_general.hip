@@ -23,6 +23,8 @@
 //    the end of its row is read word by word with the index clamped to the row.
 //  * the last chunk of a row may be partial: its activations beyond K are fetched
 //    from a clamped address and zeroed on the way to the MFMA operands.
+#include <atomic>
+
 #include "dq.cuh"
 #include "kernels.h"
 
@@ -356,29 +358,44 @@ __global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
 }
 
 struct GeneralPlan {
-  int ch, t, cpx, lds;
+  int ch, t, mt, cpx, lds;
 };
+
+// Most tiles per workgroup that an instantiation holds in registers without spilling
+// (checked against the compiler's register counts).
+constexpr int dg_tile_cap(int ch, int mt) { return (mt == 4 && ch == 5) ? 3 : 4; }
+// What general_plan() can return: everything else is never compiled.
+constexpr bool dg_planned(int ch, int t, int mt, int cpx) {
+  if (t > dg_tile_cap(ch, mt)) return false;
+  if (cpx == 2) return mt == 1 && ch > 2;
+  if (cpx == 1) return mt == 2;
+  return cpx == 0;
+}
 
 // LDS the device grants a workgroup (per-device cache); 0 on error.
 int max_lds_bytes() {
-  static int cached[64] = {};
+  static std::atomic<int> cached[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
-  if (dev >= 0 && dev < 64 && cached[dev]) return cached[dev];
+  if (dev >= 0 && dev < 64) {
+    if (const int have = cached[dev].load(std::memory_order_relaxed)) return have;
+  }
   int n = 0;
   if (hipDeviceGetAttribute(&n, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) return 0;
-  if (dev >= 0 && dev < 64) cached[dev] = n;
+  if (dev >= 0 && dev < 64) cached[dev].store(n, std::memory_order_relaxed);
   return n;
 }
 
 int cu_count() {
-  static int cached[64] = {};
+  static std::atomic<int> cached[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
-  if (dev >= 0 && dev < 64 && cached[dev]) return cached[dev];
+  if (dev >= 0 && dev < 64) {
+    if (const int have = cached[dev].load(std::memory_order_relaxed)) return have;
+  }
   int n = 0;
   if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-  if (dev >= 0 && dev < 64) cached[dev] = n;
+  if (dev >= 0 && dev < 64) cached[dev].store(n, std::memory_order_relaxed);
   return n;
 }
 
@@ -402,9 +419,7 @@ bool general_plan(const WView& v, const w4_half* x, const w4_half* c, int M, Gen
   // four; with one activation row tile the x regions may shrink to two chunks per
   // phase to make room for the parameter blocks
   int want = (v.N / 16 + cus - 1) / cus;
-  if (want > 4) want = 4;
-  // (four tiles, four activation row tiles and five chunks per wave spill 12 - 28 VGPRs)
-  if (mt == 4 && ch == 5 && want > 3) want = 3;
+  if (want > dg_tile_cap(ch, mt)) want = dg_tile_cap(ch, mt);
   auto fit = [&](int cpd, int* lds) {
     const int cp = cpd < ch ? cpd : ch;
     const int xbytes = DG_WAVES * mt * cp * 4096;
@@ -423,32 +438,46 @@ bool general_plan(const WView& v, const w4_half* x, const w4_half* c, int M, Gen
     const int t2 = fit(2, &lds2);
     if (t2 >= t) t = t2, lds = lds2, cpx = 2;
   }
+  if (mt == 2 && t < want) {
+    // Large parameter blocks (gs = 8 at K = 4104: 20.6 KB per tile) leave room for fewer
+    // tiles than the grid wants once the activations of 32 rows hold 128 KB.  With one
+    // chunk per phase they hold 64 KB and a workgroup shares them between `want` tiles
+    // again: N = 11008, K = 4104 / 4096, gs = 8, M = 32: 31.4 / 25.4 -> 20.9 / 16.2 us.
+    // (64 rows as two such passes in grid.y measured no gain: 344 workgroups of 146 KB
+    // are two rounds, 39.9 against 38.7 us.)
+    int lds1 = 0;
+    const int t1 = fit(1, &lds1);
+    if (t1 > t) t = t1, lds = lds1, cpx = 1;
+  }
   if (t < 1) return false;
-  *out = GeneralPlan{ch, t, cpx, lds};
+  *out = GeneralPlan{ch, t, mt, cpx, lds};
   return true;
 }
 
 template <bool ASYM, int CH, int T, int MT, int CPX, int GM>
 hipError_t general_gm(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                       const GeneralPlan& pl) {
-  // more than 64 KB of LDS has to be granted per device, once per instantiation
-  static bool granted[64] = {};
-  static int granted_bytes[64] = {};
-  int dev = 0;
-  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
-  if (dev < 0 || dev >= 64 || !granted[dev] || granted_bytes[dev] < pl.lds) {
-    const hipError_t e =
-        hipFuncSetAttribute((const void*)mfma_decode_general_kernel<ASYM, CH, T, MT, CPX, GM>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, pl.lds);
-    if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64) granted[dev] = true, granted_bytes[dev] = pl.lds;
+  if constexpr (!dg_planned(CH, T, MT, CPX)) {
+    return hipErrorInvalidValue;  // general_plan() never asks for it
+  } else {
+    // more than 64 KB of LDS has to be granted per device, once per instantiation
+    static std::atomic<int> granted_bytes[64] = {};
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+    if (dev < 0 || dev >= 64 || granted_bytes[dev].load(std::memory_order_acquire) < pl.lds) {
+      const hipError_t e =
+          hipFuncSetAttribute((const void*)mfma_decode_general_kernel<ASYM, CH, T, MT, CPX, GM>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, pl.lds);
+      if (e != hipSuccess) return e;
+      if (dev >= 0 && dev < 64) granted_bytes[dev].store(pl.lds, std::memory_order_release);
+    }
+    const int tiles = v.N / 16;
+    const int sh = (v.gs & (v.gs - 1)) == 0 ? __builtin_ctz((unsigned)v.gs) : -1;
+    const dim3 grid((unsigned)((tiles + T - 1) / T), (unsigned)((M + 16 * MT - 1) / (16 * MT)));
+    mfma_decode_general_kernel<ASYM, CH, T, MT, CPX, GM><<<grid, DG_THREADS, pl.lds, s>>>(
+        v.q, (const w4_half*)v.scales, v.zeros, x, c, v.N, v.K, v.gs, sh, v.G, M, tiles);
+    return hipGetLastError();
   }
-  const int tiles = v.N / 16;
-  const int sh = (v.gs & (v.gs - 1)) == 0 ? __builtin_ctz((unsigned)v.gs) : -1;
-  const dim3 grid((unsigned)((tiles + T - 1) / T), (unsigned)((M + 16 * MT - 1) / (16 * MT)));
-  mfma_decode_general_kernel<ASYM, CH, T, MT, CPX, GM><<<grid, DG_THREADS, pl.lds, s>>>(
-      v.q, (const w4_half*)v.scales, v.zeros, x, c, v.N, v.K, v.gs, sh, v.G, M, tiles);
-  return hipGetLastError();
 }
 
 template <bool ASYM, int CH, int T, int MT, int CPX>
@@ -464,13 +493,16 @@ hipError_t general_go(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
 template <bool ASYM, int CH, int T>
 hipError_t general_mt(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                       const GeneralPlan& pl) {
-  if (M <= 16) {
+  if (pl.mt == 1) {
     if constexpr (CH > 2) {
       if (pl.cpx == 2) return general_go<ASYM, CH, T, 1, 2>(v, x, c, M, s, pl);
     }
     return general_go<ASYM, CH, T, 1, 0>(v, x, c, M, s, pl);
   }
-  if (M <= 32) return general_go<ASYM, CH, T, 2, 0>(v, x, c, M, s, pl);
+  if (pl.mt == 2) {
+    if (pl.cpx == 1) return general_go<ASYM, CH, T, 2, 1>(v, x, c, M, s, pl);
+    return general_go<ASYM, CH, T, 2, 0>(v, x, c, M, s, pl);
+  }
   return general_go<ASYM, CH, T, 4, 0>(v, x, c, M, s, pl);
 }
 

@@ -501,7 +501,7 @@ def extras_gemm(b, full):
                          "simt_reps_us": raw_s, "mfma_reps_us": raw_m,
                          "best_GBs": nb / best * 1e-3, "frac_of_hbm_peak": nb / best * 1e-3 / HBM_PEAK_GBS,
                          "winner": "simt" if us_s is not None and us_s <= us_m else "mfma",
-                         "dispatcher": "simt" if M < capi.load().w4_dispatch_mma_min_m_for(N, K) else "mfma"})
+                         "dispatcher": "simt" if M < capi.load().w4_dispatch_mma_min_m_for_gs(N, K, gs) else "mfma"})
         gates.append({"N": N, "K": K, "gs": gs, "quant_rel_l2": qerr, "cases": gate.results})
         del dps, views, gate, w_ref, p
         torch.cuda.empty_cache()

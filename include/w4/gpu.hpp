@@ -106,6 +106,7 @@ inline w4_kv_f8_view abi(const DeviceKVF8& p) {
 // the matrix-core kernel, as measured on MI355X.
 inline int dispatch_mma_min_m() { return w4_dispatch_mma_min_m(); }
 inline int dispatch_mma_min_m(int N, int K) { return w4_dispatch_mma_min_m_for(N, K); }
+inline int dispatch_mma_min_m(int N, int K, int gs) { return w4_dispatch_mma_min_m_for_gs(N, K, gs); }
 inline int dispatch_mma_min_m_mx(int N, int K) { return w4_dispatch_mma_min_m_for_mx(N, K); }
 
 // dequant.cuh:62-82

@@ -91,6 +91,11 @@ int w4_dispatch_mma_min_m(void);
  * w4_dispatch_mma_min_m().  No counterpart in the reference, whose crossover is one
  * constant (dispatch.cuh:25). */
 int w4_dispatch_mma_min_m_for(int N, int K);
+/* What w4_gemm uses: the same with the group size taken into account (a group size that is
+ * no multiple of 32 keeps w4_dispatch_mma_min_m() on wide matrices at K <= 4096: its
+ * matrix-core kernel looks group parameters up per packed word and is behind the vector
+ * kernel through M = 4; gs <= 0 means "a multiple of 32").  No counterpart in the reference. */
+int w4_dispatch_mma_min_m_for_gs(int N, int K, int gs);
 /* The same for an MXFP4 matrix (what w4_gemm_mx uses): as above, and 2 for K above 4096 other
  * than 8192 (N = 4096, K = 14336, M = 2: 9.8 us against 11.5).  No counterpart in the reference. */
 int w4_dispatch_mma_min_m_for_mx(int N, int K);

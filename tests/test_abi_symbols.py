@@ -47,6 +47,10 @@ def test_validation_runs_without_a_device():
     assert lib.w4_dispatch_mma_min_m_for(4096, 6144) == 2
     assert lib.w4_dispatch_mma_min_m_for(11008, 4096) == 3
     assert lib.w4_dispatch_mma_min_m_for(8192, 4096) == lib.w4_dispatch_mma_min_m()
+    assert lib.w4_dispatch_mma_min_m_for_gs(11008, 4096, 128) == 3
+    assert lib.w4_dispatch_mma_min_m_for_gs(11008, 4096, 32) == 3
+    assert lib.w4_dispatch_mma_min_m_for_gs(11008, 4096, 48) == lib.w4_dispatch_mma_min_m()
+    assert lib.w4_dispatch_mma_min_m_for_gs(11008, 4104, 8) == 2
     assert lib.w4_dispatch_mma_min_m_for_mx(4096, 14336) == 2
     assert lib.w4_dispatch_mma_min_m_for_mx(4096, 8192) == 3
     assert lib.w4_dispatch_mma_min_m_for_mx(4096, 4096) == lib.w4_dispatch_mma_min_m()

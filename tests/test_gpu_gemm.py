@@ -157,7 +157,7 @@ def test_w4_gemm_gates(i, sym):
     cross_gate(cm, cm2, ref, "gemm_mma")
     # dispatcher: same bytes as the callee it selects at the same hook flag, hook intact
     cd, wd = _run(c.gemm, dp.view, x_d, M, N, K)
-    use_mma = M >= c.load().w4_dispatch_mma_min_m_for(N, K)
+    use_mma = M >= c.load().w4_dispatch_mma_min_m_for_gs(N, K, gs)
     assert np.array_equal(cd, cm if use_mma else cf) and np.array_equal(wd, w_ref)
     cd2, _ = _run(c.gemm, dp.view, x_d, M, N, K, hook=False)
     assert np.array_equal(cd2, cm2 if use_mma else cf2)

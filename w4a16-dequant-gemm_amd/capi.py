@@ -43,6 +43,7 @@ SIGNATURES = {
     "w4_last_error": ([], C.c_char_p),
     "w4_dispatch_mma_min_m": ([], C.c_int),
     "w4_dispatch_mma_min_m_for": ([C.c_int, C.c_int], C.c_int),
+    "w4_dispatch_mma_min_m_for_gs": ([C.c_int, C.c_int, C.c_int], C.c_int),
     "w4_dispatch_mma_min_m_for_mx": ([C.c_int, C.c_int], C.c_int),
     "w4_dequant": ([C.POINTER(PackedView), vp, vp], C.c_int),
     "w4_gemm_fused": ([C.POINTER(PackedView), vp, vp, C.c_int, vp, vp], C.c_int),

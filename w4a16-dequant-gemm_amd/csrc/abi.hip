@@ -10,6 +10,7 @@
 #include <limits.h>
 #include <stdio.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "kernels.h"
@@ -78,31 +79,37 @@ int check_mx(const w4_packed_mx_view* p) {
 
 // Grow-only device scratch for the split-S partials, one per device, shared by all
 // calls on that device (calls on different streams must not overlap, as with the
-// reference's kv_part_scratch, kvflash.cuh:56-69).
+// reference's kv_part_scratch, kvflash.cuh:56-69).  A call that finds the buffer large
+// enough takes no lock.  When it has to grow, the new buffer is at least twice the old
+// one and the old one is kept until the process ends (a call still in flight may be
+// using it, and freeing it would mean draining the device under the lock): what the
+// library ever holds per device stays below twice the largest request.
 constexpr int MAX_DEVICES = 64;
 std::mutex g_scratch_mu;
-float* g_scratch[MAX_DEVICES] = {};
-size_t g_scratch_cap[MAX_DEVICES] = {};
+std::atomic<float*> g_scratch[MAX_DEVICES] = {};
+std::atomic<size_t> g_scratch_cap[MAX_DEVICES] = {};
 
 hipError_t scratch_floats(size_t n, float** out) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   if (dev < 0 || dev >= MAX_DEVICES) return hipErrorInvalidDevice;
-  std::lock_guard<std::mutex> lk(g_scratch_mu);
-  if (n > g_scratch_cap[dev]) {
-    float* nb = nullptr;
-    e = hipMalloc((void**)&nb, n * sizeof(float));
-    if (e != hipSuccess) return e;
-    // a call still in flight may be using the old buffer: let the device drain first
-    if (g_scratch[dev]) {
-      (void)hipDeviceSynchronize();
-      (void)hipFree(g_scratch[dev]);
-    }
-    g_scratch[dev] = nb;
-    g_scratch_cap[dev] = n;
+  if (n <= g_scratch_cap[dev].load(std::memory_order_acquire)) {
+    // (the pointer published with this capacity, or a larger buffer published since)
+    *out = g_scratch[dev].load(std::memory_order_acquire);
+    return hipSuccess;
   }
-  *out = g_scratch[dev];
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  const size_t have = g_scratch_cap[dev].load(std::memory_order_relaxed);
+  if (n > have) {
+    const size_t want = n > 2 * have ? n : 2 * have;
+    float* nb = nullptr;
+    e = hipMalloc((void**)&nb, want * sizeof(float));
+    if (e != hipSuccess) return e;
+    g_scratch[dev].store(nb, std::memory_order_release);
+    g_scratch_cap[dev].store(want, std::memory_order_release);
+  }
+  *out = g_scratch[dev].load(std::memory_order_relaxed);
   return hipSuccess;
 }
 
@@ -134,23 +141,27 @@ __device__ __align__(256) float scratch[NOALLOC_SCRATCH_FLOATS];
 
 constexpr int NOALLOC_MAX_DEVICES = MAX_DEVICES;
 std::mutex g_noalloc_mu;
-float* g_noalloc_ptr[NOALLOC_MAX_DEVICES] = {};
+std::atomic<float*> g_noalloc_ptr[NOALLOC_MAX_DEVICES] = {};
 
-// Device address of `scratch` on the current device (looked up on first use).
+// Device address of `scratch` on the current device (looked up on first use; later
+// calls take no lock).
 hipError_t noalloc_scratch(float** out) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return hipErrorInvalidDevice;
-  std::lock_guard<std::mutex> lk(g_noalloc_mu);
-  if (!g_noalloc_ptr[dev]) {
-    float* ptr = nullptr;
-    e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
-    if (e != hipSuccess) return e;
-    if (!ptr) return hipErrorInvalidSymbol;
-    g_noalloc_ptr[dev] = ptr;
+  float* have = g_noalloc_ptr[dev].load(std::memory_order_acquire);
+  if (!have) {
+    std::lock_guard<std::mutex> lk(g_noalloc_mu);
+    have = g_noalloc_ptr[dev].load(std::memory_order_relaxed);
+    if (!have) {
+      e = hipGetSymbolAddress((void**)&have, HIP_SYMBOL(scratch));
+      if (e != hipSuccess) return e;
+      if (!have) return hipErrorInvalidSymbol;
+      g_noalloc_ptr[dev].store(have, std::memory_order_release);
+    }
   }
-  *out = g_noalloc_ptr[dev];
+  *out = have;
   return hipSuccess;
 }
 
@@ -168,17 +179,20 @@ extern "C" {
 const char* w4_last_error(void) { return g_msg; }
 
 int w4_dispatch_mma_min_m(void) { return DISPATCH_MMA_MIN_M; }
-int w4_dispatch_mma_min_m_for(int N, int K) {
+int w4_dispatch_mma_min_m_for_gs(int N, int K, int gs) {
   if (K % 32 != 0 && K % 8 == 0 && (long long)N * K >= (1LL << 25)) return 2;
-  if (K > 4096 && K <= 6144 && K % 128 == 0) return 2;  // 5.6 - 5.9 us against 6.3 at N = 4096
+  if (K > 4096 && K <= 6144 && K % 128 == 0) return 2;  // 5.8 us against 6.3 at N = 4096, M = 2
   if (K > 4096 && K % 32 == 0) return 3;
   // wide matrices at K <= 4096: from about 45 M weights the resident-activation kernel is
-  // ahead at M = 3 and 4 (N = 11008 / 14336, K = 4096, gs = 128: 8.6 / 9.6 us against
-  // 9.4 - 9.8 / 11.7 - 11.8; MXFP4 N = 14336: 8.8 against 9.8 - 10.3; gs = 32 is the exception,
-  // 10.5 against 9.2 - 9.6); N = 8192 still belongs to the vector kernel (6.8 - 7.0 against 7.4)
-  if (K % 32 == 0 && (long long)N * K >= 44000000LL) return 3;
+  // ahead at M = 3 and 4 (N = 11008 / 14336, K = 4096, gs = 128 or 32: 8.6 - 8.9 / 9.5 - 9.8 us
+  // against 9.5 - 9.8 / 11.2 - 11.5); N = 8192 still belongs to the vector kernel (6.8 - 6.9
+  // against 7.6).  Group sizes that are no multiple of 32 go to the matrix cores' general
+  // kernel, which is slower there (N = 11008, gs = 48, M = 4: 11.8 us against 11.3 on the
+  // vector units): they keep the plain threshold.
+  if (K % 32 == 0 && (gs <= 0 || gs % 32 == 0) && (long long)N * K >= 44000000LL) return 3;
   return DISPATCH_MMA_MIN_M;
 }
+int w4_dispatch_mma_min_m_for(int N, int K) { return w4_dispatch_mma_min_m_for_gs(N, K, 0); }
 
 int w4_dispatch_mma_min_m_for_mx(int N, int K) {
   // two activation rows at long K other than 8192 (which has the four-rows vector kernel):
@@ -219,7 +233,7 @@ int w4_gemm_mma(const w4_packed_view* p, const w4_half* x, w4_half* c, int M,
 
 int w4_gemm(const w4_packed_view* p, const w4_half* x, w4_half* c, int M, w4_stream stream,
             w4_half* w_out) {
-  const int min_m = p ? w4_dispatch_mma_min_m_for(p->N, p->K) : DISPATCH_MMA_MIN_M;
+  const int min_m = p ? w4_dispatch_mma_min_m_for_gs(p->N, p->K, p->gs) : DISPATCH_MMA_MIN_M;
   return M < min_m ? w4_gemm_fused(p, x, c, M, stream, w_out)
                    : w4_gemm_mma(p, x, c, M, stream, w_out);
 }

@@ -2,9 +2,10 @@
 // second pass of the two-pass baseline the fused kernels are measured against.
 // c[M,N] (row-major) = x[M,K] * w[N,K]^T, FP32 accumulation, FP16 output.
 //
-// The handle, its workspace and one plan per (M, N, K) -- descriptors plus the
-// algorithm the heuristic picks -- are made once and kept, so a timed call is the
-// matrix product alone, like a call of the fused entry points.
+// Per device: the handle, its workspace and one plan per (M, N, K) -- descriptors plus
+// the algorithm the heuristic picks -- are made once and kept (at most MAX_PLANS of
+// them; the least recently made goes first), so a timed call is the matrix product
+// alone, like a call of the fused entry points.
 #include <hip/hip_runtime.h>
 #include <hipblaslt/hipblaslt.h>
 #include <stdio.h>
@@ -18,16 +19,26 @@
 namespace {
 thread_local char g_blas_msg[160] = "";
 std::mutex g_mu;
-hipblasLtHandle_t g_handle = nullptr;
-void* g_ws = nullptr;
 constexpr size_t WS_BYTES = 64u << 20;
+constexpr int MAX_DEVICES = 64;
+constexpr size_t MAX_PLANS = 64;
 
 struct Plan {
   hipblasLtMatmulDesc_t desc = nullptr;
   hipblasLtMatrixLayout_t la = nullptr, lb = nullptr, lc = nullptr;
   hipblasLtMatmulAlgo_t algo;
 };
-std::map<std::tuple<int, int, int>, Plan> g_plans;
+struct PlanEntry {
+  Plan plan;
+  unsigned long long made = 0;  // creation order: the oldest is dropped when the map is full
+};
+struct DeviceState {
+  hipblasLtHandle_t handle = nullptr;
+  void* ws = nullptr;
+  std::map<std::tuple<int, int, int>, PlanEntry> plans;
+  unsigned long long clock = 0;
+};
+DeviceState g_dev[MAX_DEVICES];
 
 void destroy(Plan& p) {
   if (p.la) hipblasLtMatrixLayoutDestroy(p.la);
@@ -42,9 +53,9 @@ int fail(const char* what, int status) {
   return W4_ERUNTIME;
 }
 
-// Handle and workspace: the handle is published only once both exist.
-int ensure_handle() {
-  if (g_handle) return W4_OK;
+// Handle and workspace of one device: the handle is published only once both exist.
+int ensure_handle(DeviceState& d) {
+  if (d.handle) return W4_OK;
   void* ws = nullptr;
   if (hipMalloc(&ws, WS_BYTES) != hipSuccess) {
     snprintf(g_blas_msg, sizeof g_blas_msg, "gemm_fp16: workspace allocation failed");
@@ -56,13 +67,13 @@ int ensure_handle() {
     (void)hipFree(ws);
     return fail("hipblasLtCreate", (int)st);
   }
-  g_ws = ws;
-  g_handle = h;
+  d.ws = ws;
+  d.handle = h;
   return W4_OK;
 }
 
 // Column-major view: C^T (N x M) = W (as K x N col-major, transposed) * X^T (K x M).
-int make_plan(int M, int N, int K, Plan& p) {
+int make_plan(hipblasLtHandle_t handle, int M, int N, int K, Plan& p) {
 #define BL(call)                                             \
   do {                                                       \
     const hipblasStatus_t st_ = (call);                      \
@@ -86,13 +97,19 @@ int make_plan(int M, int N, int K, Plan& p) {
                                            sizeof ws));
   hipblasLtMatmulHeuristicResult_t heur[1];
   int found = 0;
-  BL(hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.la, p.lb, p.lc, p.lc, pref, 1, heur,
+  BL(hipblasLtMatmulAlgoGetHeuristic(handle, p.desc, p.la, p.lb, p.lc, p.lc, pref, 1, heur,
                                      &found));
   hipblasLtMatmulPreferenceDestroy(pref);
   pref = nullptr;
   if (found < 1) {
     destroy(p);
     snprintf(g_blas_msg, sizeof g_blas_msg, "gemm_fp16: no hipBLASLt algorithm");
+    return W4_ERUNTIME;
+  }
+  if (heur[0].workspaceSize > WS_BYTES) {  // the preference above caps it; never trust silently
+    destroy(p);
+    snprintf(g_blas_msg, sizeof g_blas_msg, "gemm_fp16: algorithm wants %zu workspace bytes, have %zu",
+             (size_t)heur[0].workspaceSize, WS_BYTES);
     return W4_ERUNTIME;
   }
   p.algo = heur[0].algo;
@@ -105,20 +122,34 @@ extern "C" const char* w4_blas_last_error(void) { return g_blas_msg; }
 
 extern "C" int w4_gemm_fp16_impl(const w4_half* w, const w4_half* x, w4_half* c, int M, int N,
                                  int K, w4_stream stream) {
-  std::lock_guard<std::mutex> lk(g_mu);
-  if (int rc = ensure_handle()) return rc;
-  const auto key = std::make_tuple(M, N, K);
-  auto it = g_plans.find(key);
-  if (it == g_plans.end()) {
-    Plan p;
-    if (int rc = make_plan(M, N, K, p)) return rc;
-    it = g_plans.emplace(key, p).first;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    snprintf(g_blas_msg, sizeof g_blas_msg, "gemm_fp16: no current device");
+    return W4_ERUNTIME;
   }
-  const Plan& p = it->second;
+  std::lock_guard<std::mutex> lk(g_mu);
+  DeviceState& d = g_dev[dev];
+  if (int rc = ensure_handle(d)) return rc;
+  const auto key = std::make_tuple(M, N, K);
+  auto it = d.plans.find(key);
+  if (it == d.plans.end()) {
+    if (d.plans.size() >= MAX_PLANS) {
+      auto oldest = d.plans.begin();
+      for (auto j = d.plans.begin(); j != d.plans.end(); ++j)
+        if (j->second.made < oldest->second.made) oldest = j;
+      destroy(oldest->second.plan);
+      d.plans.erase(oldest);
+    }
+    PlanEntry e;
+    if (int rc = make_plan(d.handle, M, N, K, e.plan)) return rc;
+    e.made = ++d.clock;
+    it = d.plans.emplace(key, e).first;
+  }
+  const Plan& p = it->second.plan;
   const float alpha = 1.0f, beta = 0.0f;
   const hipblasStatus_t st =
-      hipblasLtMatmul(g_handle, p.desc, &alpha, w, p.la, x, p.lb, &beta, c, p.lc, c, p.lc, &p.algo,
-                      g_ws, WS_BYTES, (hipStream_t)stream);
+      hipblasLtMatmul(d.handle, p.desc, &alpha, w, p.la, x, p.lb, &beta, c, p.lc, c, p.lc, &p.algo,
+                      d.ws, WS_BYTES, (hipStream_t)stream);
   if (st != HIPBLAS_STATUS_SUCCESS) return fail("hipblasLtMatmul", (int)st);
   return W4_OK;
 }

@@ -26,6 +26,8 @@
 // The memory path serves a compute unit's requests in order, so looking further
 // ahead with the codes than with the activations gains nothing: what matters is that
 // a wave multiplies chunk i while chunks i + 1 .. i + 4 are on their way.
+#include <atomic>
+
 #include <type_traits>
 #include <utility>
 
@@ -343,7 +345,7 @@ int longk_chunks(int K) {
 
 // Compute units of the current device (per-device cache); 0 on error.
 int lk_cus() {
-  static int cached[64] = {};
+  static std::atomic<int> cached[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
   if (dev >= 0 && dev < 64 && cached[dev]) return cached[dev];
@@ -356,7 +358,7 @@ int lk_cus() {
 template <int FMT, int CH, int MT, int NQ>
 hipError_t longk_go(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s) {
   constexpr int lds_bytes = LK_WAVES * lk_nbuf(MT, NQ) * NQ * 1024;
-  static bool granted[64] = {};  // more than 64 KB of LDS has to be granted per device, once
+  static std::atomic<bool> granted[64] = {};  // more than 64 KB of LDS has to be granted per device, once
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
   if (lds_bytes > 65536 && (dev < 0 || dev >= 64 || !granted[dev])) {

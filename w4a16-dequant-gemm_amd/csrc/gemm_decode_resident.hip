@@ -21,6 +21,8 @@
 //   * a word is expanded in natural k order (see gemm_tile_dma.hip) straight into
 //     the A operand of v_mfma_f32_16x16x32_f16.
 // Partial sums of the eight waves meet in LDS in wave order (no atomics).
+#include <atomic>
+
 #include "dq.cuh"
 #include "kernels.h"
 
@@ -403,6 +405,15 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
   }
 }
 
+// How the scales are fetched: 1, 2, 3 for gs = 128, 64, 32 at K = 2048 / 4096 with arrays
+// aligned for the vector loads of the scales (and of two zero-point words), else 0.
+int resident_gsv(const WView& v) {
+  if (!v.mx && (v.K == 2048 || v.K == 4096) && ((uintptr_t)v.scales & 15) == 0 &&
+      (v.symmetric || ((uintptr_t)v.zeros & 7) == 0))
+    return v.gs == 128 ? 1 : v.gs == 64 ? 2 : v.gs == 32 ? 3 : 0;
+  return 0;
+}
+
 // Chunks of 128 k per wave for the K this kernel is built for, else 0: K = 2048 and
 // 4096 exactly, and any multiple of 128 whose eighth rounds up to 8, 11 or 14 chunks
 // (7296 .. 8192, 10368 .. 11264, 13440 .. 14336: the long sides of the usual MLP shapes).
@@ -416,14 +427,14 @@ int resident_chunks(int K) {
 
 int device_cus();
 
-template <int FMT, int CH, bool POW2, int GSV, int T, int MT, int CPV = 0>
-hipError_t launch_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
-                    int tiles, unsigned grid) {
+template <int FMT, int CH, bool POW2, int GSV, int T, int MT, int CPV>
+hipError_t launch_t_impl(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
+                         int tiles, unsigned grid) {
   constexpr int CP = CPV ? CPV : (4 / MT) < CH ? (4 / MT) : CH;
   constexpr int lds_bytes = DR_WAVES * MT * CP * 4096;
   static_assert(DR_WAVES * T * MT * 1024 <= lds_bytes, "the reduction reuses the x regions");
   // more than 64 KB of LDS has to be granted per device, once
-  static bool granted[64] = {};
+  static std::atomic<bool> granted[64] = {};
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
   if (dev < 0 || dev >= 64 || !granted[dev]) {
@@ -437,6 +448,25 @@ hipError_t launch_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStre
       <<<dim3(grid, (unsigned)((M + 16 * MT - 1) / (16 * MT))), DR_THREADS, lds_bytes, s>>>(v, x, c, M, sh,
                                                                                           tiles);
   return hipGetLastError();
+}
+
+// Most tiles per workgroup that an instantiation holds in registers without spilling
+// (from the compiler's register counts): with zero-points, four activation row tiles
+// take three tiles; two row tiles with per-chunk scale loads (GSV == 0) take seven.
+constexpr int dr_tile_cap(int fmt, int gsv, int mt) {
+  if (fmt == 1 && mt == 4) return 3;
+  if (fmt == 1 && mt == 2 && gsv == 0) return 7;
+  return 8;
+}
+
+template <int FMT, int CH, bool POW2, int GSV, int T, int MT, int CPV = 0>
+hipError_t launch_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
+                    int tiles, unsigned grid) {
+  if constexpr (T > dr_tile_cap(FMT, GSV, MT)) {
+    return hipErrorInvalidValue;  // decode_resident_tiles() never asks for it
+  } else {
+    return launch_t_impl<FMT, CH, POW2, GSV, T, MT, CPV>(v, x, c, M, s, sh, tiles, grid);
+  }
 }
 
 template <int FMT, int CH, bool POW2, int GSV, int T>
@@ -490,11 +520,7 @@ hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
                       int tiles, int T) {
   const bool pow2 = !v.mx && (v.gs & (v.gs - 1)) == 0;
   const int sh = pow2 ? __builtin_ctz((unsigned)v.gs) : 0;
-  // the vector loads of the scales (and of two zero-point words) need aligned arrays
-  int gsv = 0;
-  if (!v.mx && (v.K == 2048 || v.K == 4096) && ((uintptr_t)v.scales & 15) == 0 &&
-      (v.symmetric || ((uintptr_t)v.zeros & 7) == 0))
-    gsv = v.gs == 128 ? 1 : v.gs == 64 ? 2 : v.gs == 32 ? 3 : 0;
+  const int gsv = resident_gsv(v);
 #define W4_GO(CHV)                                                                          \
   switch (gsv) {                                                                            \
     case 1: return launch_ch<FMT, CHV, true, 1>(v, x, c, M, s, sh, tiles, T);               \
@@ -507,13 +533,24 @@ hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
 #define W4_LONG(CHV)                                                                        \
   return pow2 ? launch_ch<FMT, CHV, true, 0>(v, x, c, M, s, sh, tiles, T)                   \
               : launch_ch<FMT, CHV, false, 0>(v, x, c, M, s, sh, tiles, T);
-  switch (resident_chunks(v.K)) {
-    case 2: W4_GO(2)
-    case 4: W4_GO(4)
-    case 8: W4_LONG(8)
-    case 11: W4_LONG(11)
-    case 14: W4_LONG(14)
-    default: return hipErrorInvalidValue;
+  if constexpr (FMT == 2) {  // MXFP4 has one form per K: no group size, no scale-load variants
+    switch (resident_chunks(v.K)) {
+      case 2: return launch_ch<FMT, 2, false, 0>(v, x, c, M, s, sh, tiles, T);
+      case 4: return launch_ch<FMT, 4, false, 0>(v, x, c, M, s, sh, tiles, T);
+      case 8: return launch_ch<FMT, 8, false, 0>(v, x, c, M, s, sh, tiles, T);
+      case 11: return launch_ch<FMT, 11, false, 0>(v, x, c, M, s, sh, tiles, T);
+      case 14: return launch_ch<FMT, 14, false, 0>(v, x, c, M, s, sh, tiles, T);
+      default: return hipErrorInvalidValue;
+    }
+  } else {
+    switch (resident_chunks(v.K)) {
+      case 2: W4_GO(2)
+      case 4: W4_GO(4)
+      case 8: W4_LONG(8)
+      case 11: W4_LONG(11)
+      case 14: W4_LONG(14)
+      default: return hipErrorInvalidValue;
+    }
   }
 #undef W4_LONG
 #undef W4_GO
@@ -521,7 +558,7 @@ hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
 
 // Compute units of the current device (per-device cache); 0 on error.
 int device_cus() {
-  static int cached[64] = {};
+  static std::atomic<int> cached[64] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return 0;
   if (dev >= 0 && dev < 64 && cached[dev]) return cached[dev];
@@ -564,9 +601,10 @@ int decode_resident_tiles(const WView& v, const w4_half* x, const w4_half* c, in
   // projections of the 11008- and 14336-wide MLPs)
   if (T > 4 && !(T <= 8 && M <= 32 && v.K == 4096)) T = 4;
   if (resident_chunks(v.K) > 4) T = 1;
-  // the one combination that does not fit the register file: four tiles, four row
-  // tiles, zero-points and per-chunk scale loads
-  if (T == 4 && M > 32 && !v.mx && !v.symmetric && v.gs != 128 && v.gs != 64 && v.gs != 32) T = 3;
+  // what does not fit the register file (dr_tile_cap)
+  const int fmt = v.mx ? 2 : v.symmetric ? 0 : 1, mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+  const int cap = dr_tile_cap(fmt, resident_gsv(v), M > 64 ? 4 : mt);
+  if (T > cap) T = cap;
   return T;
 }
 

@@ -599,12 +599,19 @@ static hipError_t launch_stream_cfg(const WView& v, const w4_half* x, w4_half* c
   // 18.4 vs 15.2 us with one (M = 16) and 19.8 vs 18.4 us with two, so only MT = 4 takes it.
   const bool lean = MT == 4 && wvec && gs32 && (v.mx || gs_shift >= 0) && v.K % (MMA_CHUNK * CPS * KW) == 0 &&
                     v.N % (16 * NW) == 0;
-  if (lean && w_out) {
-    mfma_stream_kernel<FMT, MT, NW, KW, CPS, 1, true, true, true, true>
-        <<<grid, 64 * NW * KW, 0, s>>>(v, x, c, M, w_out, gs_shift);
-  } else if (lean && cpk % DEPTH == 0) {
-    mfma_stream_kernel<FMT, MT, NW, KW, CPS, DEPTH, false, true, true, true>
-        <<<grid, 64 * NW * KW, 0, s>>>(v, x, c, M, w_out, gs_shift);
+  bool lean_done = false;
+  if constexpr (MT == 4) {  // (the lean form is compiled for four activation tiles only)
+    if (lean && w_out) {
+      mfma_stream_kernel<FMT, MT, NW, KW, CPS, 1, true, true, true, true>
+          <<<grid, 64 * NW * KW, 0, s>>>(v, x, c, M, w_out, gs_shift);
+      lean_done = true;
+    } else if (lean && cpk % DEPTH == 0) {
+      mfma_stream_kernel<FMT, MT, NW, KW, CPS, DEPTH, false, true, true, true>
+          <<<grid, 64 * NW * KW, 0, s>>>(v, x, c, M, w_out, gs_shift);
+      lean_done = true;
+    }
+  }
+  if (lean_done) {
   } else if (w_out) {
     if (gs32) W4_GO(1, true, true); else W4_GO(1, true, false);
   } else if (cpk >= DEPTH) {
@@ -623,7 +630,9 @@ template <int FMT, int MT>
 static hipError_t launch_stream_mt(const WView& v, const w4_half* x, w4_half* c, int M,
                                    hipStream_t s, w4_half* w_out, bool wvec) {
   const long long wgs = (long long)((v.N + 63) / 64) * ((M + 16 * MT - 1) / (16 * MT));
-  if (MT < 4 && wgs < 128) return launch_stream_cfg<FMT, MT, 2, 4>(v, x, c, M, s, w_out, wvec);
+  if constexpr (MT < 4) {
+    if (wgs < 128) return launch_stream_cfg<FMT, MT, 2, 4>(v, x, c, M, s, w_out, wvec);
+  }
   return launch_stream_cfg<FMT, MT, 4, 2>(v, x, c, M, s, w_out, wvec);
 }
 

@@ -21,6 +21,8 @@
 //   D: lane l holds D[4*(l/16) + i][l%16], i = 0..3
 // W supplies A (rows n), X supplies B (columns m): a lane ends with four
 // consecutive n of one m.
+#include <atomic>
+
 #include "dq.cuh"
 #include "kernels.h"
 
@@ -221,7 +223,10 @@ __global__ __launch_bounds__(NV_WAVES * 64) void mxn_decode_kernel(
   }
 }
 
-template <int MT, int NT, bool XF8>
+// FULL_ONLY: the caller has checked K % 512 == 0 and the guarded form of this shape is
+// not compiled (it does not fit the register file); unaligned operands then take two
+// row tiles.
+template <int MT, int NT, bool XF8, bool FULL_ONLY = false>
 hipError_t launch_decode_nt(const w4_packed_mx_view& w, const void* xq, const uint8_t* xs, int M,
                             w4_half* c, hipStream_t s) {
   const int N = w.N, K = w.K;
@@ -230,12 +235,15 @@ hipError_t launch_decode_nt(const w4_packed_mx_view& w, const void* xq, const ui
   const dim3 grid((unsigned)((N + 16 * NT - 1) / (16 * NT)),
                   (unsigned)((M + 16 * MT - 1) / (16 * MT)));
   const dim3 block(NV_WAVES * 64);
-  if (full)
+  if (full) {
     mxn_decode_kernel<MT, NT, true, XF8><<<grid, block, 0, s>>>(
         w.q, w.scales, (const uint32_t*)xq, xs, c, N, K, w.B, M);
-  else
+  } else if constexpr (FULL_ONLY) {
+    return launch_decode_nt<MT, 2, XF8>(w, xq, xs, M, c, s);
+  } else {
     mxn_decode_kernel<MT, NT, false, XF8><<<grid, block, 0, s>>>(
         w.q, w.scales, (const uint32_t*)xq, xs, c, N, K, w.B, M);
+  }
   return hipGetLastError();
 }
 
@@ -248,11 +256,18 @@ hipError_t launch_decode(const w4_packed_mx_view& w, const void* xq, const uint8
   // more row tiles per workgroup cut the X traffic (every workgroup reads all of
   // its X rows through L2): worth it from three X tiles on, while a workgroup per
   // CU remains (N = 14336, M = 64: 21.8 us with three row tiles, 29.5 us with one)
-  const int nt = MT >= 3 ? tiles * mblocks / 256 : 1;
-  // (four X tiles times three row tiles do not fit the register file: that instantiation
-  // spills 37 - 85 VGPRs, N = 14336, M = 64: 22.2 / 42.7 us with MXFP4 / MXFP8 activations
-  // against 18.3 / 27.1 with two row tiles)
-  if (nt >= 3 && MT < 4) return launch_decode_nt<MT, 3, XF8>(w, xq, xs, M, c, s);
+  const int nt = (MT >= 3 || (XF8 && MT == 2)) ? tiles * mblocks / 256 : 1;
+  // Four X tiles times three row tiles do not fit the register file (that instantiation
+  // spilled 37 - 85 VGPRs: N = 14336, M = 64, 22.2 / 42.7 us with MXFP4 / MXFP8 activations
+  // against 18.3 / 27.1 with two row tiles), nor do three times three with 8-bit X on a
+  // ragged K; 8-bit X never runs four X tiles (launch_skinny).  None of those is compiled.
+  if constexpr (MT < 4) {
+    if (nt >= 3) {
+      constexpr bool fits_ragged = !(XF8 && MT == 3);
+      const bool full = w.K % 512 == 0;
+      if (fits_ragged || full) return launch_decode_nt<MT, 3, XF8, !fits_ragged>(w, xq, xs, M, c, s);
+    }
+  }
   if (nt >= 2) return launch_decode_nt<MT, 2, XF8>(w, xq, xs, M, c, s);
   return launch_decode_nt<MT, 1, XF8>(w, xq, xs, M, c, s);
 }
@@ -263,7 +278,10 @@ hipError_t launch_skinny(const w4_packed_mx_view& w, const void* xq, const uint8
   if (M <= 16) return launch_decode<1, XF8>(w, xq, xs, M, c, s);
   if (M <= 32) return launch_decode<2, XF8>(w, xq, xs, M, c, s);
   if (M <= 48) return launch_decode<3, XF8>(w, xq, xs, M, c, s);
-  return launch_decode<4, XF8>(w, xq, xs, M, c, s);
+  // 8-bit X: four X tiles hold twice the operand registers of 4-bit ones and spill even
+  // with two row tiles; 49 .. 64 rows go in two passes of 32 (grid.y)
+  if constexpr (XF8) return launch_decode<2, XF8>(w, xq, xs, M, c, s);
+  else return launch_decode<4, XF8>(w, xq, xs, M, c, s);
 }
 
 // ---- large M: LDS-tiled kernel -----------------------------------------------
@@ -797,7 +815,7 @@ hipError_t launch_tile(const w4_packed_mx_view& w, const void* xq, const uint8_t
   const int tiles_n = (w.N + TL_TN - 1) / TL_TN, tiles_m = (M + TL_TM - 1) / TL_TM;
   if ((long long)tiles_n * tiles_m > 0x7FFFFFFFLL) return hipErrorInvalidConfiguration;
   // more than 64 KB of LDS has to be granted per device, once
-  static bool granted[64] = {};
+  static std::atomic<bool> granted[64] = {};
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
   const bool grant = dev < 0 || dev >= 64 || !granted[dev];

@@ -21,6 +21,8 @@
 //     product is rounded once, so the operand is bit for bit the FP16 weight the
 //     one dequant step returns (pack.hpp:58-60).
 // The accumulation is FP32 in the instruction; the output is rounded to FP16 once.
+#include <atomic>
+
 #include "dq.cuh"
 #include "kernels.h"
 
@@ -494,7 +496,7 @@ hipError_t launch(const WView& v, const w4_half* x, w4_half* c, w4_half* w_out, 
   constexpr int TD_LDS = KG * td_lds_bytes(TM, TN);
   static_assert(TD_LDS <= 160 * 1024, "the stage buffers of every set of waves fit LDS");
   // more than 64 KB of LDS has to be granted per device, once
-  static bool granted[64] = {};
+  static std::atomic<bool> granted[64] = {};
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
   if (dev < 0 || dev >= 64 || !granted[dev]) {

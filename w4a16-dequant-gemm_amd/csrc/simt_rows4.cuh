@@ -74,7 +74,13 @@ __global__ __launch_bounds__(SIMT_WAVES * 64) void simt_rows4_kernel(
 #ifndef W4_ROWS4_FOLD
 #define W4_ROWS4_FOLD 1
 #endif
-  constexpr bool FOLD = W4_ROWS4_FOLD && !MX;             // W4: scale and zero-point applied per group, in FP32
+  // W4: scale and zero-point applied per group, in FP32 (w4_dot_biased).  Where it pays:
+  // with three or four activation rows the dot products dominate a word (16 of 21 - 29
+  // instructions) and the per-row bias sums (two per group with zero-points) cost what
+  // the shorter expansion saves -- N = K = 4096, M = 4: gs = 128 4.75 -> 4.41 us
+  // symmetric but 4.77 -> 4.92 with zero-points, gs = 48 with zero-points 5.63 -> 6.19.
+  constexpr bool FOLD = W4_ROWS4_FOLD && !MX &&
+                        (ANY ? (ASYM ? MT == 1 : MT <= 2) : (ASYM ? MT <= 2 : true));
   constexpr int PW = ANY ? 4 : 1;                         // bias sums kept per packed word / per 32-k slice
   // Where the bias sums are formed: by the threads that stage the activations (once per
   // workgroup, before the barrier), or by every lane from its own registers at the head

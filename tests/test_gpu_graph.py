@@ -48,12 +48,15 @@ def test_gemm_replays_equal_eager_calls(i):
         assert np.array_equal(bits(out_g), bits(out_e)), f"replay {rep} differs from the eager call"
 
 
-def test_flash_noalloc_replays_equal_eager_calls():
+# matrix-core flash kernel (D = 128) and the vector flash kernel (D = 96, zero-points)
+@pytest.mark.parametrize("shape", [(4, 3000, 128, 32, 4, True), (3, 1500, 96, 32, 2, False)],
+                         ids=["matrix_core_kernel", "vector_kernel"])
+def test_flash_noalloc_replays_equal_eager_calls(shape):
     c = w4amd.capi()
-    H, S, D, gs, group = 4, 3000, 128, 32, 4
-    seed = 0x6A50
+    H, S, D, gs, group, sym = shape
+    seed = 0x6A50 + D
     c4 = orc.quantize_cache(orc.normal_weights(H * S * D, seed), orc.normal_weights(H * S * D, seed + 1),
-                            H, S, D, gs, True)
+                            H, S, D, gs, sym)
     dk = DevKV(c4)
     q_d = to_dev(orc.normal_activations(H * group * D, seed + 2))
     out_g = halves(H * group * D, 0x7E00)

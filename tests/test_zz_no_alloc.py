@@ -32,13 +32,19 @@ def _one(c, H, S, D, gs, group, sym, seed, hooks):
     ref = orc.attention_f16(q, kd, vd, H, group, S, D)
     dk, q_d = DevKV(c4), to_dev(q)
     want = halves(H * group * D, 0x7E00)
-    c.attention_w4_flash(dk.view, ptr(q_d), ptr(want), group=group)
-    want = bits(want).copy()
     got = halves(H * group * D, 0x7E00)
     ko = halves(H * S * D, 0x7E00) if hooks else None
     vo = halves(H * S * D, 0x7E00) if hooks else None
     print(f"noalloc case H={H} S={S} D={D} gs={gs} group={group} sym={sym} hooks={hooks}", flush=True)
+    # the entry that allocates nothing goes first (so the other entry's grow-only buffer cannot
+    # stand in for an allocation of its own) and must leave the device's free memory as it was
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
     c.attention_w4_flash_noalloc(dk.view, ptr(q_d), ptr(got), 0, ptr(ko), ptr(vo), group=group)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "the no-alloc entry changed the device's free memory"
+    c.attention_w4_flash(dk.view, ptr(q_d), ptr(want), group=group)
+    want = bits(want).copy()
     got = bits(got).copy()
     assert np.array_equal(got, want), "noalloc output differs from w4_attention_w4_flash_gqa"
     assert orc.rel_l2(got.view(np.float16), ref) <= TOL

@@ -96,6 +96,10 @@ __global__ __launch_bounds__(DG_THREADS) void mfma_decode_general_kernel(
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
           if (ph * CP + cc >= CH) continue;
+          // quads of activation rows that do not exist are not fetched (with one row tile:
+          // M = 8 moves half, M = 4 a quarter of a tile's 128 KB through L2 -> LDS); their
+          // columns of the product are never stored, whatever the region holds there
+          if (MT == 1 && m0 + 4 * rq >= M) continue;
           const int r16 = 4 * rq + (lane >> 4), row = m0 + 16 * mt + r16;
           const int cidx = chunk_of(ph * CP + cc);
           // 16-byte piece (lane % 16) ^ r16 of the chunk's 256 bytes; pieces past K repeat piece 0

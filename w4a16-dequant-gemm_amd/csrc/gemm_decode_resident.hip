@@ -253,6 +253,10 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
 #pragma unroll
         for (int rq = 0; rq < 4; ++rq) {
           if (ph * CP + cc >= CH) continue;
+          // quads of activation rows that do not exist are not fetched (with one row tile:
+          // M = 8 moves half, M = 4 a quarter of a tile's 128 KB through L2 -> LDS); their
+          // columns of the product are never stored, whatever the region holds there
+          if (MT == 1 && m0 + 4 * rq >= M) continue;
           const int r16 = 4 * rq + (lane >> 4), row = m0 + 16 * mt + r16;
           const int cidx = wave * CH + ph * CP + cc;  // a chunk past the end repeats the last one
           const uint32_t off = (uint32_t)min(row, M - 1) * (uint32_t)(K * 2) +

@@ -86,7 +86,8 @@ int w4_dispatch_mma_min_m(void);
  * three or four activation rows cost the vector kernels a second pass over their
  * staged activations, the matrix-core kernel fetches only the rows that exist
  * (N = 4096, K = 11008, M = 3: 18.2 us against 9.0; up to K = 6144 in whole chunks of
- * 128 already from M = 2), and for wide matrices at K <= 4096 (N * K >= 44 M: N = 11008 or
+ * 128 already from M = 2), and for wide matrices at K <= 4096 (N * K >= 172 000 per compute unit,
+ * 44 M on an MI355X: N = 11008 or
  * 14336 at K = 4096, M = 3 / 4: 8.6 - 9.6 us against 9.4 - 11.8).  Everywhere else this is
  * w4_dispatch_mma_min_m().  No counterpart in the reference, whose crossover is one
  * constant (dispatch.cuh:25). */

@@ -179,6 +179,19 @@ extern "C" {
 const char* w4_last_error(void) { return g_msg; }
 
 int w4_dispatch_mma_min_m(void) { return DISPATCH_MMA_MIN_M; }
+// Compute units of the current device, 256 (an MI355X) when there is none to ask: the
+// threshold functions are plain arithmetic and callable without a GPU.
+static int dispatch_cus() {
+  static std::atomic<int> cached[MAX_DEVICES] = {};
+  int dev = -1, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return 256;
+  if (const int have = cached[dev].load(std::memory_order_relaxed)) return have;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1)
+    return 256;
+  cached[dev].store(n, std::memory_order_relaxed);
+  return n;
+}
+
 int w4_dispatch_mma_min_m_for_gs(int N, int K, int gs) {
   if (K % 32 != 0 && K % 8 == 0 && (long long)N * K >= (1LL << 25)) return 2;
   if (K > 4096 && K <= 6144 && K % 128 == 0) return 2;  // 5.8 us against 6.3 at N = 4096, M = 2
@@ -189,7 +202,11 @@ int w4_dispatch_mma_min_m_for_gs(int N, int K, int gs) {
   // against 7.6).  Group sizes that are no multiple of 32 go to the matrix cores' general
   // kernel, which is slower there (N = 11008, gs = 48, M = 4: 11.8 us against 11.3 on the
   // vector units): they keep the plain threshold.
-  if (K % 32 == 0 && (gs <= 0 || gs % 32 == 0) && (long long)N * K >= 44000000LL) return 3;
+  // (measured on 256 compute units as N * K >= 44 M; what matters is that the grid holds
+  // more than about 2.6 16-row tiles of 4096 k per compute unit, so it scales with them)
+  if (K % 32 == 0 && (gs <= 0 || gs % 32 == 0) &&
+      (long long)N * K >= 172000LL * dispatch_cus())
+    return 3;
   return DISPATCH_MMA_MIN_M;
 }
 int w4_dispatch_mma_min_m_for(int N, int K) { return w4_dispatch_mma_min_m_for_gs(N, K, 0); }

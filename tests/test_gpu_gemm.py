@@ -307,3 +307,27 @@ def test_mx_dequant_exhaustive():
     assert np.array_equal(bits(w2), want)
     c.gemm_mma_mx(dp.view, ptr(x_d), ptr(c_d), 1, 0, ptr(w2.fill_(0x7E00)))
     assert np.array_equal(bits(w2), want)
+
+
+@pytest.mark.parametrize("shape", [(1024, 4096, 128, True), (1024, 4096, 128, False), (512, 11008, 128, True),
+                                   (512, 4096, 48, False), (512, 8192, 32, True)])
+def test_unhooked_vector_kernels_with_one_signed_and_offset_activations(shape):
+    """The vector kernels' unhooked arithmetic subtracts a bias sum that grows with the sum of the
+    activations; activations of one sign, with a large mean or a large magnitude are where that
+    cancellation would show.  Held to the same 5e-4 against the FP64 oracle as everywhere else."""
+    c = w4amd.capi()
+    N, K, gs, sym = shape
+    p = orc.quantize(orc.normal_weights(N * K, 0x0FF5E7) * 0.02, N, K, gs, sym)
+    w_ref = orc.dequant_all(p)
+    dp = DevPacked(p)
+    rng = np.random.default_rng(5)
+    for M in (1, 2):
+        for name, x64 in (("abs", np.abs(rng.standard_normal(M * K))), ("mean3", 3 + rng.standard_normal(M * K)),
+                          ("mean30", 30 + rng.standard_normal(M * K)),
+                          ("large", 1000 * np.abs(rng.standard_normal(M * K))), ("ones", np.ones(M * K))):
+            x = np.asarray(x64, np.float16).view(np.uint16)
+            ref = orc.gemm_oracle(x, M, K, w_ref, N)
+            x_d = to_dev(x)
+            ch, _ = _run(c.gemm, dp.view, x_d, M, N, K)
+            cu, _ = _run(c.gemm, dp.view, x_d, M, N, K, hook=False)
+            cross_gate(ch, cu, ref, name)

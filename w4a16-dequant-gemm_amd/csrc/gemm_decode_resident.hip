@@ -140,18 +140,16 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
         qw[t][i] = __builtin_nontemporal_load((const u4*)(qr + (chunk_k(i) >> 3)));
     }
   };
-  auto pair_fix = [&](int t) {
+  auto pair_fix = [&](int t, int i) {  // chunks i, i + 1 (i even)
     if (!paired) return;
     const bool lo = r < 8;
 #pragma unroll
-    for (int i = 0; i + 1 < CH; i += 2)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const uint32_t a = qw[t][i][e], bb = qw[t][i + 1][e];
-        qw[t][i][e] = lo ? a : bb;
-        // row_ror:8 -- lane r of each row of 16 takes the value of lane r ^ 8
-        qw[t][i + 1][e] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(lo ? bb : a), 0x128, 0xF, 0xF, true);
-      }
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t a = qw[t][i][e], bb = qw[t][i + 1][e];
+      qw[t][i][e] = lo ? a : bb;
+      // row_ror:8 -- lane r of each row of 16 takes the value of lane r ^ 8
+      qw[t][i + 1][e] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(lo ? bb : a), 0x128, 0xF, 0xF, true);
+    }
   };
   auto load_scales = [&](int t) {
     if constexpr (MX && !EXACT) {
@@ -344,15 +342,20 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
         __builtin_amdgcn_sched_barrier(0);
         if (t + 1 < T) load_tile(t + 1);
         __builtin_amdgcn_sched_barrier(0);
-        if (t == 1) __builtin_amdgcn_s_waitcnt(waitcnt_vm(NX1 + (T > 2 ? CH : 0)));
-        else if (t + 1 < T) __builtin_amdgcn_s_waitcnt(waitcnt_vm(CH));
-        else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+        // (only the tile's first pair of chunks has to be here: the rest of it lands while
+        // that pair is expanded -- the compiler places the waits for the later registers --
+        // so the last tile's arithmetic, which nothing overlaps, starts half a tile earlier)
+        constexpr int LATER = (PAIRC && CH >= 4) ? CH - 2 : 0;
+        static_assert(NX1 + CH + LATER < 64, "vmcnt is a 6-bit counter");
+        if (t == 1) __builtin_amdgcn_s_waitcnt(waitcnt_vm(NX1 + (T > 2 ? CH : 0) + LATER));
+        else if (t + 1 < T) __builtin_amdgcn_s_waitcnt(waitcnt_vm(CH + LATER));
+        else __builtin_amdgcn_s_waitcnt(waitcnt_vm(LATER));
       }
 #pragma unroll
       for (int cc = 0; cc < CP; ++cc) {
         const int i = ph * CP + cc;
         if (i >= CH) continue;
-        if (ph == 0 && cc == 0) pair_fix(t);
+        if (PAIRC && (i & 1) == 0 && i + 1 < CH) pair_fix(t, i);
         h2 cneg, s2;
         float sf = 0.f;
         if (MX) {

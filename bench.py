@@ -1001,18 +1001,18 @@ def probe(b, which, args):
         for M in (1, 16, 64, 2048):
             b.steps, b.warmup = (20, 3) if M > 64 else (100, 10)
             out["w4a4_M%d_us" % M] = b.w4a4_us(views, M, N, K, reps=1)
-    else:  # prefill: the fused tile kernel and the plain FP16 library GEMM, 20 calls each
+    else:  # prefill: the fused tile kernels and the plain FP16 library GEMM, 20 calls each at M = 2048 and 4096
         N = K = 4096
-        M = 2048
         views = rand_w4_views(b, N, K, 128, True, 1)
-        x = torch.randn(M * K, device="cuda").to(torch.float16)
-        c = torch.empty(M * N, dtype=torch.float16, device="cuda")
         w16 = torch.empty(N * K, dtype=torch.float16, device="cuda")
         capi.dequant(views[0][0], w16.data_ptr(), b.stream)
-        for _ in range(20):
-            capi.gemm(views[0][0], x.data_ptr(), c.data_ptr(), M, b.stream, 0)
-            capi.gemm_fp16(w16.data_ptr(), x.data_ptr(), c.data_ptr(), M, N, K, b.stream)
-        torch.cuda.synchronize()
+        for M in (2048, 4096):
+            x = torch.randn(M * K, device="cuda").to(torch.float16)
+            c = torch.empty(M * N, dtype=torch.float16, device="cuda")
+            for _ in range(20):
+                capi.gemm(views[0][0], x.data_ptr(), c.data_ptr(), M, b.stream, 0)
+                capi.gemm_fp16(w16.data_ptr(), x.data_ptr(), c.data_ptr(), M, N, K, b.stream)
+            torch.cuda.synchronize()
     print(json.dumps(out))
 
 

@@ -11,7 +11,7 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG, "csrc")
 LIB = os.path.join(PKG, "lib", "libw4amd.so")
 BENCH_LIB = os.path.join(PKG, "lib", "libw4bench.so")
-SOURCES = ["abi.hip", "dequant.hip", "gemm_simt.hip", "gemm_mfma.hip", "flash.hip", "flash_mfma.hip", "quantize.hip", "gemm_mxnative.hip", "gemm_tile_dma.hip", "gemm_decode_resident.hip", "gemm_decode_general.hip", "gemm_decode_longk.hip",
+SOURCES = ["abi.hip", "dequant.hip", "gemm_simt.hip", "gemm_mfma.hip", "flash.hip", "flash_mfma.hip", "quantize.hip", "gemm_mxnative.hip", "gemm_tile_dma.hip", "gemm_tile256.hip", "gemm_decode_resident.hip", "gemm_decode_general.hip", "gemm_decode_longk.hip",
            "baseline.hip"]
 HEADERS = ["dq.cuh", "kernels.h", "simt_rows4.cuh", "bench_kernels.hip", os.path.join("..", "..", "include", "w4_abi.h")]
 FLAGS = [

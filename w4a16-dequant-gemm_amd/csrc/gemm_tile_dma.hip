@@ -589,6 +589,8 @@ bool try_tile_dma(const WView& v, const w4_half* x, w4_half* c, int M, hipStream
   if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)v.scales & 3)) return false;
   if (!v.mx && !v.symmetric && (v.zeros == nullptr || ((uintptr_t)v.zeros & 3))) return false;
   if (w_out && ((uintptr_t)w_out & 15)) return false;
+  // grids of more than one round: 256 x 256 tiles where they halve the rounds
+  if (!w_out && try_tile256(v, x, c, M, s, 256, err)) return true;
   const int tn = (int)tiles_n, tm = (int)tiles_m;
   if (v.mx) *err = launch_hook<2, 2>(v, x, c, w_out, M, s, tn, tm, shape, sets, split_at);
   else if (v.symmetric) *err = launch_gsm<0>(gsm, v, x, c, w_out, M, s, tn, tm, shape, sets, split_at);

@@ -44,6 +44,12 @@ hipError_t launch_gemm_mfma(const WView& v, const w4_half* x, w4_half* c, int M,
 bool try_tile_dma(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s,
                   w4_half* w_out, hipError_t* err);
 
+// gemm_tile256.hip: the same scheme on 256 x 256 tiles, for try_tile_dma to hand unhooked
+// calls to once it has checked the operands; false (nothing launched) when that tile
+// would not at least halve the rounds of workgroups on `cus` compute units.
+bool try_tile256(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int cus,
+                 hipError_t* err);
+
 // gemm_decode_resident.hip: M <= 64 with the activations fetched once per workgroup
 // (several 16-row tiles each).  Same order of additions as the K-split decode
 // kernels of gemm_mfma.hip, which serve the hooked calls of these shapes.

@@ -12,6 +12,9 @@
 //     one wave per SIMD has 512);
 //   * a stage is 64 k: 32 bytes of a W row, 128 bytes of an X row (one line), 42 KB;
 //     three stage buffers, one barrier per stage (64 MFMAs per wave);
+//   * the instruction order of the main loop is fixed by hand, MFMA by MFMA: with one wave
+//     per SIMD every vector, LDS and load instruction is issued between two MFMAs of the
+//     same wave, and a dependent pair back to back costs the wave the first one's latency;
 //   * lane l of an MFMA brings row l % 32 and k 32 (l / 32) + 8 u .. + 7 in step u of a
 //     stage: its four W words are one 16-byte LDS read per stage and 32-row tile, its X
 //     operand is 16-byte piece 4 (l / 32) + u of the row.
@@ -28,9 +31,6 @@ namespace {
 typedef float f16v __attribute__((ext_vector_type(16)));
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
-#ifndef T2_WM
-#define T2_WM 1
-#endif
 constexpr int T2_THREADS = 256, T2_STAGES = 3;
 constexpr int T2_W_BYTES = 256 * 32, T2_X_BYTES = 256 * 128;
 constexpr int T2_TILE = T2_W_BYTES + T2_X_BYTES;
@@ -59,23 +59,20 @@ __device__ __forceinline__ int t2_w_at(int R, int p) { return (R * 2 + p) * 16; 
 // FMT: 0 W4 symmetric, 1 W4 with zero-points, 2 MXFP4.  GS32: W4 groups of 32 (a lane's
 // 32 k of a stage are one group, the stage two); otherwise gs is a multiple of 64 and
 // the stage lies in one group.  G: scales per row (MXFP4: E8M0 bytes per row).
-// WM: sets of four waves along m.  1: a wave holds 64 rows of W against all 256 of X; 2: against
-// 128 of them (two waves per SIMD, each with half the accumulators; both sets expand the words).
-template <int FMT, bool GS32, int WM>
-__global__ __launch_bounds__(T2_THREADS * WM) void w4_tile256_kernel(
+template <int FMT, bool GS32>
+__global__ __launch_bounds__(T2_THREADS) void w4_tile256_kernel(
     const uint32_t* __restrict__ wq, const void* __restrict__ scales,
     const uint32_t* __restrict__ zeros, const w4_half* __restrict__ x, w4_half* __restrict__ c,
     int N, int K, int G, int gs, int M, int tiles_n, int tiles_m) {
   constexpr bool ASYM = FMT == 1, MX = FMT == 2;
-  constexpr int WAVES = 4 * WM;
-  constexpr int NI = 2, MJ = 8 / WM;             // 32-row tiles of W and of X per wave
+  constexpr int WAVES = 4;
+  constexpr int NI = 2, MJ = 8;                   // 32-row tiles of W and of X per wave
   constexpr int WI = 8 / WAVES, XI = 32 / WAVES;  // 1 KB load instructions of W and of X per wave and stage
   constexpr int LOADS = WI + XI + 1 + (ASYM ? 1 : 0);
   constexpr int CH = NI * MJ / 4;  // chunks of four MFMAs per 16-k step
   static_assert(LOADS <= 4 * CH, "at most one load instruction per chunk");
   const int t = threadIdx.x, lane = t & 63;
-  const int wave_all = __builtin_amdgcn_readfirstlane(t >> 6);  // in an SGPR: LDS addresses go to M0
-  const int wave = wave_all & 3, wm = wave_all >> 2;          // 64 rows of W; the half of X (WM = 2)
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);  // in an SGPR: LDS addresses go to M0
   const int r = lane & 31, h = lane >> 5;
   // Consecutive workgroup ids land on different XCDs (each with its own L2): give each
   // XCD a block of the tile grid, or failing that a contiguous run of the tile order, m fastest.
@@ -101,17 +98,16 @@ __global__ __launch_bounds__(T2_THREADS * WM) void w4_tile256_kernel(
   uint32_t wo[WI], xo[XI];
 #pragma unroll
   for (int i = 0; i < WI; ++i) {
-    const int n = n0 + (wave_all + WAVES * i) * 32 + (lane >> 1);
+    const int n = n0 + (wave + WAVES * i) * 32 + (lane >> 1);
     wo[i] = (uint32_t)(n < N ? n : N - 1) * (uint32_t)(K >> 1) + (lane & 1) * 16;
   }
 #pragma unroll
   for (int i = 0; i < XI; ++i) {
-    const int R = (wave_all + WAVES * i) * 8 + (lane >> 3), m = m0 + R;
+    const int R = (wave + WAVES * i) * 8 + (lane >> 3), m = m0 + R;
     xo[i] = (uint32_t)(m < M ? m : M - 1) * (uint32_t)(K * 2) + (((lane & 7) ^ t2_x_key(R)) * 16);
   }
   // per stage: the dword that holds the scale(s) of W row 64 wave + lane, and (ASYM) the
-  // word that holds its zero-point (with two sets of waves both fetch them, to the same place:
-  // every wave then has the same count of loads in flight)
+  // word that holds its zero-point
   const uint32_t sn = (uint32_t)(n0 + wave * 64 + lane < N ? n0 + wave * 64 + lane : N - 1);
   const uint32_t sc_base = sn * (uint32_t)G, zw_base = sn * (uint32_t)wg;
   const char* wqb = (const char*)wq;
@@ -142,10 +138,10 @@ __global__ __launch_bounds__(T2_THREADS * WM) void w4_tile256_kernel(
     const uint32_t dd = (uint32_t)(d < stages ? d : stages - 1);
     const uint32_t st = lds0 + buf;
     if (part < WI) {  // the stage's offset goes into the scalar base: no vector arithmetic
-      dma16(wqb + dd * 32u, wo[part], st + (wave_all + WAVES * part) * 1024);
+      dma16(wqb + dd * 32u, wo[part], st + (wave + WAVES * part) * 1024);
     } else if (part < WI + XI) {
       const int i = part - WI;
-      dma16(xb + dd * 128u, xo[i], st + T2_W_BYTES + (wave_all + WAVES * i) * 1024);
+      dma16(xb + dd * 128u, xo[i], st + T2_W_BYTES + (wave + WAVES * i) * 1024);
     } else if (part == WI + XI) {
       // MXFP4: the dword around the stage's two E8M0 bytes; gs = 32: the dword of its two
       // scales; else the dword around its one scale
@@ -180,7 +176,7 @@ __global__ __launch_bounds__(T2_THREADS * WM) void w4_tile256_kernel(
   // m tile 0 (tile j is 4 KB further), its four words in n tile 0 (tile 1 is 1 KB further).
   uint32_t xoff[4];
 #pragma unroll
-  for (int u = 0; u < 4; ++u) xoff[u] = T2_W_BYTES + t2_x_at(wm * 128 + r, 4 * h + u);
+  for (int u = 0; u < 4; ++u) xoff[u] = T2_W_BYTES + t2_x_at(r, 4 * h + u);
   const uint32_t woff = t2_w_at(wrow0, h), scoff = T2_TILE + wrow0 * 4;
   auto read_x = [&](u4* dst, uint32_t buf, int u, int j0, int j1) {  // m tiles j0 .. j1 - 1 of step u
     const uint8_t* p = t2_lds + (buf + xoff[u]);
@@ -265,12 +261,12 @@ __global__ __launch_bounds__(T2_THREADS * WM) void w4_tile256_kernel(
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  // A stage is 4 CH chunks of four MFMAs, and a chunk issues at most one load instruction:
-  // a load holds up the wave's instruction stream while it is taken in, which four MFMAs
-  // in flight cover and a run of loads does not.  The barrier at the start of step 3 of
-  // stage d frees that stage's buffer; the chunks from there (step 3 of stage d, steps
-  // 0 .. 2 of stage d + 1) request stage d + 3 into it.  b0, b1, b2: byte offsets of the
-  // buffers of stages d, d + 1, d + 2 (d + 3 takes b0 again).
+  // A stage is sixteen chunks of four MFMAs.  A chunk issues at most one load instruction,
+  // reads two tiles of X and expands two operand registers of the next step, one of the four
+  // dependent instructions of each under each MFMA.  The barrier at the start of step 3 of
+  // stage d frees that stage's buffer; the sixteen chunks from there (step 3 of stage d,
+  // steps 0 .. 2 of stage d + 1) request stage d + 3 into it.  b0, b1, b2: byte offsets of
+  // the buffers of stages d, d + 1, d + 2 (d + 3 takes b0 again).
   uint32_t b0 = 0, b1 = T2_STAGE, b2 = 2 * T2_STAGE;
 #pragma unroll
   for (int part = 0; part < LOADS; ++part) request_part(0, b0, part);
@@ -291,7 +287,7 @@ __global__ __launch_bounds__(T2_THREADS * WM) void w4_tile256_kernel(
         __builtin_bit_cast(h8, av[cur][i]), __builtin_bit_cast(h8, xv[cur][j]), acc[i][j], 0, 0, 0);
   };
   constexpr int RPC = 8 / CH, XPC = MJ / CH;  // operand registers expanded, X tiles read per chunk
-  uint32_t tmp[8];
+  uint32_t tmp[4];
 #pragma unroll 1
   for (int d = 0; d < stages; ++d) {
 #pragma unroll
@@ -316,60 +312,36 @@ __global__ __launch_bounds__(T2_THREADS * WM) void w4_tile256_kernel(
     // stage d + 3, and stage d + 1 has landed for everyone (outstanding: all of stage d + 2).
     __builtin_amdgcn_s_waitcnt(t2_waitcnt_vm(LOADS));
     __syncthreads();
-    if constexpr (WM == 1) {
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        request_part(d + 3, b0, c);
-        __builtin_amdgcn_sched_barrier(0);
-        if (c == 0) {  // operands of step 0 of stage d + 1: the words, their scales, half of X
-          read_w(b1);
-          read_sc(b1);
-          read_x(xv[0], b1, 0, 0, 4);
-        } else if (c == 1) {
-          read_x(xv[0], b1, 0, 4, 8);
-          set_group(d + 1);
-        }
-        if (c < 2) {
-#pragma unroll
-          for (int k = 0; k < 4; ++k) mfma1(1, c, k);
-          if (c == 0) __builtin_amdgcn_sched_group_barrier(0x100, 4 + NI + NI * (ASYM ? 2 : 1), 0);
-          if (c == 1) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (c > 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        } else {
-#pragma unroll
-          for (int k = 0; k < 4; ++k) {
-            expand_phase(k, av[0], tmp, 0, c - 2, 0, 4);
-            mfma1(1, c, k);
-            __builtin_amdgcn_sched_barrier(0);
-          }
-        }
+    for (int c = 0; c < 4; ++c) {
+      request_part(d + 3, b0, c);
+      __builtin_amdgcn_sched_barrier(0);
+      if (c == 0) {  // operands of step 0 of stage d + 1: the words, their scales, half of X
+        read_w(b1);
+        read_sc(b1);
+        read_x(xv[0], b1, 0, 0, 4);
+      } else if (c == 1) {
+        read_x(xv[0], b1, 0, 4, 8);
+        set_group(d + 1);
       }
-    } else {
-      // two chunks: the reads of the next stage's first operands under the first four
-      // MFMAs, the group's constants and the expansion of both words under the last four
-      request_part(d + 3, b0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      read_w(b1);
-      read_sc(b1);
-      read_x(xv[0], b1, 0, 0, MJ);
+      if (c < 2) {
 #pragma unroll
-      for (int k = 0; k < 4; ++k) mfma1(1, 0, k);
-      __builtin_amdgcn_sched_barrier(0);
-      request_part(d + 3, b0, 1);
-      __builtin_amdgcn_sched_barrier(0);
-      set_group(d + 1);
-      __builtin_amdgcn_sched_barrier(0);
+        for (int k = 0; k < 4; ++k) mfma1(1, c, k);
+        if (c == 0) __builtin_amdgcn_sched_group_barrier(0x100, 4 + NI + NI * (ASYM ? 2 : 1), 0);
+        if (c == 1) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        expand_phase(k, av[0], tmp, 0, 0, 0, 4);
-        expand_phase(k, av[0], tmp + 4, 0, 1, 0, 4);
-        mfma1(1, 1, k);
+        for (int k = 0; k < 4; ++k) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (c > 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          expand_phase(k, av[0], tmp, 0, c - 2, 0, 4);
+          mfma1(1, c, k);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     }
     const uint32_t first = b0;
@@ -384,7 +356,7 @@ __global__ __launch_bounds__(T2_THREADS * WM) void w4_tile256_kernel(
   // lines: a wave lays its 256 (m) x 64 (n) block out in rows of 144 bytes and reads it
   // back 16 bytes a lane.  Rows past M and columns past N stay in LDS.
   __syncthreads();  // no wave reads a stage buffer any more, no load is landing in one
-  uint8_t* mine = t2_lds + wave_all * (32 * MJ * T2_C_PITCH);
+  uint8_t* mine = t2_lds + wave * (32 * MJ * T2_C_PITCH);
 #pragma unroll
   for (int j = 0; j < MJ; ++j) {
     // the sums of an m tile leave the accumulator registers only when its turn comes (256
@@ -405,7 +377,7 @@ __global__ __launch_bounds__(T2_THREADS * WM) void w4_tile256_kernel(
   const int nn = n0 + wave * 64 + (lane & 7) * 8;
 #pragma unroll 4
   for (int it = 0; it < 32 * MJ / 8; ++it) {
-    const int row = it * 8 + (lane >> 3), m = m0 + wm * 128 + row;
+    const int row = it * 8 + (lane >> 3), m = m0 + row;
     if (m >= M || nn >= N) continue;
     const u4 v = *(const u4*)(mine + row * T2_C_PITCH + (lane & 7) * 16);
     w4_half* dst = c + (size_t)m * N + nn;
@@ -419,7 +391,7 @@ __global__ __launch_bounds__(T2_THREADS * WM) void w4_tile256_kernel(
   }
 }
 
-template <int FMT, bool GS32, int WM = T2_WM>
+template <int FMT, bool GS32>
 hipError_t launch(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int tiles_n,
                   int tiles_m) {
   // more than 64 KB of LDS has to be granted per device, once
@@ -427,12 +399,12 @@ hipError_t launch(const WView& v, const w4_half* x, w4_half* c, int M, hipStream
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
   if (dev < 0 || dev >= 64 || !granted[dev]) {
-    const hipError_t e = hipFuncSetAttribute((const void*)w4_tile256_kernel<FMT, GS32, WM>,
+    const hipError_t e = hipFuncSetAttribute((const void*)w4_tile256_kernel<FMT, GS32>,
                                              hipFuncAttributeMaxDynamicSharedMemorySize, T2_LDS);
     if (e != hipSuccess) return e;
     if (dev >= 0 && dev < 64) granted[dev] = true;
   }
-  w4_tile256_kernel<FMT, GS32, WM><<<dim3((unsigned)(tiles_n * tiles_m)), dim3(T2_THREADS * WM), T2_LDS, s>>>(
+  w4_tile256_kernel<FMT, GS32><<<dim3((unsigned)(tiles_n * tiles_m)), dim3(T2_THREADS), T2_LDS, s>>>(
       v.q, v.scales, v.zeros, x, c, v.N, v.K, v.mx ? v.B : v.G, v.gs, M, tiles_n, tiles_m);
   return hipGetLastError();
 }

@@ -112,6 +112,7 @@ __global__ __launch_bounds__(TD_THREADS * KG) void w4_tile_dma_kernel(
   constexpr int TD_TILE = td_tile(TM, TN), TD_STAGE = td_stage(TM, TN);
   constexpr int TD_XI = TM * 256 / 1024 / TD_WAVES;        // 1 KB load instructions of X per wave
   constexpr int LOADS = TD_WI + TD_XI + NSC + (ASYM ? 1 : 0);  // load instructions per wave and stage
+  constexpr bool PHASED = NI * MJ >= 4;  // a step has the four MFMAs that the phases of an expansion go under
   const int t = threadIdx.x, lane = t & 63;
   const int wave_all = __builtin_amdgcn_readfirstlane(t >> 6);  // in an SGPR: LDS addresses go to M0
   const int wave = KG == 2 ? (wave_all & 3) : wave_all;        // within its set of four
@@ -221,7 +222,7 @@ __global__ __launch_bounds__(TD_THREADS * KG) void w4_tile_dma_kernel(
 
   u4 xv[2][MJ];           // X operands of the step in hand and of the next: [m tile]
   u4 wv[2][NI];           // packed words of the two 64-k halves: [half][n tile], word = step % 4
-  h8 av[2][NI];           // expanded W operands of the step in hand and of the next
+  u4 av[2][NI];           // expanded W operands (four packed-half registers) of the step in hand and of the next
   uint32_t sc[NI][NSC], zw[NI];  // the stage's scale dwords and zero-point word per n tile
   // what expansion needs, per [half][n tile]: -(1024 + z), -(64 + z) and the scale in
   // both halves of a register (MXFP4: the scale as a float)
@@ -281,19 +282,45 @@ __global__ __launch_bounds__(TD_THREADS * KG) void w4_tile_dma_kernel(
         }
       }
   };
-  auto expand = [&](h8* dst, int d, int u) {
+  auto hook_store = [&](const u4* src, int d, int u, int i) {
+    if (HOOK && hook && d < stages && n0 + wrow[i] < N)
+      *(u4*)(w_out + (size_t)(n0 + wrow[i]) * K + d * 128 + (u >> 2) * 64 + h * 32 + (u & 3) * 8) = src[i];
+  };
+  auto expand = [&](u4* dst, int d, int u) {
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
       if constexpr (MX) {
         h2 n4[4];
         dq_mx(wv[u >> 2][i][u & 3], sf[u >> 2][i], n4);
-        dst[i] = __builtin_bit_cast(h8, u4{as_u32(n4[0]), as_u32(n4[1]), as_u32(n4[2]), as_u32(n4[3])});
+        dst[i] = u4{as_u32(n4[0]), as_u32(n4[1]), as_u32(n4[2]), as_u32(n4[3])};
       } else {
-        dst[i] = expand_word(wv[u >> 2][i][u & 3], cneg[u >> 2][i], s2v[u >> 2][i], mask, magic);
+        dst[i] = __builtin_bit_cast(
+            u4, expand_word(wv[u >> 2][i][u & 3], cneg[u >> 2][i], s2v[u >> 2][i], mask, magic));
       }
-      if (HOOK && hook && d < stages && n0 + wrow[i] < N)
-        *(h8*)(w_out + (size_t)(n0 + wrow[i]) * K + d * 128 + (u >> 2) * 64 + h * 32 + (u & 3) * 8) =
-            dst[i];
+      hook_store(dst, d, u, i);
+    }
+  };
+  // The same in four phases over the registers e0 .. e0 + nr - 1 of n tile i, one phase per
+  // MFMA: the four instructions of a register depend on each other, and a wave that issues
+  // them back to back waits out each one's latency.  t: the values in between.
+  auto expand_phase = [&](int ph, u4* dst, uint32_t* t, int u, int i, int e0, int nr) {
+    const uint32_t w = wv[u >> 2][i][u & 3];
+#pragma unroll
+    for (int q = 0; q < nr; ++q) {
+      const int e = e0 + q;
+      if constexpr (MX) {
+        const float sc_f = sf[u >> 2][i];
+        if (ph == q % 4)
+          dst[i][e] = as_u32(e == 0   ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, sc_f, 0)
+                             : e == 1 ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, sc_f, 1)
+                             : e == 2 ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, sc_f, 2)
+                                      : __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, sc_f, 3));
+      } else {
+        if (ph == 0) t[q] = __builtin_amdgcn_perm(0u, w, 0x0c000c00u | (uint32_t)(e << 16) | (uint32_t)e);
+        if (ph == 1) t[q] = (t[q] & mask) | magic;
+        if (ph == 2) t[q] = as_u32(as_h2(t[q]) + cneg[u >> 2][i]);
+        if (ph == 3) dst[i][e] = as_u32(as_h2(t[q]) * s2v[u >> 2][i]);
+      }
     }
   };
 
@@ -359,19 +386,45 @@ __global__ __launch_bounds__(TD_THREADS * KG) void w4_tile_dma_kernel(
         __builtin_amdgcn_sched_barrier(0);
         read_x(xv[(u + 1) & 1], b0, u + 1);
         if (u == 0) read_w(wv[1], b0, 1);
-        expand(av[(u + 1) & 1], d, u + 1);
+        if constexpr (!PHASED) expand(av[(u + 1) & 1], d, u + 1);
       }
-      if (KG == 1 || d < stages) {
+      constexpr int NM = NI * MJ;  // MFMAs of a step
+      auto mfma = [&](int k) {
+        const int i = k / MJ, j = k % MJ;
+        if (KG == 1 || d < stages)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+              __builtin_bit_cast(h8, av[u & 1][i]), __builtin_bit_cast(h8, xv[u & 1][j]), acc[i][j], 0, 0, 0);
+      };
+      bool done = false;
+      if constexpr (PHASED) if (u < 7) {
+        done = true;
+        // the operands of step u + 1, expanded under this step's MFMAs: four MFMAs per group
+        // of RPG registers, one phase under each
+        constexpr int RPG = 16 * NI / NM;  // registers per group of four MFMAs
+        uint32_t tmp[RPG];
 #pragma unroll
-        for (int i = 0; i < NI; ++i)
-#pragma unroll
-          for (int j = 0; j < MJ; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                av[u & 1][i], __builtin_bit_cast(h8, xv[u & 1][j]), acc[i][j], 0, 0, 0);
+        for (int k = 0; k < NM; ++k) {
+          if constexpr (RPG == 4) {  // a group of four MFMAs per word
+            expand_phase(k & 3, av[(u + 1) & 1], tmp, u + 1, k >> 2, 0, 4);
+            if ((k & 3) == 3) hook_store(av[(u + 1) & 1], d, u + 1, k >> 2);
+          } else {  // four MFMAs in all: both words under them
+            static_assert(RPG == 8 && NI == 2, "64 rows of X against two tiles of W");
+            expand_phase(k & 3, av[(u + 1) & 1], tmp, u + 1, 0, 0, 4);
+            expand_phase(k & 3, av[(u + 1) & 1], tmp + 4, u + 1, 1, 0, 4);
+            if ((k & 3) == 3) {
+              hook_store(av[(u + 1) & 1], d, u + 1, 0);
+              hook_store(av[(u + 1) & 1], d, u + 1, 1);
+            }
+          }
+          mfma(k);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
+      if (!done) {
+#pragma unroll
+      for (int k = 0; k < NM; ++k) mfma(k);
       // LDS reads first, then the expansion spread evenly under the MFMAs: a wave
       // can issue about six vector instructions in the shadow of one MFMA
-      constexpr int NM = NI * MJ;  // MFMAs of a step
       // vector instructions of a step (16 per word, a few more), shared out over its MFMAs
       constexpr int VPM = (16 * NI + 8 + NM - 1) / NM, VPM0 = VPM + 2;
       constexpr int VPM7 = (16 * NI + 16 + NM / 2) / (NM / 2 + 1);
@@ -396,6 +449,7 @@ __global__ __launch_bounds__(TD_THREADS * KG) void w4_tile_dma_kernel(
         }
       }
       __builtin_amdgcn_sched_barrier(0);
+      }
     }
     const uint32_t first = b0;
     b0 = b1;

@@ -67,6 +67,18 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
     const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
     const int gs_shift, const int tiles) {
   constexpr bool MX = FMT == 2;
+  // LATE (gs = 128: a wave's 128-k chunk is one group): the scale and the zero-point are
+  // applied to the chunk's FP32 sums, not to the weights.  The MFMA operand is the biased
+  // code itself, (1024 + q) for even k and (64 + q) for odd k -- what one mask-and-or makes
+  // of a byte, exact in FP16 -- and the chunk's accumulator starts at -sum_k x_k (b_k + z),
+  // which two more MFMA chains per chunk give for all tiles at once (x times the constant
+  // biases; with zero-points also x times -1): 8 vector instructions per word instead of
+  // 16.  The operands swap roles (A = x, B = W) so that a lane's four sums belong to its
+  // own row of W and take that row's scale: sum[e] += s_r * chunk[e].  Outputs differ from
+  // the per-weight arithmetic by FP32 rounding only (the hooked calls keep that one).
+  // (with four activation row tiles the chunk sums and their starting values do not fit
+  // the register file beside three tiles of codes)
+  constexpr bool LATE = !MX && GSV == 1 && MT <= 2;
   // K: any multiple of 128 with ceil(K / 128 / 8) == CH; wave w owns the 128-k chunks
   // [CH w, CH (w + 1)) that exist (the last waves may own fewer: chunks past the end
   // are fetched from a clamped address and meet zero activations)
@@ -332,6 +344,29 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
       __builtin_amdgcn_sched_barrier(0);
       request_x(ph + 1);
     }
+    // LATE: what every chunk's sums start from, for all tiles: -sum_k x_k (b_k + 8) with the
+    // symmetric zero-point, else -sum_k x_k b_k and -sum_k x_k (the same in every column)
+    [[maybe_unused]] f4 negb[MT][CP], negx[MT][CP];
+    if constexpr (LATE) {
+      const uint32_t nb = FMT == 1 ? 0xD400E400u : 0xD480E408u, n1 = 0xBC00BC00u;
+      const h8 nbv = __builtin_bit_cast(h8, u4{nb, nb, nb, nb}), n1v = __builtin_bit_cast(h8, u4{n1, n1, n1, n1});
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int cc = 0; cc < CP; ++cc) {
+          negb[mt][cc] = f4{0.f, 0.f, 0.f, 0.f};
+          negx[mt][cc] = f4{0.f, 0.f, 0.f, 0.f};
+          if (ph * CP + cc >= CH) continue;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            negb[mt][cc] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, xv[mt][cc][j]), nbv,
+                                                                  negb[mt][cc], 0, 0, 0);
+            if (FMT == 1)
+              negx[mt][cc] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, xv[mt][cc][j]), n1v,
+                                                                    negx[mt][cc], 0, 0, 0);
+          }
+        }
+    }
 #pragma unroll
     for (int t = 0; t < T; ++t) {
       if (ph == 0 && t >= 1) {
@@ -356,6 +391,30 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
         const int i = ph * CP + cc;
         if (i >= CH) continue;
         if (PAIRC && (i & 1) == 0 && i + 1 < CH) pair_fix(t, i);
+        if constexpr (LATE) {
+          const float s32 = half_bits_to_float(sc[t][i]);
+          [[maybe_unused]] float zf = 0.f;
+          if (FMT == 1) zf = (float)((zw[t][i] >> (4 * (gidx[i] & 7))) & 0xFu);
+          f4 part[MT];
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            part[mt] = negb[mt][cc];
+            if (FMT == 1) part[mt] += negx[mt][cc] * zf;
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            u4 a;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              a[e] = (__builtin_amdgcn_perm(0u, qw[t][i][j], 0x0c000c00u | (uint32_t)(e << 16) | (uint32_t)e) & mask) | magic;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+              part[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, xv[mt][cc][j]),
+                                                                __builtin_bit_cast(h8, a), part[mt], 0, 0, 0);
+          }
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) acc[t][mt] += part[mt] * s32;
+        } else {
         h2 cneg, s2;
         float sf = 0.f;
         if (MX) {
@@ -380,6 +439,7 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
             acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, __builtin_bit_cast(h8, xv[mt][cc][j]),
                                                                 acc[t][mt], 0, 0, 0);
         }
+        }
       }
     }
   }
@@ -403,6 +463,14 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
     f4 s = red[e * 64 + lane];
 #pragma unroll
     for (int w = 1; w < DR_WAVES; ++w) s += red[(w * E + e) * 64 + lane];
+    if constexpr (LATE) {  // lane: weight row 16 tile + r, activation rows 4 b .. + 3 of the row tile
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int m = m0 + 16 * mt + 4 * b + k;
+        if (m < M) c[(size_t)m * p.N + tile * 16 + r] = __builtin_bit_cast(uint16_t, (_Float16)s[k]);
+      }
+      continue;
+    }
     const int m = m0 + 16 * mt + r;
     if (m < M) {  // lane: activation row m, weight rows 16 tile + 4 b .. + 3
       uint16_t hv[4];
@@ -468,6 +536,7 @@ hipError_t launch_t_impl(const WView& v, const w4_half* x, w4_half* c, int M, hi
 constexpr int dr_tile_cap(int fmt, int gsv, int mt) {
   if (fmt == 1 && mt == 4) return 3;
   if (fmt == 1 && mt == 2 && gsv == 0) return 7;
+  if (fmt == 1 && mt == 2 && gsv == 1) return 6;  // the chunk sums' starting values take registers too
   return 8;
 }
 

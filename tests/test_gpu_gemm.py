@@ -311,17 +311,18 @@ def test_mx_dequant_exhaustive():
 
 @pytest.mark.parametrize("shape", [(1024, 4096, 128, True), (1024, 4096, 128, False), (512, 11008, 128, True),
                                    (512, 4096, 48, False), (512, 8192, 32, True)])
-def test_unhooked_vector_kernels_with_one_signed_and_offset_activations(shape):
-    """The vector kernels' unhooked arithmetic subtracts a bias sum that grows with the sum of the
-    activations; activations of one sign, with a large mean or a large magnitude are where that
-    cancellation would show.  Held to the same 5e-4 against the FP64 oracle as everywhere else."""
+def test_unhooked_kernels_with_one_signed_and_offset_activations(shape):
+    """The unhooked arithmetic of the vector kernels (M <= 2 here) and of the gs = 128 decode-batch
+    kernel (M = 8, 24) subtracts a bias sum that grows with the sum of the activations; activations
+    of one sign, with a large mean or a large magnitude are where that cancellation would show.
+    Held to the same 5e-4 against the FP64 oracle as everywhere else."""
     c = w4amd.capi()
     N, K, gs, sym = shape
     p = orc.quantize(orc.normal_weights(N * K, 0x0FF5E7) * 0.02, N, K, gs, sym)
     w_ref = orc.dequant_all(p)
     dp = DevPacked(p)
     rng = np.random.default_rng(5)
-    for M in (1, 2):
+    for M in (1, 2, 8, 24):
         for name, x64 in (("abs", np.abs(rng.standard_normal(M * K))), ("mean3", 3 + rng.standard_normal(M * K)),
                           ("mean30", 30 + rng.standard_normal(M * K)),
                           ("large", 1000 * np.abs(rng.standard_normal(M * K))), ("ones", np.ones(M * K))):

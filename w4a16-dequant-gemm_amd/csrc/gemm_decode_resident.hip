@@ -118,7 +118,8 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
 #pragma unroll
   for (int i = 0; i < CH; ++i) {
     const int k = chunk_k(i);
-    gidx[i] = MX ? (k >> 5) : GSV ? (k >> (8 - GSV)) : POW2 ? (k >> gs_shift) : k / p.gs;
+    gidx[i] = MX ? (k >> 5) : GSV == 1 ? wave * CH + i  // (one group per chunk: the same for every lane)
+              : GSV ? (k >> (8 - GSV)) : POW2 ? (k >> gs_shift) : k / p.gs;
   }
   // Codes.  The operand layout wants lane (r, b) to hold row r, 32 k of chunk i: fetched
   // as such, a load instruction takes 64 bytes of each of 16 rows, half of every

@@ -76,8 +76,10 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
   // 16.  The operands swap roles (A = x, B = W) so that a lane's four sums belong to its
   // own row of W and take that row's scale: sum[e] += s_r * chunk[e].  Outputs differ from
   // the per-weight arithmetic by FP32 rounding only (the hooked calls keep that one).
-  // (with four activation row tiles the chunk sums and their starting values do not fit
-  // the register file beside three tiles of codes)
+  // (not with four activation row tiles: their sixteen MFMAs per chunk already keep the
+  // matrix pipe as busy as the expansion keeps the vector pipe, the extra chains would
+  // make it the longer of the two, and the chunk sums do not fit the register file beside
+  // three tiles of codes)
   constexpr bool LATE = !MX && GSV == 1 && MT <= 2;
   // K: any multiple of 128 with ceil(K / 128 / 8) == CH; wave w owns the 128-k chunks
   // [CH w, CH (w + 1)) that exist (the last waves may own fewer: chunks past the end

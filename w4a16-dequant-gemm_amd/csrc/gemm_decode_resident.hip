@@ -67,15 +67,16 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
     const WView p, const w4_half* __restrict__ x, w4_half* __restrict__ c, const int M,
     const int gs_shift, const int tiles) {
   constexpr bool MX = FMT == 2;
-  // LATE (gs = 128: a wave's 128-k chunk is one group): the scale and the zero-point are
-  // applied to the chunk's FP32 sums, not to the weights.  The MFMA operand is the biased
-  // code itself, (1024 + q) for even k and (64 + q) for odd k -- what one mask-and-or makes
-  // of a byte, exact in FP16 -- and the chunk's accumulator starts at -sum_k x_k (b_k + z),
-  // which two more MFMA chains per chunk give for all tiles at once (x times the constant
-  // biases; with zero-points also x times -1): 8 vector instructions per word instead of
-  // 16.  The operands swap roles (A = x, B = W) so that a lane's four sums belong to its
-  // own row of W and take that row's scale: sum[e] += s_r * chunk[e].  Outputs differ from
-  // the per-weight arithmetic by FP32 rounding only (the hooked calls keep that one).
+  // LATE (gs = 128: a wave's 128-k chunk is one group): the scale is applied to the chunk's
+  // FP32 sums, not to the weights.  The operands swap roles (A = x, B = W) so that a lane's
+  // four sums belong to its own row of W and take that row's scale: sum[e] += s_r * chunk[e].
+  // Symmetric weights: the MFMA operand is the biased code itself, (1024 + q) for even k and
+  // (64 + q) for odd k -- what one mask-and-or makes of a byte, exact in FP16 -- and the
+  // chunk's accumulator starts at -sum_k x_k (b_k + 8), which one more MFMA chain per chunk
+  // (x times the constant biases) gives for all tiles at once: 8 vector instructions per
+  // word instead of 16.  With zero-points the operand is q - z (one packed add more: 12 per
+  // word; the zero-point's share through a chain of its own measured no faster).  Outputs
+  // differ from the per-weight arithmetic by FP32 rounding only (the hooked calls keep that).
   // (not with four activation row tiles: their sixteen MFMAs per chunk already keep the
   // matrix pipe as busy as the expansion keeps the vector pipe, the extra chains would
   // make it the longer of the two, and the chunk sums do not fit the register file beside
@@ -347,27 +348,22 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
       __builtin_amdgcn_sched_barrier(0);
       request_x(ph + 1);
     }
-    // LATE: what every chunk's sums start from, for all tiles: -sum_k x_k (b_k + 8) with the
-    // symmetric zero-point, else -sum_k x_k b_k and -sum_k x_k (the same in every column)
-    [[maybe_unused]] f4 negb[MT][CP], negx[MT][CP];
-    if constexpr (LATE) {
-      const uint32_t nb = FMT == 1 ? 0xD400E400u : 0xD480E408u, n1 = 0xBC00BC00u;
-      const h8 nbv = __builtin_bit_cast(h8, u4{nb, nb, nb, nb}), n1v = __builtin_bit_cast(h8, u4{n1, n1, n1, n1});
+    // LATE, symmetric: what every chunk's sums start from, for all tiles: -sum_k x_k (b_k + 8),
+    // the same in every column
+    [[maybe_unused]] f4 negb[MT][CP];
+    if constexpr (LATE && FMT == 0) {
+      const uint32_t nb = 0xD480E408u;  // -(1024 + 8) | -(64 + 8)
+      const h8 nbv = __builtin_bit_cast(h8, u4{nb, nb, nb, nb});
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
         for (int cc = 0; cc < CP; ++cc) {
           negb[mt][cc] = f4{0.f, 0.f, 0.f, 0.f};
-          negx[mt][cc] = f4{0.f, 0.f, 0.f, 0.f};
           if (ph * CP + cc >= CH) continue;
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
+          for (int j = 0; j < 4; ++j)
             negb[mt][cc] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, xv[mt][cc][j]), nbv,
                                                                   negb[mt][cc], 0, 0, 0);
-            if (FMT == 1)
-              negx[mt][cc] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, xv[mt][cc][j]), n1v,
-                                                                    negx[mt][cc], 0, 0, 0);
-          }
         }
     }
 #pragma unroll
@@ -396,13 +392,13 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
         if (PAIRC && (i & 1) == 0 && i + 1 < CH) pair_fix(t, i);
         if constexpr (LATE) {
           const float s32 = half_bits_to_float(sc[t][i]);
-          [[maybe_unused]] float zf = 0.f;
-          if (FMT == 1) zf = (float)((zw[t][i] >> (4 * (gidx[i] & 7))) & 0xFu);
           f4 part[MT];
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            part[mt] = negb[mt][cc];
-            if (FMT == 1) part[mt] += negx[mt][cc] * zf;
+          for (int mt = 0; mt < MT; ++mt) part[mt] = FMT == 1 ? f4{0.f, 0.f, 0.f, 0.f} : negb[mt][cc];
+          [[maybe_unused]] h2 cneg;
+          if (FMT == 1) {
+            const uint32_t z = (zw[t][i] >> (4 * (gidx[i] & 7))) & 0xFu;
+            cneg = as_h2(0xD400E400u | (z << 20) | z);
           }
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
@@ -410,13 +406,19 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
 #pragma unroll
             for (int e = 0; e < 4; ++e)
               a[e] = (__builtin_amdgcn_perm(0u, qw[t][i][j], 0x0c000c00u | (uint32_t)(e << 16) | (uint32_t)e) & mask) | magic;
+            if (FMT == 1) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) a[e] = as_u32(as_h2(a[e]) + cneg);
+            }
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
               part[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, xv[mt][cc][j]),
                                                                 __builtin_bit_cast(h8, a), part[mt], 0, 0, 0);
           }
 #pragma unroll
-          for (int mt = 0; mt < MT; ++mt) acc[t][mt] += part[mt] * s32;
+          for (int mt = 0; mt < MT; ++mt) {
+            acc[t][mt] += part[mt] * s32;
+          }
         } else {
         h2 cneg, s2;
         float sf = 0.f;

@@ -93,6 +93,35 @@ def test_c3_mxfp4_outliers_n14336():
         _sampled_gemm_check(c.gemm_mx, dp.view, w_ref, x, M, N, K, rows_m, n_rows=96, hook=(M != 16))
 
 
+@pytest.mark.parametrize("K,sym,Ms", [(8192, True, (24, 64)), (8192, False, (32, 64)), (11008, False, (24,)),
+                                      (13824, True, (32,))])
+def test_long_k_two_tiles_per_workgroup(K, sym, Ms):
+    """Long K on a grid of more 16-row tiles than compute units (N = 4128: 258) with more than 16
+    activation rows: two tiles share a workgroup's activations.  Hook bytes on the device, sampled
+    outputs against the oracle, hooked against unhooked within the cross gate."""
+    c = w4amd.capi()
+    N, gs = 4128, 128
+    p = orc.quantize(orc.normal_weights(N * K, 0x10C + K) * 0.02 + (0.0 if sym else 0.01), N, K, gs, sym)
+    w_ref = orc.dequant_all(p)
+    dp = DevPacked(p)
+    for M in Ms:
+        x = orc.normal_activations(M * K, 0x10C + M)
+        rows_m = np.array([0, M // 3, M - 1])
+        for fn in (c.gemm_mma, c.gemm):
+            _sampled_gemm_check(fn, dp.view, w_ref, x, M, N, K, rows_m, n_rows=96)
+
+
+def test_long_k_two_tiles_per_workgroup_mxfp4():
+    c = w4amd.capi()
+    N, K = 4128, 8192
+    p = orc.quantize_mx(orc.outlier_weights(N, K, 0x10D), N, K)
+    w_ref = orc.dequant_all_mx(p)
+    dp = DevPackedMx(p)
+    for M in (24, 64):
+        x = orc.normal_activations(M * K, 0x10D + M)
+        _sampled_gemm_check(c.gemm_mx, dp.view, w_ref, x, M, N, K, np.array([0, M // 2, M - 1]), n_rows=96)
+
+
 # ---- C5: batch 8, 8 kv heads, 4 query heads per kv head, D = 128, S = 32768 -------------------
 B5, HKV, GROUP, D5, S5, NS5 = 8, 8, 4, 128, 32768, 4
 H5 = B5 * HKV

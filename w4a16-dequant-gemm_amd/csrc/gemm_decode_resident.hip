@@ -538,7 +538,11 @@ hipError_t launch_t_impl(const WView& v, const w4_half* x, w4_half* c, int M, hi
 // Most tiles per workgroup that an instantiation holds in registers without spilling
 // (from the compiler's register counts): with zero-points, four activation row tiles
 // take three tiles; two row tiles with per-chunk scale loads (GSV == 0) take seven.
-constexpr int dr_tile_cap(int fmt, int gsv, int mt) {
+constexpr int dr_tile_cap(int fmt, int gsv, int mt, int ch = 4) {
+  // long K (8, 11 or 14 chunks per wave): two tiles where their codes still fit
+  if (ch == 8) return 2;
+  if (ch == 11) return (fmt != 0 && mt == 4) ? 1 : 2;
+  if (ch == 14) return (fmt != 1 && mt <= 2) ? 2 : 1;
   if (fmt == 1 && mt == 4) return 3;
   if (fmt == 1 && mt == 2 && gsv == 0) return 7;
   if (fmt == 1 && mt == 2 && gsv == 1) return 6;  // the chunk sums' starting values take registers too
@@ -548,7 +552,7 @@ constexpr int dr_tile_cap(int fmt, int gsv, int mt) {
 template <int FMT, int CH, bool POW2, int GSV, int T, int MT, int CPV = 0>
 hipError_t launch_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
                     int tiles, unsigned grid) {
-  if constexpr (T > dr_tile_cap(FMT, GSV, MT)) {
+  if constexpr (T > dr_tile_cap(FMT, GSV, MT, CH)) {
     return hipErrorInvalidValue;  // decode_resident_tiles() never asks for it
   } else {
     return launch_t_impl<FMT, CH, POW2, GSV, T, MT, CPV>(v, x, c, M, s, sh, tiles, grid);
@@ -573,7 +577,8 @@ template <int FMT, int CH, bool POW2, int GSV>
 hipError_t launch_ch(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
                      int tiles, int T) {
   const unsigned grid = (unsigned)((tiles + T - 1) / T);
-  if constexpr (CH > 4) {  // long K: one tile per workgroup (the codes of a tile fill the registers)
+  if constexpr (CH > 4) {  // long K: one tile per workgroup, or two that share the activations
+    if (T == 2) return launch_mt<FMT, CH, POW2, GSV, 2>(v, x, c, M, s, sh, tiles, grid);
     return launch_mt<FMT, CH, POW2, GSV, 1>(v, x, c, M, s, sh, tiles, grid);
   } else {
     switch (T) {
@@ -686,10 +691,15 @@ int decode_resident_tiles(const WView& v, const w4_half* x, const w4_half* c, in
   // workgroups beats two rounds of four-tile ones: N = 22016 / 28672, the fused gate and up
   // projections of the 11008- and 14336-wide MLPs)
   if (T > 4 && !(T <= 8 && M <= 32 && v.K == 4096)) T = 4;
-  if (resident_chunks(v.K) > 4) T = 1;
+  // long K: one tile per workgroup, unless there are more tiles than compute units and
+  // more than one activation row tile: then two tiles share a workgroup's activations,
+  // which every workgroup pulls out of L2 in full (K = 8192, M = 64: N = 8192 31.7 -> 24.5 us,
+  // N = 28672 105 -> 88; K = 13824, N = 5120 50 -> 35; at N = 4096, one tile per compute unit,
+  // halving the workgroups is slower, 23 -> 30 us at K = 11008)
+  if (resident_chunks(v.K) > 4) T = (M > 16 && v.N / 16 > cus) ? 2 : 1;
   // what does not fit the register file (dr_tile_cap)
   const int fmt = v.mx ? 2 : v.symmetric ? 0 : 1, mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
-  const int cap = dr_tile_cap(fmt, resident_gsv(v), M > 64 ? 4 : mt);
+  const int cap = dr_tile_cap(fmt, resident_gsv(v), M > 64 ? 4 : mt, resident_chunks(v.K));
   if (T > cap) T = cap;
   return T;
 }
@@ -698,6 +708,10 @@ int decode_resident_tiles(const WView& v, const w4_half* x, const w4_half* c, in
 
 bool decode_resident_applies(const WView& v, const w4_half* x, const w4_half* c, int M) {
   return decode_resident_tiles(v, x, c, M) != 0;
+}
+
+bool decode_resident_shares_long_k(const WView& v, const w4_half* x, const w4_half* c, int M) {
+  return resident_chunks(v.K) > 4 && decode_resident_tiles(v, x, c, M) > 1;
 }
 
 // Precondition: decode_resident_applies(v, x, c, M); no hook.

@@ -1112,6 +1112,12 @@ def summarize(extra, cold_gbs):
         s["c4_frac_mfma"] = _r(c4["frac_of_mfma_peak"], 3)
         s["c4_two_pass_TFLOPs"] = _r(c4["two_pass_TFLOPs"], 1)
         s["c4_hipblaslt_TFLOPs"] = _r(c4["hipblaslt_only_TFLOPs"], 1)
+        for r in extra.get("c4_prefill_other_M", []):
+            if r["M"] == 4096:  # where the 256 x 256 tiles take over: fused against dequant + library GEMM
+                s["c4_M4096_fused_two_pass_us"] = [_r(r["fused_us"], 1), _r(r["two_pass_us"], 1)]
+        c2 = [r for r in extra.get("c2_w4_asym", []) if r["gs"] == 128 and r["M"] == 8]
+        if c2:
+            s["c2_gs128_M8_us"] = _r(min(v for v in (c2[0].get("simt_us"), c2[0].get("mfma_us")) if v), 2)
     for key, name in (("c2_w4_asym", "c2"), ("c3_mxfp4", "c3")):
         rows = extra.get(key)
         if rows:

@@ -37,6 +37,8 @@ def _canned_extra():
         "c3_mxfp4": c3,
         "c4_prefill": {"M": 2048, "fused_TFLOPs": 905.1, "two_pass_TFLOPs": 875.2,
                        "hipblaslt_only_TFLOPs": 995.4, "frac_of_mfma_peak": 0.362, "fused_reps_ms": reps},
+        "c4_prefill_other_M": [{"weights": "w4_sym_gs128", "M": m, "fused_us": 116.07325077056885,
+                                "two_pass_us": 101.78505182266235, "fused_TFLOPs": 1184.07} for m in (256, 1024, 4096)],
         "c5_flash_decode": {"B": 8, "w4_gs32": fmt, "paged_w4_page16": paged,
                             "w4_gs32_noalloc_entry": {"ms": 0.0599, "reps_ms": reps[:5], "equals_allocating_entry": True}, "fp16": fmt,
                             "fp8_row_scale": fmt, "fp8_head_scale": fmt, "cpu": {"a_s": 0.07}},

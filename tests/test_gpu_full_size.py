@@ -93,7 +93,7 @@ def test_c3_mxfp4_outliers_n14336():
         _sampled_gemm_check(c.gemm_mx, dp.view, w_ref, x, M, N, K, rows_m, n_rows=96, hook=(M != 16))
 
 
-@pytest.mark.parametrize("K,sym,Ms", [(8192, True, (24, 64)), (8192, False, (32, 64)), (11008, False, (24,)),
+@pytest.mark.parametrize("K,sym,Ms", [(8192, True, (13, 24, 64)), (8192, False, (32, 64)), (11008, False, (24,)),
                                       (13824, True, (32,))])
 def test_long_k_two_tiles_per_workgroup(K, sym, Ms):
     """Long K on a grid of more 16-row tiles than compute units (N = 4128: 258) with more than 16

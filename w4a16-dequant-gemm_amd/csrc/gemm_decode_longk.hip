@@ -416,7 +416,7 @@ bool decode_longk_applies(const WView& v, const w4_half* x, const w4_half* c, in
   if (M < 1 || M > LK_MAX_M || v.N % 16 || longk_chunks(v.K) == 0) return false;
   if (!v.mx && v.gs % 32) return false;
   if ((((uintptr_t)v.q | (uintptr_t)x) & 15) || ((uintptr_t)c & 7)) return false;
-  // more tiles than compute units and several activation row tiles: the kernel that shares a
+  // more tiles than compute units and more than 12 to 16 activation rows: the kernel that shares a
   // workgroup's activations between two tiles is ahead where it exists (8, 11, 14 chunks per wave)
   if (decode_resident_shares_long_k(v, x, c, M)) return false;
   // K up to 5120 on grids of more than one tile per compute unit, W4: from M = 9 the kernel

@@ -692,11 +692,13 @@ int decode_resident_tiles(const WView& v, const w4_half* x, const w4_half* c, in
   // projections of the 11008- and 14336-wide MLPs)
   if (T > 4 && !(T <= 8 && M <= 32 && v.K == 4096)) T = 4;
   // long K: one tile per workgroup, unless there are more tiles than compute units and
-  // more than one activation row tile: then two tiles share a workgroup's activations,
+  // more than a dozen activation rows: then two tiles share a workgroup's activations,
   // which every workgroup pulls out of L2 in full (K = 8192, M = 64: N = 8192 31.7 -> 24.5 us,
   // N = 28672 105 -> 88; K = 13824, N = 5120 50 -> 35; at N = 4096, one tile per compute unit,
   // halving the workgroups is slower, 23 -> 30 us at K = 11008)
-  if (resident_chunks(v.K) > 4) T = (M > 16 && v.N / 16 > cus) ? 2 : 1;
+  // (from 13 rows on with symmetric weights: N = K = 8192, M = 16 17.2 -> 15.7 us, M = 12 even, M = 8
+  // 13.4 -> 14.8; with zero-points M = 16 is even)
+  if (resident_chunks(v.K) > 4) T = (M > (!v.mx && v.symmetric ? 12 : 16) && v.N / 16 > cus) ? 2 : 1;
   // what does not fit the register file (dr_tile_cap)
   const int fmt = v.mx ? 2 : v.symmetric ? 0 : 1, mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
   const int cap = dr_tile_cap(fmt, resident_gsv(v), M > 64 ? 4 : mt, resident_chunks(v.K));

@@ -56,7 +56,7 @@ bool try_tile256(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_
 bool decode_resident_applies(const WView& v, const w4_half* x, const w4_half* c, int M);
 hipError_t launch_decode_resident(const WView& v, const w4_half* x, w4_half* c, int M,
                                   hipStream_t s);
-// Long K (8, 11 or 14 chunks of 128 k per wave) with several activation row tiles on a grid of
+// Long K (8, 11 or 14 chunks of 128 k per wave) with more than 12 to 16 activation rows on a grid of
 // more tiles than compute units: the resident kernel then gives a workgroup two tiles, and the
 // long-K kernel below leaves the shape to it.
 bool decode_resident_shares_long_k(const WView& v, const w4_half* x, const w4_half* c, int M);

@@ -27,7 +27,7 @@ def _check(fn, view, w_ref, x, M, N, K, seed):
     rng = np.random.default_rng(seed)
     # the corners of the grid and a sample of its inside
     ms = np.unique(np.concatenate([[0, 255, 256, M - 1], rng.choice(M, size=12, replace=False)]))
-    ns = np.unique(np.concatenate([[0, 63, 64, 255, 256, N - 1], rng.choice(N, size=90, replace=False)]))
+    ns = np.unique(np.concatenate([[0, 63, 64, 255, 256, N - 1], rng.choice(N, size=min(N, 90), replace=False)]))
     ref = orc.gemm_oracle(np.ascontiguousarray(x.reshape(M, K)[ms]), len(ms), K,
                           np.ascontiguousarray(w_ref.reshape(N, K)[ns]), len(ns))
     got = np.ascontiguousarray(bits(c_u).reshape(M, N)[ms][:, ns]).view(np.float16)
@@ -40,6 +40,7 @@ SHAPES = [
     (3900, 4072, 256),   # ragged rows of X, a ragged last tile of W rows
     (3850, 4090, 128),   # N not a multiple of 8: element stores; two stages only
     (4096, 4096, 384),   # six stages
+    (12200, 1280, 128),  # five tiles along N: the plain order of tiles over the XCDs
 ]
 
 

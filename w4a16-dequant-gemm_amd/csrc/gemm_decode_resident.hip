@@ -50,6 +50,7 @@ __device__ __forceinline__ h8 expand_word(uint32_t w, h2 cneg, h2 s2, uint32_t m
 
 // FMT: 0 W4 symmetric, 1 W4 with zero-points, 2 MXFP4.  K = 1024 CH.  POW2: gs is a
 // power of two (shift gs_shift); GSV: 1, 2, 3 for gs = 128, 64, 32 with scale arrays
+// (4: gs a power of two from 128 on at long K, scales loaded one by one: a chunk lies in one group)
 // aligned for vector loads, else 0.  T tiles of 16 rows per
 // workgroup: tile g + gridDim.x t for t < T (tiles past the end are computed on
 // the last tile's rows and not stored).  MT tiles of 16 activation rows (M <= 16 MT).
@@ -81,7 +82,8 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
   // matrix pipe as busy as the expansion keeps the vector pipe, the extra chains would
   // make it the longer of the two, and the chunk sums do not fit the register file beside
   // three tiles of codes)
-  constexpr bool LATE = !MX && GSV == 1 && MT <= 2;
+  // (nor where two tiles of fourteen chunks and two row tiles leave no registers for the chunk sums)
+  constexpr bool LATE = !MX && (GSV == 1 || GSV == 4) && MT <= 2 && !(CH == 14 && T == 2 && MT == 2);
   // K: any multiple of 128 with ceil(K / 128 / 8) == CH; wave w owns the 128-k chunks
   // [CH w, CH (w + 1)) that exist (the last waves may own fewer: chunks past the end
   // are fetched from a clamped address and meet zero activations)
@@ -114,7 +116,7 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
   // loads and a per-lane pick, and their zero-points sit in one or two words;
   // MXFP4's CH bytes are 4 apart in 4 CH consecutive ones.  Other group sizes load
   // them one by one.
-  constexpr bool VEC = (MX && EXACT) || GSV != 0;
+  constexpr bool VEC = (MX && EXACT) || (GSV != 0 && GSV != 4);
   constexpr int PER = MX ? 4 : GSV == 1 ? 1 : GSV == 2 ? 2 : 4;  // groups per 128-k chunk
   uint32_t sc[T][CH], zw[T][CH];
   int gidx[CH];
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
   for (int i = 0; i < CH; ++i) {
     const int k = chunk_k(i);
     gidx[i] = MX ? (k >> 5) : GSV == 1 ? wave * CH + i  // (one group per chunk: the same for every lane)
-              : GSV ? (k >> (8 - GSV)) : POW2 ? (k >> gs_shift) : k / p.gs;
+              : (GSV && GSV != 4) ? (k >> (8 - GSV)) : POW2 ? (k >> gs_shift) : k / p.gs;
   }
   // Codes.  The operand layout wants lane (r, b) to hold row r, 32 k of chunk i: fetched
   // as such, a load instruction takes 64 bytes of each of 16 rows, half of every
@@ -251,7 +253,8 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
       }
     }
   };
-  static_assert(EXACT || GSV == 0, "vector scale loads assume K = 1024 CH");
+  static_assert(EXACT || GSV == 0 || GSV == 4, "vector scale loads assume K = 1024 CH");
+  static_assert(GSV != 4 || POW2, "chunk-wise scaling at long K: gs a power of two from 128 on");
 
   // Phase ph of this wave's slice of x -> its LDS region: block (mt, cc, rq) = rows
   // 16 mt + 4 rq .. + 3 of the 128-k chunk CP ph + cc; lane l fetches row l/16 of the
@@ -493,6 +496,8 @@ __global__ __launch_bounds__(DR_THREADS) void mfma_decode_resident_kernel(
 // How the scales are fetched: 1, 2, 3 for gs = 128, 64, 32 at K = 2048 / 4096 with arrays
 // aligned for the vector loads of the scales (and of two zero-point words), else 0.
 int resident_gsv(const WView& v) {
+  // long K (any other K this kernel takes): 4 where a chunk lies in one group, scales loaded one by one
+  if (v.K != 2048 && v.K != 4096) return (!v.mx && v.gs >= 128 && (v.gs & (v.gs - 1)) == 0) ? 4 : 0;
   if (!v.mx && (v.K == 2048 || v.K == 4096) && ((uintptr_t)v.scales & 15) == 0 &&
       (v.symmetric || ((uintptr_t)v.zeros & 7) == 0))
     return v.gs == 128 ? 1 : v.gs == 64 ? 2 : v.gs == 32 ? 3 : 0;
@@ -622,6 +627,7 @@ hipError_t launch_fmt(const WView& v, const w4_half* x, w4_half* c, int M, hipSt
                   : launch_ch<FMT, CHV, false, 0>(v, x, c, M, s, sh, tiles, T);             \
   }
 #define W4_LONG(CHV)                                                                        \
+  if (gsv == 4) return launch_ch<FMT, CHV, true, 4>(v, x, c, M, s, sh, tiles, T);           \
   return pow2 ? launch_ch<FMT, CHV, true, 0>(v, x, c, M, s, sh, tiles, T)                   \
               : launch_ch<FMT, CHV, false, 0>(v, x, c, M, s, sh, tiles, T);
   if constexpr (FMT == 2) {  // MXFP4 has one form per K: no group size, no scale-load variants

@@ -991,6 +991,14 @@ def probe(b, which, args):
                 out["w4_gemm_K%d_M%d_us" % (K, M)] = b.gemm_us("w4_gemm", views, x, c, M)[0]
             del views
             torch.cuda.empty_cache()
+        # more 16-row tiles than compute units: from 13 activation rows on two tiles share a workgroup's activations
+        views = [v[0] for v in rand_w4_views(b, 8192, 8192, 128, True, 6)]
+        for M in (16, 64):
+            x = torch.randn(M * 8192, device="cuda").to(torch.float16)
+            c = torch.empty(M * 8192, dtype=torch.float16, device="cuda")
+            out["w4_gemm_N8192_K8192_M%d_us" % M] = b.gemm_us("w4_gemm", views, x, c, M)[0]
+        del views
+        torch.cuda.empty_cache()
     elif which == "attention":  # C5 flash decode over FP16 / W4 / paged W4 / FP8 caches
         b.steps = 200
         out.update(extras_attention(b, False))

@@ -567,15 +567,21 @@ hipError_t launch_t(const WView& v, const w4_half* x, w4_half* c, int M, hipStre
 template <int FMT, int CH, bool POW2, int GSV, int T>
 hipError_t launch_mt(const WView& v, const w4_half* x, w4_half* c, int M, hipStream_t s, int sh,
                      int tiles, unsigned grid) {
-  if (M <= 16) {
-    if constexpr (CH == 4 && T == 4) {
-      // more workgroups than compute units: half the LDS each, two per compute unit
-      if ((int)grid > device_cus()) return launch_t<FMT, CH, POW2, GSV, T, 1, 2>(v, x, c, M, s, sh, tiles, grid);
+  if constexpr (CH > 4 && T == 1) {
+    // long K, one tile per workgroup: up to 64 rows belong to the pipelined long-K kernel, so
+    // only the four-row-tile form exists here (it is correct for fewer rows as well)
+    return launch_t<FMT, CH, POW2, GSV, T, 4>(v, x, c, M, s, sh, tiles, grid);
+  } else {
+    if (M <= 16) {
+      if constexpr (CH == 4 && T == 4) {
+        // more workgroups than compute units: half the LDS each, two per compute unit
+        if ((int)grid > device_cus()) return launch_t<FMT, CH, POW2, GSV, T, 1, 2>(v, x, c, M, s, sh, tiles, grid);
+      }
+      return launch_t<FMT, CH, POW2, GSV, T, 1>(v, x, c, M, s, sh, tiles, grid);
     }
-    return launch_t<FMT, CH, POW2, GSV, T, 1>(v, x, c, M, s, sh, tiles, grid);
+    if (M <= 32) return launch_t<FMT, CH, POW2, GSV, T, 2>(v, x, c, M, s, sh, tiles, grid);
+    return launch_t<FMT, CH, POW2, GSV, T, 4>(v, x, c, M, s, sh, tiles, grid);
   }
-  if (M <= 32) return launch_t<FMT, CH, POW2, GSV, T, 2>(v, x, c, M, s, sh, tiles, grid);
-  return launch_t<FMT, CH, POW2, GSV, T, 4>(v, x, c, M, s, sh, tiles, grid);
 }
 
 template <int FMT, int CH, bool POW2, int GSV>

@@ -38,11 +38,11 @@ def _one(c, H, S, D, gs, group, sym, seed, hooks):
     print(f"noalloc case H={H} S={S} D={D} gs={gs} group={group} sym={sym} hooks={hooks}", flush=True)
     # the entry that allocates nothing goes first (so the other entry's grow-only buffer cannot
     # stand in for an allocation of its own) and must leave the device's free memory as it was.
-    # The first call is not measured: a kernel's first launch in a process may make the HIP
-    # runtime itself take device memory (code, kernel-argument and signal pools; seen as 6 MB
-    # once, in one order of the test files).  An allocation made by the entry would show on
-    # every call, so the measured calls follow, and one of two in a row has to leave the free
-    # memory untouched.
+    # The first call is not measured: it is where the entry sets itself up on a device (the
+    # address of its built-in 4 MiB array, which the runtime may materialize only then, and the
+    # runtime's own first-launch pools; seen as 6 MiB once, in one order of the test files).  An
+    # allocation made per call would show on every call, so the measured calls follow, and one of
+    # two in a row has to leave the free memory untouched.
     c.attention_w4_flash_noalloc(dk.view, ptr(q_d), ptr(got), 0, ptr(ko), ptr(vo), group=group)
     torch.cuda.synchronize()
     unchanged = False
